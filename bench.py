@@ -1,0 +1,268 @@
+#!/usr/bin/env python
+"""Headline benchmark: forward+backward of the block-dropout matmul at M=N=K=8192 fp16, 64x64 blocks.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--size 8192] [--p 0.5] [--no-sweep] [--no-cpu]
+
+One "step" is one pass of the hot path over one batch of synthetic input already resident in HBM:
+kept-block list build, DSD forward Y, SDD backward dX, DSD backward dW (the three launches the
+reference's autograd function issues, flash_dropout/functional/blockwise_dropout_matmul_cuda.py:26,46,49).
+Prints ONE JSON line.  `value` is the effective dense-equivalent rate 6*M*N*K / t at p = 0.5; the same line
+carries the p-sweep (0, 0.25, 0.5, 0.75) with kept-work rates (the reference's FLOP convention,
+benchmark/full.py:160-163: 2MNK forward + 4MNK backward, times the kept fraction), the t(p=.5)/t(p=0)
+ratio, a roofline object for the dominant kernel (HIP-event timed per launch) and the CPU baseline.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+for _p in (ROOT, ROOT / "sparse-dropout_amd"):
+    if str(_p) not in sys.path:
+        sys.path.insert(0, str(_p))
+
+PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA peak
+METRIC = "fwd+bwd ms & effective TFLOP/s vs p (0–0.75) at 8192³ fp16; % of MFMA peak"
+
+
+def make_problem(size: int, p: float, bs: int, seed: int = 0):
+    import torch
+
+    gen = torch.Generator().manual_seed(seed)
+    M = N = K = size
+    dev = torch.device("cuda:0")
+    x = torch.randn(M, K, generator=gen).half().to(dev)
+    w = (torch.randn(N, K, generator=gen) / K ** 0.5).half().to(dev)
+    dy = torch.randn(M, N, generator=gen).half().to(dev)
+    mask = (torch.rand(M // bs, K // bs, generator=gen) < p).to(dev)  # CPU generator: device independent
+    return x, w, dy, mask
+
+
+class Step:
+    """The hot path with preallocated outputs, called through the C-ABI shim."""
+
+    def __init__(self, x, w, dy, mask, bs, p):
+        import torch
+
+        from flash_dropout.hip import GEMM
+
+        self.ext = GEMM()
+        self.x, self.w, self.dy, self.mask, self.bs = x, w, dy, mask, bs
+        self.scale = 1.0 / (1.0 - p)
+        M, K = x.shape
+        N = w.shape[0]
+        self.y = torch.empty(M, N, dtype=x.dtype, device=x.device)
+        self.dx = torch.empty(M, K, dtype=x.dtype, device=x.device)
+        self.dw_t = torch.empty(N, K, dtype=x.dtype, device=x.device).t()  # [K, N] view of row-major [N, K]
+        self.lists = self.ext.build_lists(mask)
+        kept = int((~mask).sum().item())
+        self.kept_area = kept * bs * bs
+        self.flops_fwd = 2.0 * self.kept_area * N
+        self.flops_total = 6.0 * self.kept_area * N
+        self.flops_dense = 6.0 * M * N * K
+
+    def build(self):
+        self.lists = self.ext.build_lists(self.mask)
+
+    def fwd(self):
+        self.ext.gemm_dsd_lists(self.x, self.w, self.lists, self.bs, self.scale, out=self.y)
+
+    def dx_(self):
+        self.ext.gemm_sdd_lists(self.dy, self.w.t(), self.lists, self.bs, self.scale, out=self.dx)
+
+    def dw_(self):
+        self.ext.gemm_dsd_lists(self.x.t(), self.dy.t(), self.lists.transposed(), self.bs, self.scale,
+                                out=self.dw_t)
+
+    def __call__(self):
+        self.build()
+        self.fwd()
+        self.dx_()
+        self.dw_()
+
+
+def time_steps(step, steps: int, warmup: int) -> float:
+    import torch
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def time_kernel_events(fn, reps: int, flush=None) -> float:
+    """Average launch duration in ms, HIP events on the launch stream, one pair per launch."""
+    import torch
+
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    for a, b in ev:
+        if flush is not None:
+            flush.zero_()
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return statistics.fmean(a.elapsed_time(b) for a, b in ev)
+
+
+def cpu_baseline(size: int, bs: int, p: float, reps: int):
+    """The oracle's literal naive path (mask expand + dense linear + autograd backward) on the host
+    cores, fp32, same kind of workload at a bounded size."""
+    import torch
+
+    from oracle import naive_torch
+
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(size, size, generator=gen)
+    w = torch.randn(size, size, generator=gen) / size ** 0.5
+    dy = torch.randn(size, size, generator=gen)
+    mask = torch.rand(size // bs, size // bs, generator=gen) < p
+    naive_torch.forward_backward(x, w, dy, mask, bs, p)
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        naive_torch.forward_backward(x, w, dy, mask, bs, p)
+        ts.append(time.perf_counter() - t0)
+    t = statistics.median(ts)
+    return {
+        "value": round(6.0 * size ** 3 / t / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"oracle/naive_torch.py fwd+bwd fp32 at M=N=K={size}, bs={bs}, p={p}, median of {reps} reps "
+                  f"({t * 1e3:.1f} ms each; host has {os.cpu_count()} logical cpus); dense-equivalent 6MNK/t",
+        "ms": round(t * 1e3, 2),
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--size", type=int, default=8192)
+    ap.add_argument("--p", type=float, default=0.5)
+    ap.add_argument("--block-size", type=int, default=64)
+    ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--cpu-size", type=int, default=4096)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
+              "(the path has no collectives; sharding is described in DESIGN.md)", file=sys.stderr)
+        return 2
+
+    import torch
+
+    import __graft_entry__ as entry
+
+    entry.ensure_built()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    size, bs = args.size, args.block_size
+
+    # ---- headline: K timed steps at p -----------------------------------------------------
+    step = Step(*make_problem(size, args.p, bs), bs, args.p)
+    ms = time_steps(step, args.steps, args.warmup)
+    value = step.flops_dense / (ms * 1e-3) / 1e12
+    kept_tflops = step.flops_total / (ms * 1e-3) / 1e12
+
+    # ---- per-kernel launch durations (HIP events on the launch stream) ---------------------
+    reps = max(5, min(args.steps, 20))
+    kern_ms = {
+        "build_lists": time_kernel_events(step.build, reps),
+        "dsd_forward": time_kernel_events(step.fwd, reps),
+        "sdd_dx": time_kernel_events(step.dx_, reps),
+        "dsd_dw": time_kernel_events(step.dw_, reps),
+    }
+    dominant = max(("dsd_forward", "sdd_dx", "dsd_dw"), key=lambda k: kern_ms[k])
+    achieved = step.flops_fwd / (kern_ms[dominant] * 1e-3) / 1e12  # each GEMM does 2*kept_area*N flops
+    roofline = {
+        "bound": "mfma",
+        "kernel": dominant,
+        "achieved": round(achieved, 2),
+        "peak": PEAK_FP16_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": round(achieved / PEAK_FP16_TFLOPS, 4),
+        "traffic": None,
+        "flops_per_launch": step.flops_fwd,
+        "avg_launch_ms": round(kern_ms[dominant], 4),
+        "all_kernels_ms": {k: round(v, 4) for k, v in kern_ms.items()},
+        "all_kernels_tflops": {k: round(step.flops_fwd / (kern_ms[k] * 1e-3) / 1e12, 2)
+                               for k in ("dsd_forward", "sdd_dx", "dsd_dw")},
+    }
+
+    # ---- p sweep (reference protocol: L2-sized buffer zeroed before each call, median) ------
+    sweep = []
+    ratio = None
+    if not args.no_sweep:
+        flush = torch.empty(512 << 20, dtype=torch.int8, device="cuda")  # > L2 + MALL
+        t_by_p = {}
+        for p in (0.0, 0.25, 0.5, 0.75):
+            st = Step(*make_problem(size, p, bs), bs, p)
+            for _ in range(3):
+                st()
+            ts = []
+            for _ in range(max(5, args.steps // 2)):
+                flush.zero_()
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                st()
+                b.record()
+                torch.cuda.synchronize()
+                ts.append(a.elapsed_time(b))
+            t = statistics.median(ts)
+            t_by_p[p] = t
+            sweep.append({
+                "p": p,
+                "kept_fraction": round(st.kept_area / (size * size), 4),
+                "fwd_bwd_ms": round(t, 4),
+                "kept_work_tflops": round(st.flops_total / (t * 1e-3) / 1e12, 2),
+                "dense_equiv_tflops": round(st.flops_dense / (t * 1e-3) / 1e12, 2),
+                "pct_mfma_peak_kept_work": round(100 * st.flops_total / (t * 1e-3) / 1e12 / PEAK_FP16_TFLOPS, 2),
+            })
+            del st
+        ratio = round(t_by_p[0.5] / t_by_p[0.0], 4)
+        del flush
+
+    out = {
+        "metric": METRIC,
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"square GEMM sweep M=N=K={size} fp16, 64x64 block mask, fwd DSD + bwd SDD/DSD "
+                        f"(list build included), value at p={args.p}",
+            "M": size, "N": size, "K": size, "block_size": bs, "p": args.p,
+            "value_definition": "dense-equivalent 6*M*N*K / t",
+        },
+        "kept_work_tflops": round(kept_tflops, 2),
+        "pct_mfma_peak_kept_work": round(100 * kept_tflops / PEAK_FP16_TFLOPS, 2),
+        "ratio_t_p50_over_t_p0": ratio,
+        "sweep": sweep,
+        "roofline": roofline,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(args.cpu_size, bs, args.p, reps=3)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

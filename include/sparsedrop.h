@@ -1,0 +1,171 @@
+/*
+ * libsparsedrop — C ABI of the MI355X (gfx950) SparseDrop kernels.
+ *
+ * Block-wise dropout fused into the following matmul: one Bernoulli per block_size x block_size
+ * tile of the activation matrix X[M,K]; dropped tiles are never loaded or multiplied.
+ *
+ *     Y  = s * (keep (.) X) * W^T        "DSD"  (dense = sparse x dense)      s = 1/(1-p)
+ *     dX = s * (dY * W) (.) keep         "SDD"  (sparse = dense x dense)
+ *     dW = s * dY^T * (keep (.) X)       "DSD"  on transposed operands
+ *
+ * This header replaces, entry point for entry point, the pybind11 module "gemm" of the reference
+ * (flash_dropout/cuda/src/gemm_binding.cu:137-141) and the Python shim that loads it
+ * (flash_dropout/cuda/binding_gemm.py:26-47).  Everything is plain pointers and sizes:
+ * no torch types cross this boundary.
+ *
+ * Conventions (all entry points)
+ *   - Every pointer is a DEVICE pointer on the current HIP device, unless stated otherwise.
+ *   - A matrix is (ptr, stride_r, stride_c) in ELEMENTS; like the reference's check_operand
+ *     (gemm_binding.cu:18-22) one of the two strides must be 1 (row- or column-major).  The
+ *     reference derives this from the tensor strides (gemm_binding.cu:90-92); here the caller
+ *     passes the strides themselves.
+ *   - "B" operands are [N, K]: out-features x reduction, as in the reference (gemm_binding.cu:56-69).
+ *   - mask is one byte per block, non-zero = DROPPED (flash_dropout/functional/utils.py:15),
+ *     with its own two strides in bytes.
+ *   - dtype: SD_F16 or SD_BF16 for A, B and C; accumulation is always fp32 and the scale is applied
+ *     to the fp32 accumulator before the single rounding at the store (gemm.cuh:55-66).
+ *   - stream is a hipStream_t passed as void* (NULL = the null stream).  All work is enqueued on it
+ *     and the call returns without synchronising.  The reference launches on the legacy default
+ *     stream (matmul_dsd.cuh:105); callers pass torch's current stream instead.
+ *   - Return value: SD_OK, or an error code with the reason in sd_last_error() (thread-local).
+ *     Shapes and strides are always validated on the host (the reference only has assert()s,
+ *     matmul_dsd.cuh:79-95).  The library allocates no device memory; workspaces are the caller's.
+ *   - Supported block sizes: multiples of 64.  M, N, K are arbitrary (edge tiles are predicated);
+ *     the mask has ceil(M/block_size) x ceil(K/block_size) entries.
+ */
+#ifndef SPARSEDROP_H_
+#define SPARSEDROP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum sd_status {
+  SD_OK = 0,
+  SD_ERR_INVALID = 1,     /* bad shape / stride / pointer / argument */
+  SD_ERR_UNSUPPORTED = 2, /* valid request this build has no kernel for */
+  SD_ERR_RUNTIME = 3      /* HIP launch or runtime failure */
+};
+
+enum sd_dtype { SD_F16 = 0, SD_BF16 = 1 };
+
+/* Library version (major*10000 + minor*100 + patch). No reference counterpart. */
+int sd_version(void);
+
+/* Message of the last failing call on this thread ("" if none).  Replaces the TORCH_CHECK
+ * exceptions of gemm_binding.cu:18-22,87-89. */
+const char* sd_last_error(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * (a) block-mask -> compacted kept-block lists
+ *
+ * Replaces the torch ops of flash_dropout/functional/utils.py:57-60 (row widths, cumsum, nonzero)
+ * and torch.nonzero(~mask) of flash_dropout/functional/blockwise_dropout_matmul_triton.py:48,
+ * without the device->host synchronisation those imply.
+ *
+ *   CSR: row_ptr[mb+1], col_idx[capacity mb*kb]; kept column blocks of row r, ascending, are
+ *        col_idx[row_ptr[r] .. row_ptr[r+1]).  col_idx[0..nnz) equals nonzero(~mask)[:,1].
+ *   CSC: col_ptr[kb+1], row_idx[capacity mb*kb]; kept row blocks of column c, ascending.
+ * Either pair may be NULL (both NULL is an error).  Entries past nnz are left untouched.
+ * ------------------------------------------------------------------------------------------- */
+int sd_build_lists(const uint8_t* mask, int64_t mb, int64_t kb, int64_t mask_stride_r,
+                   int64_t mask_stride_c, int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr,
+                   int32_t* row_idx, void* stream);
+
+/* Pointer-increment table of flash_dropout/functional/utils.py:19-69 from a CSR list:
+ * table[i] = col_idx[i]*block_k for the first kept block of a row, else (col_idx[i]-col_idx[i-1])*block_k;
+ * row_indices[r] = row_ptr[r]; row_widths[r] = row_ptr[r+1]-row_ptr[r].
+ * table has capacity >= nnz (mb*kb is always enough). */
+int sd_increment_table(const int32_t* row_ptr, const int32_t* col_idx, int64_t mb, int64_t block_k,
+                       int64_t* table, int64_t* row_indices, int64_t* row_widths, void* stream);
+
+/* Bytes of workspace the mask-taking GEMM entry points need for an mb x kb mask. */
+int64_t sd_workspace_bytes(int64_t mb, int64_t kb);
+
+/* ---------------------------------------------------------------------------------------------
+ * dense C[M,N] = A[M,K] * B[N,K]^T            replaces gemm()      gemm_binding.cu:47-54
+ * ------------------------------------------------------------------------------------------- */
+int sd_gemm(const void* A, int64_t a_stride_r, int64_t a_stride_c,
+            const void* B, int64_t b_stride_r, int64_t b_stride_c,
+            void* C, int64_t c_stride_r, int64_t c_stride_c,
+            int64_t M, int64_t N, int64_t K, int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * (b)/(d) DSD: C[M,N] = scale * sum over kept K-blocks of A's row-block of A_blk * B_blk^T
+ *         mask is [ceil(M/bs), ceil(K/bs)] over A.            replaces gemm_dsd()  gemm_binding.cu:82-94
+ * (c)     SDD: C tile = scale * A * B^T where kept, exactly 0 where dropped
+ *         mask is [ceil(M/bs), ceil(N/bs)] over C.            replaces gemm_sdd()  gemm_binding.cu:122-135
+ *
+ * The *_lists forms take the CSR list of the same mask (built once by sd_build_lists and shared by
+ * forward and backward); the mask forms build it into `workspace` (>= sd_workspace_bytes) on `stream`
+ * first.  For the weight gradient call sd_gemm_dsd*(X^T, dY^T, mask^T) exactly as
+ * flash_dropout/functional/blockwise_dropout_matmul_cuda.py:49-51 does — with the CSC list of the
+ * forward mask as the CSR list of mask^T — and pass C strides (1, ldc) to get dW[N,K] row-major
+ * directly instead of a transposed view.
+ * ------------------------------------------------------------------------------------------- */
+int sd_gemm_dsd(const void* A, int64_t a_stride_r, int64_t a_stride_c,
+                const void* B, int64_t b_stride_r, int64_t b_stride_c,
+                void* C, int64_t c_stride_r, int64_t c_stride_c,
+                const uint8_t* mask, int64_t mask_stride_r, int64_t mask_stride_c,
+                int64_t M, int64_t N, int64_t K, int64_t block_size, float scale, int dtype,
+                void* workspace, int64_t workspace_bytes, void* stream);
+
+int sd_gemm_sdd(const void* A, int64_t a_stride_r, int64_t a_stride_c,
+                const void* B, int64_t b_stride_r, int64_t b_stride_c,
+                void* C, int64_t c_stride_r, int64_t c_stride_c,
+                const uint8_t* mask, int64_t mask_stride_r, int64_t mask_stride_c,
+                int64_t M, int64_t N, int64_t K, int64_t block_size, float scale, int dtype,
+                void* workspace, int64_t workspace_bytes, void* stream);
+
+int sd_gemm_dsd_lists(const void* A, int64_t a_stride_r, int64_t a_stride_c,
+                      const void* B, int64_t b_stride_r, int64_t b_stride_c,
+                      void* C, int64_t c_stride_r, int64_t c_stride_c,
+                      const int32_t* row_ptr, const int32_t* col_idx,
+                      int64_t M, int64_t N, int64_t K, int64_t block_size, float scale, int dtype,
+                      void* stream);
+
+int sd_gemm_sdd_lists(const void* A, int64_t a_stride_r, int64_t a_stride_c,
+                      const void* B, int64_t b_stride_r, int64_t b_stride_c,
+                      void* C, int64_t c_stride_r, int64_t c_stride_c,
+                      const int32_t* row_ptr, const int32_t* col_idx,
+                      int64_t M, int64_t N, int64_t K, int64_t block_size, float scale, int dtype,
+                      void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * (e) im2col gather feeding the same GEMMs for conv.
+ *
+ * cols[(n*P+p)*Q+q, c*R*S + r*S + s] = x[n, c, p*stride_h + r*dil_h - pad_h, q*stride_w + s*dil_w - pad_w]
+ * (zero outside the image): the matrix F.unfold(...).permute(0,2,1) of
+ * flash_dropout/functional/im2col_conv2d.py:17-20, materialised row-major [N*P*Q, C*R*S] (ld = cols_ld).
+ * x is addressed by four element strides, so NCHW and channels-last both work (the reference's dead
+ * kernel, flash_dropout/cuda/src/im2col.cuh:21-72, was channels-last only with (r,s,c) columns).
+ * With a CSR list (row_ptr/col_idx over the [ceil(NPQ/bs), ceil(CRS/bs)] block mask) only kept blocks
+ * are written; dropped blocks are left untouched (the DSD kernels never read them).  NULL lists = all.
+ *
+ * sd_col2im is the adjoint (dx[n,c,h,w] = sum of every cols entry that im2col filled from that pixel;
+ * dx is fully overwritten): the backward of the gather.  With a mask (one byte per block of cols,
+ * non-zero = dropped, strides in bytes) dropped blocks are not read and count as zero; NULL = read all.
+ * ------------------------------------------------------------------------------------------- */
+int sd_im2col(const void* x, int64_t x_stride_n, int64_t x_stride_c, int64_t x_stride_h,
+              int64_t x_stride_w, void* cols, int64_t cols_ld,
+              int64_t n, int64_t c, int64_t h, int64_t w, int64_t r, int64_t s,
+              int64_t pad_h, int64_t pad_w, int64_t stride_h, int64_t stride_w,
+              int64_t dil_h, int64_t dil_w,
+              const int32_t* row_ptr, const int32_t* col_idx, int64_t block_size,
+              int dtype, void* stream);
+
+int sd_col2im(const void* cols, int64_t cols_ld, void* dx, int64_t dx_stride_n,
+              int64_t dx_stride_c, int64_t dx_stride_h, int64_t dx_stride_w,
+              int64_t n, int64_t c, int64_t h, int64_t w, int64_t r, int64_t s,
+              int64_t pad_h, int64_t pad_w, int64_t stride_h, int64_t stride_w,
+              int64_t dil_h, int64_t dil_w,
+              const uint8_t* mask, int64_t mask_stride_r, int64_t mask_stride_c, int64_t block_size,
+              int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPARSEDROP_H_ */

@@ -1,0 +1,239 @@
+"""CPU oracle for the SparseDrop hot path (block-wise dropout fused into matmul).
+
+TEST INFRASTRUCTURE ONLY.  Nothing that ships (the ``flash_dropout`` package, the
+C-ABI library) may import this module; it exists so that tests, the smoke check and
+the ``cpu_baseline`` leg of the benchmark have an independent statement of what the
+HIP kernels must compute.  Everything is plain numpy, written from the reference's
+definitions (paths relative to the reference checkout):
+
+  mask polarity / shape      flash_dropout/functional/utils.py:11-16   (True = dropped, ceil shapes)
+  increment table            flash_dropout/functional/utils.py:19-69   (docstring known answer :36-56)
+  kept-block table           flash_dropout/functional/blockwise_dropout_matmul_triton.py:48
+  forward                    flash_dropout/functional/naive.py:8-25
+  backward operand algebra   flash_dropout/functional/blockwise_dropout_matmul_cuda.py:44-53
+  gemm_dsd / gemm_sdd        flash_dropout/cuda/src/matmul_dsd.cuh:47-66, matmul_sdd.cuh:44-65
+  SDD reference recipe       flash_dropout/cuda/binding_gemm.py:122-129
+  im2col conv                flash_dropout/functional/im2col_conv2d.py:5-27  (column = c*R*S + r*S + s)
+
+Parity status of each function (what pins it is in tests/test_oracle.py):
+  compact_csr / compact_csc / kept_table   pinned: numpy.nonzero identity, hand cases, brute force
+  mask_to_increment_table                  pinned: the reference's docstring known answer
+  gemm_dsd / gemm_sdd / dsd_forward /
+  sdd_dx / dsd_dw                          pinned: brute-force loops on tiny inputs, p=0 == dense,
+                                           single-kept-block closed form, torch autograd of the
+                                           literal naive.py restatement (oracle/naive_torch.py)
+  im2col / col2im / conv2d_blockdrop       pinned: torch F.unfold / F.fold / F.conv2d library routines
+No function here is "parity unpinned".
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+__all__ = [
+    "mask_shape",
+    "expand_keep",
+    "compact_csr",
+    "compact_csc",
+    "kept_table",
+    "mask_to_increment_table",
+    "gemm_dsd",
+    "gemm_sdd",
+    "dsd_forward",
+    "sdd_dx",
+    "dsd_dw",
+    "conv_out_hw",
+    "im2col",
+    "col2im",
+    "conv2d_blockdrop",
+]
+
+
+# --------------------------------------------------------------------------------------
+# mask + compaction (integer work; bit-exact contract)
+# --------------------------------------------------------------------------------------
+def mask_shape(m: int, k: int, block_size: int) -> tuple[int, int]:
+    """Shape of the block mask of an [m, k] matrix (utils.py:13-14: ceil on both axes)."""
+    return (math.ceil(m / block_size), math.ceil(k / block_size))
+
+
+def expand_keep(mask: np.ndarray, block_size: int, m: int, k: int) -> np.ndarray:
+    """Element-granular KEEP matrix [m, k] from the block mask (True = dropped, utils.py:15).
+
+    Each mask entry covers a block_size x block_size tile; tiles on the bottom / right edge
+    are cropped, which is what a ceil-shaped mask means for a matrix that is not a multiple
+    of the block size.
+    """
+    mask = np.asarray(mask, dtype=bool)
+    assert mask.shape == mask_shape(m, k, block_size), (mask.shape, (m, k, block_size))
+    keep = ~mask
+    return np.repeat(np.repeat(keep, block_size, axis=0), block_size, axis=1)[:m, :k]
+
+
+def compact_csr(mask: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
+    """Per-row-block list of kept column blocks.
+
+    row_ptr[int32, Mb+1], col_idx[int32, nnz]; row r's kept blocks are
+    col_idx[row_ptr[r]:row_ptr[r+1]], ascending.  Concatenated this is exactly the
+    second column of nonzero(~mask) (blockwise_dropout_matmul_triton.py:48).
+    """
+    keep = ~np.asarray(mask, dtype=bool)
+    widths = keep.sum(axis=1)
+    row_ptr = np.zeros(keep.shape[0] + 1, dtype=np.int32)
+    np.cumsum(widths, out=row_ptr[1:])
+    col_idx = np.nonzero(keep)[1].astype(np.int32)
+    return row_ptr, col_idx
+
+
+def compact_csc(mask: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
+    """Per-column-block list of kept row blocks (the CSR of mask.T): col_ptr[Kb+1], row_idx[nnz].
+
+    This is the skip list of the weight-gradient product, which the reference expresses as
+    gemm_dsd(X.T, dY.T, mask.T) (blockwise_dropout_matmul_cuda.py:49-51).
+    """
+    return compact_csr(np.asarray(mask, dtype=bool).T)
+
+
+def kept_table(mask: np.ndarray) -> np.ndarray:
+    """[nnz, 2] int64 (row_blk, col_blk) of kept blocks in row-major order (…_triton.py:48)."""
+    r, c = np.nonzero(~np.asarray(mask, dtype=bool))
+    return np.stack([r, c], axis=1).astype(np.int64)
+
+
+def mask_to_increment_table(mask: np.ndarray, block_k: int):
+    """Pointer-increment table of utils.py:19-69.
+
+    offsets = kept column index * block_k in row-major order; table = first difference of
+    offsets, except that each row's first entry is the absolute offset (utils.py:63-67).
+    Rows whose start index is past the end of the table (trailing rows with nothing kept)
+    are skipped when patching, as the reference does (:64-67).  A row with nothing kept that
+    is *followed* by a non-empty row shares its start index with that row, so the patch
+    lands on the next row's first entry — which is that entry's absolute offset, as wanted.
+    Returns (table[int64, nnz], row_indices[int64, Mb], row_widths[int64, Mb]).
+    """
+    keep = ~np.asarray(mask, dtype=bool)
+    row_widths = keep.sum(axis=1).astype(np.int64)
+    row_indices = np.zeros(keep.shape[0], dtype=np.int64)
+    row_indices[1:] = np.cumsum(row_widths[:-1])
+    offsets = np.nonzero(keep)[1].astype(np.int64) * block_k
+    table = np.diff(offsets, prepend=np.int64(0))
+    in_range = row_indices[row_indices < len(table)]
+    table[in_range] = offsets[in_range]
+    return table, row_indices, row_widths
+
+
+# --------------------------------------------------------------------------------------
+# the three products
+# --------------------------------------------------------------------------------------
+def gemm_dsd(a, b, mask, block_size: int, scale: float, dtype=np.float64) -> np.ndarray:
+    """C[M,N] = scale * (A ⊙ keep) @ B.T with A[M,K], B[N,K], mask over A (matmul_dsd.cuh:47-66)."""
+    a = np.asarray(a, dtype=dtype)
+    b = np.asarray(b, dtype=dtype)
+    m, k = a.shape
+    keep = expand_keep(mask, block_size, m, k)
+    return (np.where(keep, a, 0) @ b.T) * dtype(scale)
+
+
+def gemm_sdd(a, b, mask, block_size: int, scale: float, dtype=np.float64) -> np.ndarray:
+    """C[M,N] = scale * (A @ B.T) ⊙ keep with mask over the OUTPUT (matmul_sdd.cuh:44-65).
+
+    Dropped tiles are exactly zero (the kernel writes cleared accumulators)."""
+    a = np.asarray(a, dtype=dtype)
+    b = np.asarray(b, dtype=dtype)
+    m, n = a.shape[0], b.shape[0]
+    keep = expand_keep(mask, block_size, m, n)
+    return np.where(keep, (a @ b.T) * dtype(scale), 0)
+
+
+def dsd_forward(x, w, mask, block_size: int, p: float, dtype=np.float64) -> np.ndarray:
+    """Y = (keep ⊙ X)/(1-p) @ W.T  (naive.py:8-25)."""
+    assert 0 <= p < 1
+    return gemm_dsd(x, w, mask, block_size, 1.0 / (1.0 - p), dtype)
+
+
+def sdd_dx(dy, w, mask, block_size: int, p: float, dtype=np.float64) -> np.ndarray:
+    """dX = (dY @ W) ⊙ keep /(1-p): gemm_sdd(dY, W.T, mask)  (…_cuda.py:46)."""
+    assert 0 <= p < 1
+    w = np.asarray(w, dtype=dtype)
+    return gemm_sdd(dy, w.T, mask, block_size, 1.0 / (1.0 - p), dtype)
+
+
+def dsd_dw(dy, x, mask, block_size: int, p: float, dtype=np.float64) -> np.ndarray:
+    """dW[N,K] = dY.T @ (keep ⊙ X)/(1-p): gemm_dsd(X.T, dY.T, mask.T).T  (…_cuda.py:49-51)."""
+    assert 0 <= p < 1
+    x = np.asarray(x, dtype=dtype)
+    dy = np.asarray(dy, dtype=dtype)
+    mask = np.asarray(mask, dtype=bool)
+    return gemm_dsd(x.T, dy.T, mask.T, block_size, 1.0 / (1.0 - p), dtype).T
+
+
+# --------------------------------------------------------------------------------------
+# conv via im2col
+# --------------------------------------------------------------------------------------
+def conv_out_hw(h, w, r, s, padding, stride, dilation) -> tuple[int, int]:
+    """Output extent P, Q (im2col_conv2d.py:14-15)."""
+    p_ = (h + 2 * padding[0] - dilation[0] * (r - 1) - 1) // stride[0] + 1
+    q_ = (w + 2 * padding[1] - dilation[1] * (s - 1) - 1) // stride[1] + 1
+    return p_, q_
+
+
+def im2col(x, r: int, s: int, padding=(0, 0), stride=(1, 1), dilation=(1, 1)) -> np.ndarray:
+    """[N*P*Q, C*R*S] patch matrix; row = (n, p, q), column = c*R*S + rr*S + ss
+    (F.unfold order, im2col_conv2d.py:17-20).  Out-of-image taps read zero."""
+    x = np.asarray(x)
+    n, c, h, w = x.shape
+    p_, q_ = conv_out_hw(h, w, r, s, padding, stride, dilation)
+    xp = np.zeros((n, c, h + 2 * padding[0], w + 2 * padding[1]), dtype=x.dtype)
+    xp[:, :, padding[0]:padding[0] + h, padding[1]:padding[1] + w] = x
+    cols = np.zeros((n, p_, q_, c, r, s), dtype=x.dtype)
+    for rr in range(r):
+        for ss in range(s):
+            h0 = rr * dilation[0]
+            w0 = ss * dilation[1]
+            patch = xp[:, :, h0:h0 + (p_ - 1) * stride[0] + 1:stride[0],
+                       w0:w0 + (q_ - 1) * stride[1] + 1:stride[1]]  # n c p q
+            cols[:, :, :, :, rr, ss] = patch.transpose(0, 2, 3, 1)
+    return cols.reshape(n * p_ * q_, c * r * s)
+
+
+def col2im(cols, x_shape, r: int, s: int, padding=(0, 0), stride=(1, 1), dilation=(1, 1)) -> np.ndarray:
+    """Adjoint of im2col: scatter-add a [N*P*Q, C*R*S] matrix back to [N,C,H,W]."""
+    n, c, h, w = x_shape
+    p_, q_ = conv_out_hw(h, w, r, s, padding, stride, dilation)
+    cols = np.asarray(cols).reshape(n, p_, q_, c, r, s)
+    xp = np.zeros((n, c, h + 2 * padding[0], w + 2 * padding[1]), dtype=cols.dtype)
+    for rr in range(r):
+        for ss in range(s):
+            h0 = rr * dilation[0]
+            w0 = ss * dilation[1]
+            xp[:, :, h0:h0 + (p_ - 1) * stride[0] + 1:stride[0],
+               w0:w0 + (q_ - 1) * stride[1] + 1:stride[1]] += cols[:, :, :, :, rr, ss].transpose(0, 3, 1, 2)
+    return xp[:, :, padding[0]:padding[0] + h, padding[1]:padding[1] + w]
+
+
+def conv2d_blockdrop(x, kernel, mask, block_size: int, p: float, padding=(0, 0), stride=(1, 1),
+                     dilation=(1, 1), dy=None, dtype=np.float64):
+    """Block dropout applied to the im2col matrix, then the linear layer, then back to NKPQ.
+
+    The reference never finished this variant (layers/dropout_conv.py:86-99 are comments), so
+    the oracle is *defined* by composition: im2col (im2col_conv2d.py:17-20) -> dsd_forward
+    (naive.py:8-25) -> reshape (im2col_conv2d.py:24-25).  ``mask`` is over [N*P*Q, C*R*S].
+    With ``dy`` [N,K,P,Q] also returns (dx [N,C,H,W], dkernel [K,C,R,S]).
+    """
+    x = np.asarray(x, dtype=dtype)
+    kernel = np.asarray(kernel, dtype=dtype)
+    n, c, h, w = x.shape
+    kk, _, r, s = kernel.shape
+    p_, q_ = conv_out_hw(h, w, r, s, padding, stride, dilation)
+    cols = im2col(x, r, s, padding, stride, dilation)
+    w2 = kernel.reshape(kk, c * r * s)
+    y2 = dsd_forward(cols, w2, mask, block_size, p, dtype)  # [N*P*Q, K]
+    y = y2.reshape(n, p_ * q_, kk).transpose(0, 2, 1).reshape(n, kk, p_, q_)
+    if dy is None:
+        return y
+    dy2 = np.asarray(dy, dtype=dtype).reshape(n, kk, p_ * q_).transpose(0, 2, 1).reshape(n * p_ * q_, kk)
+    dcols = sdd_dx(dy2, w2, mask, block_size, p, dtype)
+    dx = col2im(dcols, x.shape, r, s, padding, stride, dilation)
+    dw2 = dsd_dw(dy2, cols, mask, block_size, p, dtype)
+    return y, dx, dw2.reshape(kernel.shape)

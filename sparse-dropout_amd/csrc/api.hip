@@ -1,0 +1,220 @@
+// extern "C" surface of libsparsedrop: argument validation and dispatch.  No kernels here.
+#include "common.h"
+
+#include <cstdlib>
+#include <cstring>
+
+namespace sd {
+
+char* last_error_buf() {
+  static thread_local char buf[512] = {0};
+  return buf;
+}
+
+int build_lists(const uint8_t* mask, int64_t mb, int64_t kb, int64_t msr, int64_t msc,
+                int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx,
+                hipStream_t stream);
+int increment_table(const int32_t* row_ptr, const int32_t* col_idx, int64_t mb, int64_t block_k,
+                    int64_t* table, int64_t* row_indices, int64_t* row_widths, hipStream_t stream);
+int im2col(const void* x, int64_t sn, int64_t sc, int64_t sh, int64_t sw, void* cols, int64_t ld,
+           int64_t n, int64_t c, int64_t h, int64_t w, int64_t r, int64_t s, int64_t pad_h,
+           int64_t pad_w, int64_t stride_h, int64_t stride_w, int64_t dil_h, int64_t dil_w,
+           const int32_t* row_ptr, const int32_t* col_idx, int64_t bs, hipStream_t stream);
+int col2im(const void* cols, int64_t ld, void* dx, int64_t sn, int64_t sc, int64_t sh, int64_t sw,
+           int64_t n, int64_t c, int64_t h, int64_t w, int64_t r, int64_t s, int64_t pad_h,
+           int64_t pad_w, int64_t stride_h, int64_t stride_w, int64_t dil_h, int64_t dil_w,
+           const uint8_t* mask, int64_t msr, int64_t msc, int64_t bs, int dtype, hipStream_t stream);
+
+namespace {
+
+constexpr int64_t kMaxDim = 1LL << 31;
+
+int check_mat(const char* name, const void* p, int64_t sr, int64_t sc, int64_t rows, int64_t cols) {
+  SD_REQUIRE(p != nullptr || rows == 0 || cols == 0, "%s: null pointer", name);
+  SD_REQUIRE(sr == 1 || sc == 1, "%s must be row or column major (strides %lld, %lld)", name,
+             (long long)sr, (long long)sc);
+  SD_REQUIRE(sr >= 1 && sc >= 1, "%s: strides must be positive", name);
+  // the non-unit stride must span the contiguous extent, or rows overlap
+  if (sc == 1 && rows > 1) SD_REQUIRE(sr >= cols, "%s: row stride %lld < %lld columns", name, (long long)sr, (long long)cols);
+  if (sr == 1 && sc != 1 && cols > 1) SD_REQUIRE(sc >= rows, "%s: column stride %lld < %lld rows", name, (long long)sc, (long long)rows);
+  return SD_OK;
+}
+
+int check_common(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc,
+                 void* C, int64_t csr, int64_t csc, int64_t M, int64_t N, int64_t K, int dtype) {
+  SD_REQUIRE(M >= 0 && N >= 0 && K >= 0, "negative dimension");
+  SD_REQUIRE(M < kMaxDim && N < kMaxDim && K < kMaxDim, "dimension too large");
+  SD_REQUIRE(dtype == SD_F16 || dtype == SD_BF16, "dtype must be SD_F16 or SD_BF16 (got %d)", dtype);
+  if (int rc = check_mat("A", A, asr, asc, M, K)) return rc;
+  if (int rc = check_mat("B", B, bsr, bsc, N, K)) return rc;
+  if (int rc = check_mat("C", C, csr, csc, M, N)) return rc;
+  return SD_OK;
+}
+
+int check_sparse(int64_t bs, float scale) {
+  SD_REQUIRE(bs > 0, "block_size must be positive");
+  if (bs % 64 != 0) return fail(SD_ERR_UNSUPPORTED, "block_size %lld: only multiples of 64 are supported", (long long)bs);
+  SD_REQUIRE(scale == scale, "scale is NaN");
+  return SD_OK;
+}
+
+int run(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
+  static const bool force_generic = [] {
+    const char* e = std::getenv("SPARSEDROP_FORCE_GENERIC");
+    return e && e[0] == '1';
+  }();
+  if (!force_generic) {
+    const int rc = launch_fast(g, mode, dtype, stream);
+    if (rc != SD_ERR_UNSUPPORTED) return rc;
+  }
+  return launch_generic(g, mode, dtype, stream);
+}
+
+GemmArgs make_args(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc,
+                   void* C, int64_t csr, int64_t csc, int64_t M, int64_t N, int64_t K, int64_t bs,
+                   float scale, const int32_t* row_ptr, const int32_t* col_idx) {
+  GemmArgs g;
+  g.a = Mat{(const uint16_t*)A, asr, asc};
+  g.b = Mat{(const uint16_t*)B, bsr, bsc};
+  g.c = (uint16_t*)C;
+  g.c_sr = csr;
+  g.c_sc = csc;
+  g.M = M;
+  g.N = N;
+  g.K = K;
+  g.bs = bs;
+  g.scale = scale;
+  g.row_ptr = row_ptr;
+  g.col_idx = col_idx;
+  return g;
+}
+
+}  // namespace
+}  // namespace sd
+
+using namespace sd;
+
+extern "C" {
+
+int sd_version(void) { return 100; }
+
+const char* sd_last_error(void) { return last_error_buf(); }
+
+int64_t sd_workspace_bytes(int64_t mb, int64_t kb) {
+  if (mb < 0 || kb < 0) return 0;
+  // row_ptr[mb+1] then col_idx[mb*kb], the first padded to a 16-byte boundary
+  const int64_t ptr_bytes = ((mb + 1) * 4 + 15) / 16 * 16;
+  return ptr_bytes + mb * kb * 4;
+}
+
+int sd_build_lists(const uint8_t* mask, int64_t mb, int64_t kb, int64_t msr, int64_t msc,
+                   int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx,
+                   void* stream) {
+  SD_REQUIRE(mask != nullptr, "build_lists: null mask");
+  SD_REQUIRE(mb > 0 && kb > 0, "build_lists: mask must be non-empty (got %lld x %lld)", (long long)mb, (long long)kb);
+  SD_REQUIRE(mb * kb < kMaxDim, "build_lists: mask too large for 32-bit lists");
+  SD_REQUIRE(msr >= 1 && msc >= 1 && (msr == 1 || msc == 1), "build_lists: mask must be row or column major");
+  SD_REQUIRE((row_ptr == nullptr) == (col_idx == nullptr), "build_lists: pass both CSR arrays or neither");
+  SD_REQUIRE((col_ptr == nullptr) == (row_idx == nullptr), "build_lists: pass both CSC arrays or neither");
+  SD_REQUIRE(row_ptr || col_ptr, "build_lists: nothing to build");
+  return build_lists(mask, mb, kb, msr, msc, row_ptr, col_idx, col_ptr, row_idx, (hipStream_t)stream);
+}
+
+int sd_increment_table(const int32_t* row_ptr, const int32_t* col_idx, int64_t mb, int64_t block_k,
+                       int64_t* table, int64_t* row_indices, int64_t* row_widths, void* stream) {
+  SD_REQUIRE(row_ptr && col_idx && table && row_indices && row_widths, "increment_table: null pointer");
+  SD_REQUIRE(mb > 0 && block_k > 0, "increment_table: mb and block_k must be positive");
+  return increment_table(row_ptr, col_idx, mb, block_k, table, row_indices, row_widths, (hipStream_t)stream);
+}
+
+int sd_gemm(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc, void* C,
+            int64_t csr, int64_t csc, int64_t M, int64_t N, int64_t K, int dtype, void* stream) {
+  if (int rc = check_common(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, dtype)) return rc;
+  GemmArgs g = make_args(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, 0, 1.0f, nullptr, nullptr);
+  return run(g, kDense, dtype, (hipStream_t)stream);
+}
+
+int sd_gemm_dsd_lists(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc,
+                      void* C, int64_t csr, int64_t csc, const int32_t* row_ptr, const int32_t* col_idx,
+                      int64_t M, int64_t N, int64_t K, int64_t bs, float scale, int dtype, void* stream) {
+  if (int rc = check_common(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, dtype)) return rc;
+  if (int rc = check_sparse(bs, scale)) return rc;
+  SD_REQUIRE(row_ptr && col_idx, "gemm_dsd: null list");
+  GemmArgs g = make_args(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, bs, scale, row_ptr, col_idx);
+  return run(g, kDsd, dtype, (hipStream_t)stream);
+}
+
+int sd_gemm_sdd_lists(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc,
+                      void* C, int64_t csr, int64_t csc, const int32_t* row_ptr, const int32_t* col_idx,
+                      int64_t M, int64_t N, int64_t K, int64_t bs, float scale, int dtype, void* stream) {
+  if (int rc = check_common(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, dtype)) return rc;
+  if (int rc = check_sparse(bs, scale)) return rc;
+  SD_REQUIRE(row_ptr && col_idx, "gemm_sdd: null list");
+  GemmArgs g = make_args(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, bs, scale, row_ptr, col_idx);
+  return run(g, kSdd, dtype, (hipStream_t)stream);
+}
+
+static int lists_in_workspace(const uint8_t* mask, int64_t msr, int64_t msc, int64_t mb, int64_t kb,
+                              void* workspace, int64_t workspace_bytes, int32_t** row_ptr,
+                              int32_t** col_idx, void* stream) {
+  SD_REQUIRE(mask != nullptr, "null mask");
+  SD_REQUIRE(mb > 0 && kb > 0, "empty mask");
+  const int64_t need = sd_workspace_bytes(mb, kb);
+  SD_REQUIRE(workspace != nullptr && workspace_bytes >= need, "workspace too small: need %lld bytes, got %lld",
+             (long long)need, (long long)workspace_bytes);
+  SD_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, "workspace must be 16-byte aligned");
+  *row_ptr = (int32_t*)workspace;
+  *col_idx = (int32_t*)((char*)workspace + ((mb + 1) * 4 + 15) / 16 * 16);
+  return sd_build_lists(mask, mb, kb, msr, msc, *row_ptr, *col_idx, nullptr, nullptr, stream);
+}
+
+int sd_gemm_dsd(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc, void* C,
+                int64_t csr, int64_t csc, const uint8_t* mask, int64_t msr, int64_t msc, int64_t M,
+                int64_t N, int64_t K, int64_t bs, float scale, int dtype, void* workspace,
+                int64_t workspace_bytes, void* stream) {
+  if (int rc = check_common(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, dtype)) return rc;
+  if (int rc = check_sparse(bs, scale)) return rc;
+  if (M == 0 || N == 0) return SD_OK;
+  SD_REQUIRE(K > 0, "gemm_dsd: K must be positive");
+  int32_t *row_ptr, *col_idx;
+  if (int rc = lists_in_workspace(mask, msr, msc, ceil_div(M, bs), ceil_div(K, bs), workspace,
+                                  workspace_bytes, &row_ptr, &col_idx, stream))
+    return rc;
+  return sd_gemm_dsd_lists(A, asr, asc, B, bsr, bsc, C, csr, csc, row_ptr, col_idx, M, N, K, bs, scale,
+                           dtype, stream);
+}
+
+int sd_gemm_sdd(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc, void* C,
+                int64_t csr, int64_t csc, const uint8_t* mask, int64_t msr, int64_t msc, int64_t M,
+                int64_t N, int64_t K, int64_t bs, float scale, int dtype, void* workspace,
+                int64_t workspace_bytes, void* stream) {
+  if (int rc = check_common(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, dtype)) return rc;
+  if (int rc = check_sparse(bs, scale)) return rc;
+  if (M == 0 || N == 0) return SD_OK;
+  int32_t *row_ptr, *col_idx;
+  if (int rc = lists_in_workspace(mask, msr, msc, ceil_div(M, bs), ceil_div(N, bs), workspace,
+                                  workspace_bytes, &row_ptr, &col_idx, stream))
+    return rc;
+  return sd_gemm_sdd_lists(A, asr, asc, B, bsr, bsc, C, csr, csc, row_ptr, col_idx, M, N, K, bs, scale,
+                           dtype, stream);
+}
+
+int sd_im2col(const void* x, int64_t sn, int64_t sc, int64_t sh, int64_t sw, void* cols, int64_t ld,
+              int64_t n, int64_t c, int64_t h, int64_t w, int64_t r, int64_t s, int64_t pad_h,
+              int64_t pad_w, int64_t stride_h, int64_t stride_w, int64_t dil_h, int64_t dil_w,
+              const int32_t* row_ptr, const int32_t* col_idx, int64_t bs, int dtype, void* stream) {
+  SD_REQUIRE(dtype == SD_F16 || dtype == SD_BF16, "dtype must be SD_F16 or SD_BF16 (got %d)", dtype);
+  return im2col(x, sn, sc, sh, sw, cols, ld, n, c, h, w, r, s, pad_h, pad_w, stride_h, stride_w, dil_h,
+                dil_w, row_ptr, col_idx, bs, (hipStream_t)stream);
+}
+
+int sd_col2im(const void* cols, int64_t ld, void* dx, int64_t sn, int64_t sc, int64_t sh, int64_t sw,
+              int64_t n, int64_t c, int64_t h, int64_t w, int64_t r, int64_t s, int64_t pad_h,
+              int64_t pad_w, int64_t stride_h, int64_t stride_w, int64_t dil_h, int64_t dil_w,
+              const uint8_t* mask, int64_t msr, int64_t msc, int64_t bs, int dtype, void* stream) {
+  SD_REQUIRE(dtype == SD_F16 || dtype == SD_BF16, "dtype must be SD_F16 or SD_BF16 (got %d)", dtype);
+  return col2im(cols, ld, dx, sn, sc, sh, sw, n, c, h, w, r, s, pad_h, pad_w, stride_h, stride_w, dil_h,
+                dil_w, mask, msr, msc, bs, dtype, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,116 @@
+// Shared device/host helpers for the SparseDrop gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "sparsedrop.h"
+
+namespace sd {
+
+// ---- error plumbing -------------------------------------------------------------------------
+char* last_error_buf();  // thread-local, 512 bytes (api.hip)
+
+inline int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(last_error_buf(), 512, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define SD_REQUIRE(cond, ...)                                  \
+  do {                                                         \
+    if (!(cond)) return ::sd::fail(SD_ERR_INVALID, __VA_ARGS__); \
+  } while (0)
+
+inline int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(SD_ERR_RUNTIME, "%s: %s", what, hipGetErrorString(e));
+  return SD_OK;
+}
+
+// ---- vector types ---------------------------------------------------------------------------
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint16_t u16x8 __attribute__((ext_vector_type(8)));
+typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+
+struct F16 {
+  using vec8 = f16x8;
+  static constexpr int id = SD_F16;
+  __device__ static inline uint16_t from_float(float x) {
+    _Float16 h = (_Float16)x;
+    return __builtin_bit_cast(uint16_t, h);
+  }
+  __device__ static inline float to_float(uint16_t v) { return (float)__builtin_bit_cast(_Float16, v); }
+  // D(32x32) += A(32x16) * B(16x32); lane l supplies row/col l%32, k = 8*(l/32)..+7 of its operand.
+  __device__ static inline f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  __device__ static inline f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+
+struct BF16 {
+  using vec8 = bf16x8;
+  static constexpr int id = SD_BF16;
+  __device__ static inline uint16_t from_float(float x) {
+    __bf16 h = (__bf16)x;
+    return __builtin_bit_cast(uint16_t, h);
+  }
+  __device__ static inline float to_float(uint16_t v) {
+    return __builtin_bit_cast(float, (uint32_t)v << 16);
+  }
+  __device__ static inline f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  __device__ static inline f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+
+__host__ __device__ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ---- operand descriptors --------------------------------------------------------------------
+// A matrix operand as the kernels see it: base pointer plus element strides along its row index
+// and along its second index.
+struct Mat {
+  const uint16_t* ptr;
+  int64_t sr;  // stride of the row index
+  int64_t sc;  // stride of the column index
+};
+
+struct GemmArgs {
+  Mat a;         // [M, K]
+  Mat b;         // [N, K]
+  uint16_t* c;   // [M, N]
+  int64_t c_sr, c_sc;
+  int64_t M, N, K;
+  int64_t bs;     // mask block size (0 for dense)
+  float scale;
+  const int32_t* row_ptr;  // CSR of the mask (DSD: over A; SDD: over C); null for dense
+  const int32_t* col_idx;
+};
+
+enum Mode { kDense = 0, kDsd = 1, kSdd = 2 };
+
+// launchers (one per translation unit)
+int launch_generic(const GemmArgs& g, int mode, int dtype, hipStream_t stream);
+// returns SD_ERR_UNSUPPORTED (without setting an error message) when the fast path does not apply
+int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream);
+
+}  // namespace sd

@@ -1,0 +1,91 @@
+"""Block-dropout matmul on the HIP kernels, as an autograd Function.
+
+Counterpart of the reference's ``BlockwiseDropoutMatmulCUDA``
+(flash_dropout/functional/blockwise_dropout_matmul_cuda.py:7-59):
+
+    forward   Y  = gemm_dsd(X, W, mask)            (:26)
+    backward  dX = gemm_sdd(dY, W.T, mask)         (:46)
+              dW = gemm_dsd(X.T, dY.T, mask.T).T   (:49-51)
+
+Differences that matter to a caller: the kept-block lists are built once on the GPU in forward and
+reused by both backward products (no per-iteration mask reads, no host sync); dW comes back as a
+contiguous [N, K] tensor instead of a transposed view; bf16 works as well as fp16; shapes need not
+be multiples of anything; launches go to torch's current stream.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..hip.binding_gemm import GEMM, KeptLists, _block_size
+from .utils import blockwise_dropout_mask
+
+
+class BlockwiseDropoutMatmulHIP(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input: torch.Tensor, weight: torch.Tensor, mask: torch.Tensor, block_size: int,
+                p: float):
+        ext = GEMM()
+        scale = 1.0 / (1.0 - p)
+        lists = ext.build_lists(mask)
+        # C (M N) = A (M K sparse) * B (N K)
+        out = ext.gemm_dsd_lists(input, weight, lists, block_size, scale)
+        ctx.save_for_backward(input, weight, mask, lists.row_ptr, lists.col_idx, lists.col_ptr,
+                              lists.row_idx)
+        ctx.block_size = block_size
+        ctx.scale = scale
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output: torch.Tensor):
+        input, weight, mask, row_ptr, col_idx, col_ptr, row_idx = ctx.saved_tensors
+        lists = KeptLists(row_ptr, col_idx, col_ptr, row_idx, tuple(mask.shape))
+        ext = GEMM()
+        if grad_output.dtype != input.dtype:
+            grad_output = grad_output.to(input.dtype)
+        if grad_output.stride(0) != 1 and grad_output.stride(1) != 1:
+            grad_output = grad_output.contiguous()
+        grad_input = grad_weight = None
+        if ctx.needs_input_grad[0]:
+            # dA (M K sparse) = dC (M N) * B.T (K N): the mask is over the output
+            grad_input = ext.gemm_sdd_lists(grad_output, weight.t(), lists, ctx.block_size, ctx.scale)
+        if ctx.needs_input_grad[1]:
+            # dB.T (K N) = A.T (K M sparse) * dC.T (N M), written straight into a row-major [N, K]
+            grad_weight = ext.gemm_dsd_lists(input.t(), grad_output.t(), lists.transposed(),
+                                             ctx.block_size, ctx.scale, transposed_out=True).t()
+        return grad_input, grad_weight, None, None, None
+
+
+def _prepare(input: torch.Tensor, weight: torch.Tensor):
+    """Autocast contract of the reference (``custom_fwd(cast_inputs=torch.float16)``, …_cuda.py:9):
+    under autocast the operands are cast to the autocast dtype; outside it they must already be
+    float16 / bfloat16."""
+    if input.dim() != 2 or weight.dim() != 2:
+        raise ValueError("input must be [M, K] and weight [N, K]")
+    if torch.is_autocast_enabled("cuda"):
+        dt = torch.get_autocast_dtype("cuda")
+        input, weight = input.to(dt), weight.to(dt)
+    if input.stride(0) != 1 and input.stride(1) != 1:
+        input = input.contiguous()
+    if weight.stride(0) != 1 and weight.stride(1) != 1:
+        weight = weight.contiguous()
+    return input, weight
+
+
+def blockwise_dropout_matmul_mask(input: torch.Tensor, mask: torch.Tensor, block_size, p: float,
+                                  weight: torch.Tensor) -> torch.Tensor:
+    """Same as :func:`blockwise_dropout_matmul` with the mask given (True = dropped); argument order
+    of the reference's naive counterpart (functional/naive.py:8-14)."""
+    if not 0 <= p < 1:
+        raise ValueError("Dropout probability must be in [0, 1)")
+    bs = _block_size(block_size)
+    input, weight = _prepare(input, weight)
+    with torch.autocast("cuda", enabled=False):
+        return BlockwiseDropoutMatmulHIP.apply(input, weight, mask, bs, float(p))
+
+
+def blockwise_dropout_matmul(input: torch.Tensor, weight: torch.Tensor, block_size, p: float) -> torch.Tensor:
+    """``(keep ⊙ input)/(1-p) @ weight.T`` with a fresh block mask (reference: …_cuda.py:56-59)."""
+    if not 0 <= p < 1:
+        raise ValueError("Dropout probability must be in [0, 1)")
+    mask = blockwise_dropout_mask(input, block_size, p)
+    return blockwise_dropout_matmul_mask(input, mask, block_size, p, weight)

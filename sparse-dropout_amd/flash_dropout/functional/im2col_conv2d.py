@@ -1,0 +1,153 @@
+"""2-D convolution as im2col + matmul, dense and with block dropout on the patch matrix.
+
+Reference: flash_dropout/functional/im2col_conv2d.py:5-27 — ``F.unfold`` to (N, C*R*S, P*Q), permute
+to (N, P*Q, C*R*S), ``F.linear`` with ``kernel.view(K, -1)``, back to (N, K, P, Q).  Here the patch
+matrix [N*P*Q, C*R*S] (same column order c*R*S + r*S + s) is produced by the HIP gather kernel and
+multiplied by the HIP GEMMs; the result is returned, like the reference's, as an (N, K, P, Q) view
+of an (N, P*Q, K) buffer.
+
+The block-dropout variant is the one the reference left as comments in its conv layer
+(flash_dropout/layers/dropout_conv.py:86-99): one Bernoulli per block_size x block_size tile of the
+patch matrix; dropped tiles are neither gathered nor multiplied.
+"""
+from __future__ import annotations
+
+from math import ceil
+
+import torch
+import torch.nn.functional as F
+
+from ..hip.binding_gemm import GEMM, KeptLists, _block_size
+
+
+def _pair(v) -> tuple[int, int]:
+    if isinstance(v, int):
+        return (v, v)
+    a, b = v
+    return (int(a), int(b))
+
+
+def _to_matrix_grad(grad_output: torch.Tensor, dtype) -> torch.Tensor:
+    """(N, K, P, Q) gradient -> [N*P*Q, K] row-major (free when it is channels-last in memory)."""
+    n, k, p, q = grad_output.shape
+    return grad_output.to(dtype).permute(0, 2, 3, 1).reshape(n * p * q, k)
+
+
+class _Im2colConv2d(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input, kernel, mask, block_size, p, padding, stride, dilation):
+        ext = GEMM()
+        n, c, h, w = input.shape
+        k, _, r, s = kernel.shape
+        po, qo = ext.conv_out_hw(h, w, r, s, padding, stride, dilation)
+        w2 = kernel.reshape(k, c * r * s)
+        lists = None
+        if mask is not None:
+            lists = ext.build_lists(mask)
+            cols = ext.im2col(input, (r, s), padding, stride, dilation, lists, block_size)
+            y2 = ext.gemm_dsd_lists(cols, w2, lists, block_size, 1.0 / (1.0 - p))
+            ctx.save_for_backward(cols, w2, mask, lists.row_ptr, lists.col_idx, lists.col_ptr, lists.row_idx)
+        else:
+            cols = ext.im2col(input, (r, s), padding, stride, dilation)
+            y2 = ext.gemm(cols, w2)
+            ctx.save_for_backward(cols, w2)
+        ctx.geom = (tuple(input.shape), tuple(kernel.shape), padding, stride, dilation, block_size, p,
+                    input.is_contiguous(memory_format=torch.channels_last) and not input.is_contiguous())
+        return y2.view(n, po * qo, k).permute(0, 2, 1).view(n, k, po, qo)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        ext = GEMM()
+        x_shape, k_shape, padding, stride, dilation, block_size, p, ch_last = ctx.geom
+        r, s = k_shape[2], k_shape[3]
+        saved = ctx.saved_tensors
+        cols, w2 = saved[0], saved[1]
+        dy2 = _to_matrix_grad(grad_output, cols.dtype)
+        dx = dk = None
+        if len(saved) > 2:
+            mask = saved[2]
+            lists = KeptLists(saved[3], saved[4], saved[5], saved[6], tuple(mask.shape))
+            scale = 1.0 / (1.0 - p)
+            if ctx.needs_input_grad[0]:
+                dcols = ext.gemm_sdd_lists(dy2, w2.t(), lists, block_size, scale)
+                dx = ext.col2im(dcols, x_shape, (r, s), padding, stride, dilation, mask, block_size, ch_last)
+            if ctx.needs_input_grad[1]:
+                dk = ext.gemm_dsd_lists(cols.t(), dy2.t(), lists.transposed(), block_size, scale,
+                                        transposed_out=True).t().reshape(k_shape)
+        else:
+            if ctx.needs_input_grad[0]:
+                dcols = ext.gemm(dy2, w2.t())
+                dx = ext.col2im(dcols, x_shape, (r, s), padding, stride, dilation, channels_last=ch_last)
+            if ctx.needs_input_grad[1]:
+                dk = ext.gemm(cols.t(), dy2.t(), transposed_out=True).t().reshape(k_shape)
+        return dx, dk, None, None, None, None, None, None
+
+
+def _prepare(input: torch.Tensor, kernel: torch.Tensor):
+    if input.dim() != 4 or kernel.dim() != 4:
+        raise ValueError("input must be (N, C, H, W) and kernel (K, C, R, S)")
+    if input.shape[1] != kernel.shape[1]:
+        raise ValueError(f"channel mismatch: input {input.shape[1]}, kernel {kernel.shape[1]}")
+    if torch.is_autocast_enabled("cuda"):
+        dt = torch.get_autocast_dtype("cuda")
+        input, kernel = input.to(dt), kernel.to(dt)
+    return input, kernel.contiguous()
+
+
+def im2col_conv2d(input: torch.Tensor, kernel: torch.Tensor, padding=(0, 0), stride=(1, 1),
+                  dilation=(1, 1)) -> torch.Tensor:
+    """Dense convolution through the patch matrix (reference: im2col_conv2d.py:5-27)."""
+    input, kernel = _prepare(input, kernel)
+    with torch.autocast("cuda", enabled=False):
+        return _Im2colConv2d.apply(input, kernel, None, 0, 0.0, _pair(padding), _pair(stride), _pair(dilation))
+
+
+def conv_patch_matrix_shape(input_shape, kernel_shape, padding=(0, 0), stride=(1, 1), dilation=(1, 1)):
+    """(N*P*Q, C*R*S): the matrix the block mask of the conv variant is drawn over."""
+    n, c, h, w = input_shape
+    _, _, r, s = kernel_shape
+    po, qo = GEMM.conv_out_hw(h, w, r, s, _pair(padding), _pair(stride), _pair(dilation))
+    return n * po * qo, c * r * s
+
+
+def blockwise_dropout_conv2d_mask(input, mask, block_size, p: float, kernel, padding=(0, 0),
+                                  stride=(1, 1), dilation=(1, 1)) -> torch.Tensor:
+    """Block-dropout convolution with the mask given: ``mask`` is bool
+    [ceil(N*P*Q/bs), ceil(C*R*S/bs)], True = dropped."""
+    if not 0 <= p < 1:
+        raise ValueError("Dropout probability must be in [0, 1)")
+    bs = _block_size(block_size)
+    input, kernel = _prepare(input, kernel)
+    with torch.autocast("cuda", enabled=False):
+        return _Im2colConv2d.apply(input, kernel, mask, bs, float(p), _pair(padding), _pair(stride), _pair(dilation))
+
+
+def blockwise_dropout_conv2d(input, kernel, block_size, p: float, padding=(0, 0), stride=(1, 1),
+                             dilation=(1, 1)) -> torch.Tensor:
+    """Block-dropout convolution with a fresh mask over the patch matrix."""
+    bs = _block_size(block_size)
+    rows, ncols = conv_patch_matrix_shape(input.shape, kernel.shape, padding, stride, dilation)
+    mask = torch.rand(ceil(rows / bs), ceil(ncols / bs), device=input.device) < p
+    return blockwise_dropout_conv2d_mask(input, mask, bs, p, kernel, padding, stride, dilation)
+
+
+def naive_blockwise_dropout_conv2d_mask(input, mask, block_size, p: float, kernel, padding=(0, 0),
+                                        stride=(1, 1), dilation=(1, 1)) -> torch.Tensor:
+    """The same function in plain torch ops (unfold, expanded mask, dense linear); no work skipped."""
+    from .naive import blockwise_dropout_matmul_mask
+
+    n, c, h, w = input.shape
+    k, _, r, s = kernel.shape
+    po, qo = GEMM.conv_out_hw(h, w, r, s, _pair(padding), _pair(stride), _pair(dilation))
+    cols = F.unfold(input, (r, s), dilation=_pair(dilation), padding=_pair(padding), stride=_pair(stride))
+    cols = cols.permute(0, 2, 1).reshape(n * po * qo, c * r * s)
+    y2 = blockwise_dropout_matmul_mask(cols, mask, block_size, p, kernel.reshape(k, -1))
+    return y2.view(n, po * qo, k).permute(0, 2, 1).reshape(n, k, po, qo)
+
+
+def naive_blockwise_dropout_conv2d(input, kernel, block_size, p: float, padding=(0, 0), stride=(1, 1),
+                                   dilation=(1, 1)) -> torch.Tensor:
+    bs = _block_size(block_size)
+    rows, ncols = conv_patch_matrix_shape(input.shape, kernel.shape, padding, stride, dilation)
+    mask = torch.rand(ceil(rows / bs), ceil(ncols / bs), device=input.device) < p
+    return naive_blockwise_dropout_conv2d_mask(input, mask, bs, p, kernel, padding, stride, dilation)

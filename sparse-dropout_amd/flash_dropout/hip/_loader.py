@@ -1,0 +1,54 @@
+"""ctypes loader for libsparsedrop.so (the C ABI declared in include/sparsedrop.h).
+
+The library is built ahead of time by ``sparse-dropout_amd/csrc/build.py``; there is no JIT step and
+no fallback: if the shared object is missing, loading raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+from functools import lru_cache
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent.parent / "_lib" / "libsparsedrop.so"
+
+_mat = [c_void_p, c_int64, c_int64]  # ptr, stride_r, stride_c
+
+# name -> (restype, argtypes); mirrors include/sparsedrop.h declaration by declaration
+SIGNATURES = {
+    "sd_version": (c_int, []),
+    "sd_last_error": (c_char_p, []),
+    "sd_workspace_bytes": (c_int64, [c_int64, c_int64]),
+    "sd_build_lists": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64,
+                               c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sd_increment_table": (c_int, [c_void_p, c_void_p, c_int64, c_int64,
+                                   c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sd_gemm": (c_int, [*_mat, *_mat, *_mat, c_int64, c_int64, c_int64, c_int, c_void_p]),
+    "sd_gemm_dsd": (c_int, [*_mat, *_mat, *_mat, *_mat, c_int64, c_int64, c_int64, c_int64,
+                            c_float, c_int, c_void_p, c_int64, c_void_p]),
+    "sd_gemm_sdd": (c_int, [*_mat, *_mat, *_mat, *_mat, c_int64, c_int64, c_int64, c_int64,
+                            c_float, c_int, c_void_p, c_int64, c_void_p]),
+    "sd_gemm_dsd_lists": (c_int, [*_mat, *_mat, *_mat, c_void_p, c_void_p, c_int64, c_int64,
+                                  c_int64, c_int64, c_float, c_int, c_void_p]),
+    "sd_gemm_sdd_lists": (c_int, [*_mat, *_mat, *_mat, c_void_p, c_void_p, c_int64, c_int64,
+                                  c_int64, c_int64, c_float, c_int, c_void_p]),
+    "sd_im2col": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64,
+                          *([c_int64] * 12), c_void_p, c_void_p, c_int64, c_int, c_void_p]),
+    "sd_col2im": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                          *([c_int64] * 12), c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
+}
+
+
+@lru_cache(maxsize=None)
+def load() -> ctypes.CDLL:
+    if not LIB_PATH.exists():
+        raise RuntimeError(
+            f"{LIB_PATH} not found: build it with `python sparse-dropout_amd/csrc/build.py` "
+            "(hipcc, gfx950). There is no fallback implementation."
+        )
+    lib = ctypes.CDLL(str(LIB_PATH))
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError here = header and library disagree
+        fn.restype = res
+        fn.argtypes = args
+    return lib

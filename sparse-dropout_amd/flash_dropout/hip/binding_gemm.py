@@ -1,0 +1,298 @@
+"""Python face of the C ABI: the counterpart of the reference's ``flash_dropout/cuda/binding_gemm.py``.
+
+``GEMM`` keeps the reference's three methods with the same argument meaning
+(binding_gemm.py:26-47: ``gemm(A, B)``, ``gemm_dsd(A, B, mask, block_size, scale)``,
+``gemm_sdd(A, B, mask, block_size, scale)``; A is [M, K], B is [N, K], each row- or column-major,
+result a new row-major [M, N] tensor) and adds what the HIP path needs on top: the kept-block list
+builder, list-taking GEMMs (so forward and backward share one list build), and im2col / col2im.
+
+torch is plumbing here: it owns device memory and the stream; every computation is a call into
+libsparsedrop.so with raw pointers.  Tensors must live on the GPU; there is no CPU path.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from functools import cache
+from math import ceil
+
+import torch
+
+from . import _loader
+
+SD_F16, SD_BF16 = 0, 1
+_DTYPES = {torch.float16: SD_F16, torch.bfloat16: SD_BF16}
+
+
+class SparseDropError(RuntimeError):
+    """A libsparsedrop call returned a non-zero status."""
+
+
+@dataclass
+class KeptLists:
+    """Compacted kept-block lists of one block mask (True = dropped), all int32 on the mask's device.
+
+    CSR: kept column blocks of row block r are ``col_idx[row_ptr[r]:row_ptr[r+1]]`` (ascending);
+    CSC: kept row blocks of column block c are ``row_idx[col_ptr[c]:col_ptr[c+1]]``.
+    ``col_idx`` / ``row_idx`` have capacity Mb*Kb; only the first nnz entries are meaningful.
+    """
+
+    row_ptr: torch.Tensor
+    col_idx: torch.Tensor
+    col_ptr: torch.Tensor
+    row_idx: torch.Tensor
+    shape: tuple[int, int]
+
+    def nnz(self) -> int:
+        """Number of kept blocks (synchronises with the device)."""
+        return int(self.row_ptr[-1].item())
+
+    def transposed(self) -> "KeptLists":
+        """Lists of mask.T: CSR and CSC swap roles."""
+        return KeptLists(self.col_ptr, self.row_idx, self.row_ptr, self.col_idx,
+                         (self.shape[1], self.shape[0]))
+
+
+def _block_size(block_size) -> int:
+    """int, or a (bm, bk) pair with bm == bk (the reference's configs pass (128, 128) tuples,
+    eval/mlp/config.py:26, while its kernels take an int, gemm_binding.cu:82-83)."""
+    if isinstance(block_size, (tuple, list)):
+        if len(block_size) != 2 or block_size[0] != block_size[1]:
+            raise ValueError(f"block_size must be an int or a pair of equal ints, got {block_size!r}")
+        block_size = block_size[0]
+    if int(block_size) != block_size or block_size <= 0:
+        raise ValueError(f"block_size must be a positive integer, got {block_size!r}")
+    return int(block_size)
+
+
+def _check_operand(name: str, x: torch.Tensor) -> None:
+    # same rules as the reference's check_operand + dtype checks (gemm_binding.cu:18-22, 87-89)
+    if not isinstance(x, torch.Tensor):
+        raise TypeError(f"{name} must be a tensor")
+    if not x.is_cuda:
+        raise ValueError(f"{name} must be on the GPU (got {x.device})")
+    if x.dim() != 2:
+        raise ValueError(f"{name} must be 2D (got {x.dim()}D)")
+    if x.dtype not in _DTYPES:
+        raise TypeError(f"{name} must be float16 or bfloat16 (got {x.dtype})")
+    if x.numel() and x.stride(0) != 1 and x.stride(1) != 1:
+        raise ValueError(f"{name} must be row or column major (strides {x.stride()})")
+
+
+def _mat(x: torch.Tensor):
+    return x.data_ptr(), max(x.stride(0), 1), max(x.stride(1), 1)
+
+
+def _check_mask(mask: torch.Tensor, shape: tuple[int, int], like: torch.Tensor) -> torch.Tensor:
+    if mask.dtype != torch.bool:
+        raise TypeError(f"Mask must be bool (got {mask.dtype})")
+    if mask.device != like.device:
+        raise ValueError("mask must be on the same device as the operands")
+    if tuple(mask.shape) != shape:
+        raise ValueError(f"mask shape {tuple(mask.shape)} does not match blocks {shape}")
+    if mask.numel() and mask.stride(0) != 1 and mask.stride(1) != 1:
+        mask = mask.contiguous()
+    return mask
+
+
+def _mask_strides(mask: torch.Tensor):
+    sr, sc = mask.stride()
+    if sr != 1 and sc != 1:  # only possible for degenerate shapes
+        sr, sc = mask.shape[1], 1
+    return max(sr, 1), max(sc, 1)
+
+
+@cache
+class GEMM:
+    """Process-wide handle on libsparsedrop.so (the reference caches its JIT-built module the same
+    way, binding_gemm.py:7)."""
+
+    def __init__(self) -> None:
+        self.lib = _loader.load()
+
+    # ------------------------------------------------------------------ plumbing
+    def _call(self, fn, *args) -> None:
+        rc = fn(*args)
+        if rc != 0:
+            msg = self.lib.sd_last_error().decode(errors="replace")
+            exc = {1: ValueError, 2: NotImplementedError}.get(rc, SparseDropError)
+            raise exc(f"{fn.__name__}: {msg}")
+
+    @staticmethod
+    def _stream(t: torch.Tensor) -> int:
+        return torch.cuda.current_stream(t.device).cuda_stream
+
+    def _check_pair(self, A, B):
+        _check_operand("A", A)
+        _check_operand("B", B)
+        if A.dtype != B.dtype:
+            raise TypeError(f"A and B must have the same dtype ({A.dtype} vs {B.dtype})")
+        if A.device != B.device:
+            raise ValueError("A and B must be on the same device")
+        if A.shape[1] != B.shape[1]:
+            raise ValueError(f"reduction dims differ: A {tuple(A.shape)}, B {tuple(B.shape)}")
+
+    @staticmethod
+    def _out(A, B, out, transposed_out):
+        M, N = A.shape[0], B.shape[0]
+        if out is None:
+            if transposed_out:
+                return torch.empty((N, M), dtype=A.dtype, device=A.device).t()
+            return torch.empty((M, N), dtype=A.dtype, device=A.device)
+        if tuple(out.shape) != (M, N) or out.dtype != A.dtype or out.device != A.device:
+            raise ValueError("out has the wrong shape, dtype or device")
+        _check_operand("out", out)
+        return out
+
+    # ------------------------------------------------------------------ reference methods
+    def gemm(self, A: torch.Tensor, B: torch.Tensor, out=None, transposed_out=False) -> torch.Tensor:
+        """Dense ``A @ B.T`` (reference: binding_gemm.py:26-27)."""
+        self._check_pair(A, B)
+        C = self._out(A, B, out, transposed_out)
+        with torch.cuda.device(A.device):
+            self._call(self.lib.sd_gemm, *_mat(A), *_mat(B), *_mat(C), A.shape[0], B.shape[0],
+                       A.shape[1], _DTYPES[A.dtype], self._stream(A))
+        return C
+
+    def _masked(self, fn, mask_cols, A, B, mask, block_size, scale, out, transposed_out):
+        self._check_pair(A, B)
+        bs = _block_size(block_size)
+        M, N, K = A.shape[0], B.shape[0], A.shape[1]
+        mb, cb = ceil(M / bs), ceil((K if mask_cols == "K" else N) / bs)
+        mask = _check_mask(mask, (mb, cb), A)
+        C = self._out(A, B, out, transposed_out)
+        if M == 0 or N == 0:
+            return C
+        ws_bytes = self.lib.sd_workspace_bytes(mb, cb)
+        ws = torch.empty((ws_bytes + 3) // 4, dtype=torch.int32, device=A.device)
+        with torch.cuda.device(A.device):
+            self._call(fn, *_mat(A), *_mat(B), *_mat(C), mask.data_ptr(), *_mask_strides(mask),
+                       M, N, K, bs, float(scale), _DTYPES[A.dtype], ws.data_ptr(), ws_bytes,
+                       self._stream(A))
+        return C
+
+    def gemm_dsd(self, A, B, mask, block_size, scale, out=None, transposed_out=False) -> torch.Tensor:
+        """``scale * (A ⊙ keep) @ B.T`` with ``mask`` [ceil(M/bs), ceil(K/bs)] over A, True = dropped
+        (reference: binding_gemm.py:29-37)."""
+        return self._masked(self.lib.sd_gemm_dsd, "K", A, B, mask, block_size, scale, out, transposed_out)
+
+    def gemm_sdd(self, A, B, mask, block_size, scale, out=None, transposed_out=False) -> torch.Tensor:
+        """``scale * (A @ B.T) ⊙ keep`` with ``mask`` [ceil(M/bs), ceil(N/bs)] over the output; dropped
+        tiles are written as zeros (reference: binding_gemm.py:39-47)."""
+        return self._masked(self.lib.sd_gemm_sdd, "N", A, B, mask, block_size, scale, out, transposed_out)
+
+    # ------------------------------------------------------------------ lists
+    def build_lists(self, mask: torch.Tensor) -> KeptLists:
+        """Mask -> CSR + CSC kept-block lists in one launch, no host synchronisation."""
+        if mask.dim() != 2 or mask.dtype != torch.bool or not mask.is_cuda:
+            raise ValueError("mask must be a 2D bool tensor on the GPU")
+        mb, kb = mask.shape
+        if mb == 0 or kb == 0:
+            raise ValueError("mask must be non-empty")
+        if mask.stride(0) != 1 and mask.stride(1) != 1:
+            mask = mask.contiguous()
+        dev = mask.device
+        # one allocation: row_ptr | col_ptr | col_idx | row_idx
+        buf = torch.empty(mb + 1 + kb + 1 + 2 * mb * kb, dtype=torch.int32, device=dev)
+        row_ptr, col_ptr, col_idx, row_idx = torch.split(buf, [mb + 1, kb + 1, mb * kb, mb * kb])
+        with torch.cuda.device(dev):
+            self._call(self.lib.sd_build_lists, mask.data_ptr(), mb, kb, *_mask_strides(mask),
+                       row_ptr.data_ptr(), col_idx.data_ptr(), col_ptr.data_ptr(), row_idx.data_ptr(),
+                       self._stream(mask))
+        return KeptLists(row_ptr, col_idx, col_ptr, row_idx, (mb, kb))
+
+    def increment_table(self, lists: KeptLists, block_k: int):
+        """(table, row_indices, row_widths) of the reference's ``mask_to_increment_table``
+        (functional/utils.py:19-69), int64.  Reads nnz back to size ``table`` (one sync), as the
+        reference's ``nonzero`` does."""
+        mb = lists.shape[0]
+        dev = lists.row_ptr.device
+        table = torch.empty(lists.col_idx.numel(), dtype=torch.int64, device=dev)
+        row_indices = torch.empty(mb, dtype=torch.int64, device=dev)
+        row_widths = torch.empty(mb, dtype=torch.int64, device=dev)
+        with torch.cuda.device(dev):
+            self._call(self.lib.sd_increment_table, lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(),
+                       mb, int(block_k), table.data_ptr(), row_indices.data_ptr(),
+                       row_widths.data_ptr(), self._stream(table))
+        return table[: lists.nnz()], row_indices, row_widths
+
+    def _listed(self, fn, mask_cols, A, B, lists, block_size, scale, out, transposed_out):
+        self._check_pair(A, B)
+        bs = _block_size(block_size)
+        M, N, K = A.shape[0], B.shape[0], A.shape[1]
+        want = (ceil(M / bs), ceil((K if mask_cols == "K" else N) / bs))
+        if tuple(lists.shape) != want:
+            raise ValueError(f"lists are for a {lists.shape} mask, operands need {want}")
+        C = self._out(A, B, out, transposed_out)
+        if M == 0 or N == 0:
+            return C
+        with torch.cuda.device(A.device):
+            self._call(fn, *_mat(A), *_mat(B), *_mat(C), lists.row_ptr.data_ptr(),
+                       lists.col_idx.data_ptr(), M, N, K, bs, float(scale), _DTYPES[A.dtype],
+                       self._stream(A))
+        return C
+
+    def gemm_dsd_lists(self, A, B, lists: KeptLists, block_size, scale, out=None, transposed_out=False):
+        return self._listed(self.lib.sd_gemm_dsd_lists, "K", A, B, lists, block_size, scale, out, transposed_out)
+
+    def gemm_sdd_lists(self, A, B, lists: KeptLists, block_size, scale, out=None, transposed_out=False):
+        return self._listed(self.lib.sd_gemm_sdd_lists, "N", A, B, lists, block_size, scale, out, transposed_out)
+
+    # ------------------------------------------------------------------ conv feed
+    @staticmethod
+    def conv_out_hw(h, w, r, s, padding, stride, dilation):
+        # reference: functional/im2col_conv2d.py:14-15
+        p = (h + 2 * padding[0] - dilation[0] * (r - 1) - 1) // stride[0] + 1
+        q = (w + 2 * padding[1] - dilation[1] * (s - 1) - 1) // stride[1] + 1
+        return p, q
+
+    def im2col(self, x: torch.Tensor, kernel_size, padding=(0, 0), stride=(1, 1), dilation=(1, 1),
+               lists: KeptLists | None = None, block_size=None) -> torch.Tensor:
+        """[N*P*Q, C*R*S] patch matrix in F.unfold column order.  With ``lists`` (over the block mask
+        of that matrix) only kept blocks are written; the rest of the buffer is uninitialised."""
+        if x.dim() != 4 or not x.is_cuda or x.dtype not in _DTYPES:
+            raise ValueError("x must be a 4D float16/bfloat16 tensor on the GPU")
+        n, c, h, w = x.shape
+        r, s = kernel_size
+        p, q = self.conv_out_hw(h, w, r, s, padding, stride, dilation)
+        if p <= 0 or q <= 0:
+            raise ValueError("kernel does not fit the padded image")
+        cols = torch.empty((n * p * q, c * r * s), dtype=x.dtype, device=x.device)
+        rp = ci = None
+        bs = 0
+        if lists is not None:
+            bs = _block_size(block_size)
+            want = (ceil(n * p * q / bs), ceil(c * r * s / bs))
+            if tuple(lists.shape) != want:
+                raise ValueError(f"lists are for a {lists.shape} mask, patch matrix needs {want}")
+            rp, ci = lists.row_ptr.data_ptr(), lists.col_idx.data_ptr()
+        with torch.cuda.device(x.device):
+            self._call(self.lib.sd_im2col, x.data_ptr(), *x.stride(), cols.data_ptr(), cols.stride(0),
+                       n, c, h, w, r, s, *padding, *stride, *dilation, rp, ci, bs, _DTYPES[x.dtype],
+                       self._stream(x))
+        return cols
+
+    def col2im(self, cols: torch.Tensor, x_shape, kernel_size, padding=(0, 0), stride=(1, 1),
+               dilation=(1, 1), mask: torch.Tensor | None = None, block_size=None,
+               channels_last: bool = False) -> torch.Tensor:
+        """Adjoint of :meth:`im2col`: [N*P*Q, C*R*S] -> [N, C, H, W] (scatter-add expressed as a gather).
+        With ``mask`` dropped blocks of ``cols`` are not read."""
+        n, c, h, w = x_shape
+        r, s = kernel_size
+        if cols.dim() != 2 or not cols.is_cuda or cols.dtype not in _DTYPES or cols.stride(1) != 1:
+            raise ValueError("cols must be a row-major 2D float16/bfloat16 tensor on the GPU")
+        p, q = self.conv_out_hw(h, w, r, s, padding, stride, dilation)
+        if tuple(cols.shape) != (n * p * q, c * r * s):
+            raise ValueError(f"cols shape {tuple(cols.shape)} != {(n * p * q, c * r * s)}")
+        fmt = torch.channels_last if channels_last else torch.contiguous_format
+        dx = torch.empty((n, c, h, w), dtype=cols.dtype, device=cols.device, memory_format=fmt)
+        mp, msr, msc, bs = None, 0, 0, 0
+        if mask is not None:
+            bs = _block_size(block_size)
+            mask = _check_mask(mask, (ceil(n * p * q / bs), ceil(c * r * s / bs)), cols)
+            mp = mask.data_ptr()
+            msr, msc = _mask_strides(mask)
+        with torch.cuda.device(cols.device):
+            self._call(self.lib.sd_col2im, cols.data_ptr(), cols.stride(0), dx.data_ptr(), *dx.stride(),
+                       n, c, h, w, r, s, *padding, *stride, *dilation, mp, msr, msc, bs,
+                       _DTYPES[cols.dtype], self._stream(cols))
+        return dx

@@ -1,0 +1,167 @@
+"""Kernel (e): im2col gather / col2im and the conv path built on them, against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from _util import REL_FRO_TOL, cpu_mask, rel_fro, to_np
+from oracle import sparsedrop_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+GEOMS = [
+    dict(n=2, c=3, h=8, w=8, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)),
+    dict(n=3, c=5, h=13, w=9, r=3, s=2, padding=(0, 1), stride=(2, 1), dilation=(1, 2)),
+    dict(n=4, c=64, h=16, w=16, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)),
+    dict(n=2, c=16, h=10, w=10, r=1, s=1, padding=(0, 0), stride=(1, 1), dilation=(1, 1)),
+    dict(n=1, c=8, h=12, w=12, r=5, s=5, padding=(2, 2), stride=(2, 2), dilation=(1, 1)),
+]
+
+
+def _geo(cfg):
+    return dict(padding=cfg["padding"], stride=cfg["stride"], dilation=cfg["dilation"])
+
+
+@pytest.mark.parametrize("cfg", GEOMS)
+@pytest.mark.parametrize("channels_last", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_im2col_bit_exact(cfg, channels_last, dtype):
+    from flash_dropout.hip import GEMM
+
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(cfg["n"], cfg["c"], cfg["h"], cfg["w"], generator=gen).to(dtype)
+    xg = x.cuda()
+    if channels_last:
+        xg = xg.contiguous(memory_format=torch.channels_last)
+    cols = GEMM().im2col(xg, (cfg["r"], cfg["s"]), **_geo(cfg))
+    ref = O.im2col(x.float().numpy(), cfg["r"], cfg["s"], **_geo(cfg))
+    assert cols.shape == ref.shape
+    assert np.array_equal(cols.float().cpu().numpy(), ref)  # a gather: bit exact
+
+
+@pytest.mark.parametrize("cfg", GEOMS[2:3])
+def test_im2col_writes_only_kept_blocks(cfg):
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(1)
+    x = torch.randn(cfg["n"], cfg["c"], cfg["h"], cfg["w"], generator=gen).half().cuda()
+    rows, ncols = cfg["n"] * 16 * 16, cfg["c"] * 9
+    mask = cpu_mask(O.mask_shape(rows, ncols, 64), 0.5, gen)
+    lists = ext.build_lists(mask.cuda())
+    full = ext.im2col(x, (3, 3), **_geo(cfg))
+    # poison the allocator's next block so untouched entries are recognisable
+    poison = torch.full((rows, ncols), 7.0, dtype=torch.float16, device="cuda")
+    del poison
+    part = ext.im2col(x, (3, 3), lists=lists, block_size=64, **_geo(cfg))
+    keep = torch.from_numpy(O.expand_keep(mask.numpy(), 64, rows, ncols)).cuda()
+    assert torch.equal(part[keep], full[keep])
+
+
+@pytest.mark.parametrize("cfg", GEOMS)
+@pytest.mark.parametrize("channels_last", [False, True])
+def test_col2im_vs_oracle(cfg, channels_last):
+    from flash_dropout.hip import GEMM
+
+    gen = torch.Generator().manual_seed(2)
+    p_, q_ = O.conv_out_hw(cfg["h"], cfg["w"], cfg["r"], cfg["s"], **_geo(cfg))
+    rows, ncols = cfg["n"] * p_ * q_, cfg["c"] * cfg["r"] * cfg["s"]
+    g = torch.randn(rows, ncols, generator=gen).half()
+    shape = (cfg["n"], cfg["c"], cfg["h"], cfg["w"])
+    dx = GEMM().col2im(g.cuda(), shape, (cfg["r"], cfg["s"]), channels_last=channels_last, **_geo(cfg))
+    ref = O.col2im(g.float().numpy(), shape, cfg["r"], cfg["s"], **_geo(cfg))
+    assert dx.shape == shape
+    assert rel_fro(dx, ref) <= 2e-3  # fp32 sum of <= R*S fp16 values, one rounding
+    # with a mask: dropped blocks count as zero and are not read
+    mask = cpu_mask(O.mask_shape(rows, ncols, 64), 0.5, gen)
+    keep = O.expand_keep(mask.numpy(), 64, rows, ncols)
+    dxm = GEMM().col2im(g.cuda(), shape, (cfg["r"], cfg["s"]), mask=mask.cuda(), block_size=64, **_geo(cfg))
+    refm = O.col2im(np.where(keep, g.float().numpy(), 0), shape, cfg["r"], cfg["s"], **_geo(cfg))
+    assert rel_fro(dxm, refm) <= 2e-3
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(n=8, c=64, h=32, w=32, k=128, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)),
+    dict(n=4, c=24, h=17, w=15, k=40, r=3, s=3, padding=(1, 0), stride=(2, 1), dilation=(1, 1)),
+])
+@pytest.mark.parametrize("p", [0.0, 0.5])
+def test_blockdrop_conv_forward_backward(cfg, p):
+    """Reduced-batch version of the conv configuration (same 64->128 3x3 stride 1 pad 1 layer, 8 images
+    instead of 128) plus a ragged geometry: forward, dx and dkernel against the oracle."""
+    import flash_dropout.functional as F
+
+    gen = torch.Generator().manual_seed(5)
+    x = torch.randn(cfg["n"], cfg["c"], cfg["h"], cfg["w"], generator=gen).half()
+    fan_in = cfg["c"] * cfg["r"] * cfg["s"]
+    k = ((torch.rand(cfg["k"], cfg["c"], cfg["r"], cfg["s"], generator=gen) * 2 - 1) * fan_in ** -0.5).half()
+    p_, q_ = O.conv_out_hw(cfg["h"], cfg["w"], cfg["r"], cfg["s"], **_geo(cfg))
+    rows = cfg["n"] * p_ * q_
+    mask = cpu_mask(O.mask_shape(rows, fan_in, 64), p, gen)
+    dy = torch.randn(cfg["n"], cfg["k"], p_, q_, generator=gen).half()
+
+    xg, kg = x.cuda().requires_grad_(), k.cuda().requires_grad_()
+    y = F.blockwise_dropout_conv2d_mask(xg, mask.cuda(), 64, p, kg, **_geo(cfg))
+    assert y.shape == dy.shape
+    y.backward(dy.cuda())
+    ry, rdx, rdk = O.conv2d_blockdrop(to_np(x), to_np(k), mask.numpy(), 64, p, dy=to_np(dy), dtype=np.float32, **_geo(cfg))
+    assert rel_fro(y, ry) <= REL_FRO_TOL
+    assert rel_fro(xg.grad, rdx) <= REL_FRO_TOL
+    assert rel_fro(kg.grad, rdk) <= REL_FRO_TOL
+
+
+def test_dense_im2col_conv_matches_conv2d():
+    """The reference's implied check for its im2col path: equal to F.conv2d (benchmark/conv.py:20-75)."""
+    import flash_dropout.functional as F
+
+    torch.manual_seed(6)
+    x = torch.randn(4, 32, 20, 20, device="cuda", dtype=torch.float16, requires_grad=True)
+    k = (torch.randn(48, 32, 3, 3, device="cuda", dtype=torch.float16) * 0.06).requires_grad_()
+    y = F.im2col_conv2d(x, k, padding=(1, 1), stride=(1, 1), dilation=(1, 1))
+    dy = torch.randn_like(y)
+    y.backward(dy)
+    xr, kr = x.detach().float().requires_grad_(), k.detach().float().requires_grad_()
+    yr = torch.nn.functional.conv2d(xr, kr, padding=1)
+    yr.backward(dy.float())
+    assert rel_fro(y, yr) <= REL_FRO_TOL
+    assert rel_fro(x.grad, xr.grad) <= REL_FRO_TOL
+    assert rel_fro(k.grad, kr.grad) <= REL_FRO_TOL
+
+
+def test_conv_layer_variants_on_gpu():
+    from flash_dropout.layers import DropoutConv2d
+
+    torch.manual_seed(7)
+    x = torch.randn(4, 16, 12, 12, device="cuda", dtype=torch.float16)
+    for variant in ("im2col", "blockwise[hip]", "blockwise[naive]"):
+        conv = DropoutConv2d(16, 32, (3, 3), padding=(1, 1), p=0.0, variant=variant, block_size=64).cuda().half()
+        ref = torch.nn.functional.conv2d(x, conv.weight, padding=1)
+        assert rel_fro(conv(x), ref) <= REL_FRO_TOL, variant
+    conv = DropoutConv2d(16, 32, (3, 3), padding=(1, 1), p=0.5, variant="blockwise[hip]", block_size=64).cuda().half()
+    y = conv(x)
+    y.float().sum().backward()
+    assert y.shape == (4, 32, 12, 12) and conv.weight.grad is not None
+
+
+def test_full_size_conv_config_properties():
+    """The full conv configuration ([128,64,32,32] -> patch matrix [131072 x 576], 3x3 64->128) checked
+    through what does not need the full oracle: sampled images against the oracle (images are
+    independent rows of the patch matrix) and the adjoint identity <im2col(x), g> == <x, col2im(g)>."""
+    import flash_dropout.functional as F
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(8)
+    geo = dict(padding=(1, 1), stride=(1, 1), dilation=(1, 1))
+    x = torch.randn(128, 64, 32, 32, generator=gen).half()
+    k = ((torch.rand(128, 64, 3, 3, generator=gen) * 2 - 1) * 576 ** -0.5).half()
+    mask = cpu_mask((2048, 9), 0.5, gen)
+    y = F.blockwise_dropout_conv2d_mask(x.cuda(), mask.cuda(), 64, 0.5, k.cuda(), **geo)
+    for img in (0, 77, 127):
+        sub = mask[img * 16:(img + 1) * 16]
+        ry = O.conv2d_blockdrop(to_np(x[img:img + 1]), to_np(k), sub.numpy(), 64, 0.5, dtype=np.float32, **geo)
+        assert rel_fro(y[img:img + 1], ry) <= REL_FRO_TOL
+    xs = x[:16].cuda()
+    cols = ext.im2col(xs, (3, 3), **geo)
+    g = torch.randn(cols.shape, generator=gen).half().cuda()
+    lhs = (cols.double() * g.double()).sum().item()
+    rhs = (xs.double() * ext.col2im(g, xs.shape, (3, 3), **geo).double()).sum().item()
+    assert abs(lhs - rhs) <= 2e-3 * max(abs(lhs), (cols.double().norm() * g.double().norm()).item() * 1e-2)

@@ -1,0 +1,188 @@
+"""The public API on the GPU: autograd function, layers, autocast — against the CPU oracle."""
+import json
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from _util import REL_FRO_TOL, cpu_mask, rel_fro, to_np
+from oracle import naive_torch
+from oracle import sparsedrop_oracle as O
+
+pytestmark = pytest.mark.gpu
+GOLDEN = Path(__file__).parent / "golden"
+
+
+def _fwd_bwd(x, w, dy, mask, bs, p):
+    import flash_dropout.functional as F
+
+    x = x.detach().clone().requires_grad_()
+    w = w.detach().clone().requires_grad_()
+    y = F.hip_blockwise_dropout_matmul_mask(x, mask, bs, p, w)
+    y.backward(dy)
+    return y.detach(), x.grad, w.grad
+
+
+def test_cfg1_cpu_reference_configuration():
+    """X[1024x1024] ~N(0,1), W ~N(0,1/1024), 64x64 blocks, keep 0.5, seed 0, committed mask fixture.
+    Expected values come from autograd through the literal naive restatement in fp32, the HIP path
+    runs on the fp16-rounded tensors (the reference's own test does the same, test/test_cuda.py:45-51)."""
+    fx = json.loads((GOLDEN / "cfg1_mask.json").read_text())
+    mask = torch.tensor([[ch == "1" for ch in row] for row in fx["rows"]])
+    torch.manual_seed(0)
+    x = torch.randn(1024, 1024)
+    w = torch.randn(1024, 1024) / 32
+    dy = torch.randn(1024, 1024)
+    xh, wh, dyh = x.half(), w.half(), dy.half()
+    ry, rdx, rdw = naive_torch.forward_backward(xh.float(), wh.float(), dyh.float(), mask, 64, 0.5)
+    y, dx, dw = _fwd_bwd(xh.cuda(), wh.cuda(), dyh.cuda(), mask.cuda(), 64, 0.5)
+    assert y.dtype == torch.float16 and dw.is_contiguous() and dw.shape == (1024, 1024)
+    assert rel_fro(y, ry) <= REL_FRO_TOL
+    assert rel_fro(dx, rdx) <= REL_FRO_TOL
+    assert rel_fro(dw, rdw) <= REL_FRO_TOL
+    # and against the unrounded fp32 problem the reference's tolerances still hold
+    fy, fdx, fdw = naive_torch.forward_backward(x, w, dy, mask, 64, 0.5)
+    torch.testing.assert_close(y.float().cpu(), fy, atol=0.2, rtol=0.01)
+    torch.testing.assert_close(dw.float().cpu(), fdw, atol=0.2, rtol=0.01)
+    torch.testing.assert_close(dx.float().cpu(), fdx, atol=0.2, rtol=0.01)
+
+
+@pytest.mark.parametrize("p", [0.1, 0.3, 0.5])
+def test_cfg4_transformer_mlp(p):
+    """64x256 tokens -> X[16384x384]; Linear 384->1536, GELU, 1536->384; block dropout on both inputs."""
+    import flash_dropout.functional as F
+
+    gen = torch.Generator().manual_seed(4)
+    x = torch.randn(16384, 384, generator=gen).half()
+    w1 = (torch.rand(1536, 384, generator=gen) * 2 - 1).mul(384 ** -0.5).half()
+    w2 = (torch.rand(384, 1536, generator=gen) * 2 - 1).mul(1536 ** -0.5).half()
+    m1 = cpu_mask((256, 6), p, gen)
+    m2 = cpu_mask((256, 24), p, gen)
+    dy = torch.randn(16384, 384, generator=gen).half()
+
+    xg, w1g, w2g = (t.cuda().requires_grad_() for t in (x, w1, w2))
+    h = F.hip_blockwise_dropout_matmul_mask(xg, m1.cuda(), 64, p, w1g)
+    a = torch.nn.functional.gelu(h)
+    y = F.hip_blockwise_dropout_matmul_mask(a, m2.cuda(), 64, p, w2g)
+    y.backward(dy.cuda())
+
+    # oracle: same graph in fp32 with the naive restatement
+    xr, w1r, w2r = (t.float().requires_grad_() for t in (x, w1, w2))
+    hr = naive_torch.forward(xr, w1r, m1, 64, p)
+    ar = torch.nn.functional.gelu(hr)
+    yr = naive_torch.forward(ar, w2r, m2, 64, p)
+    yr.backward(dy.float())
+    assert rel_fro(h, hr) <= REL_FRO_TOL
+    assert rel_fro(y, yr) <= REL_FRO_TOL
+    assert rel_fro(xg.grad, xr.grad) <= REL_FRO_TOL
+    assert rel_fro(w1g.grad, w1r.grad) <= REL_FRO_TOL
+    assert rel_fro(w2g.grad, w2r.grad) <= REL_FRO_TOL
+
+
+def test_cfg3_mlp_on_28x28_images_through_layers():
+    """X[4096x784] uniform[0,1]; 784->1024->1024->10 with ReLU; block dropout p=0.5 on each hidden
+    input (layers 2 and 3) and, to exercise the K tail 784 = 12*64+16, on layer 1 as well."""
+    from flash_dropout.layers import DropoutMM
+
+    torch.manual_seed(3)
+    dims = [784, 1024, 1024, 10]
+    layers = [DropoutMM(dims[i], dims[i + 1], p=0.5, variant="blockwise[hip]", block_size=64) for i in range(3)]
+    x = torch.rand(4096, 784).half()
+    dy = torch.randn(4096, 10).half()
+    mods = [l.cuda().half() for l in layers]
+    xg = x.cuda().requires_grad_()
+
+    # run the HIP layers with a fixed generator state so the masks can be re-drawn for the oracle
+    torch.cuda.manual_seed(123)
+    state = torch.cuda.get_rng_state()
+    h = xg
+    for i, l in enumerate(mods):
+        h = l(h)
+        if i < 2:
+            h = torch.relu(h)
+    h.backward(dy.cuda())
+
+    torch.cuda.set_rng_state(state)
+    masks = []
+    for i in range(3):
+        masks.append((torch.rand(64, -(-dims[i] // 64), device="cuda") < 0.5).cpu())
+
+    def expand(mask, m, k):
+        return torch.from_numpy(O.expand_keep(mask.numpy(), 64, m, k)).float()
+
+    xr = x.float().requires_grad_()
+    ws = [l.weight.detach().float().cpu().requires_grad_() for l in mods]
+    hr = xr
+    for i in range(3):
+        hr = torch.nn.functional.linear(hr * expand(masks[i], 4096, dims[i]) * 2.0, ws[i])
+        if i < 2:
+            hr = torch.relu(hr)
+    hr.backward(dy.float())
+    assert rel_fro(h, hr) <= REL_FRO_TOL
+    assert rel_fro(xg.grad, xr.grad) <= REL_FRO_TOL
+    for l, wr in zip(mods, ws):
+        assert rel_fro(l.weight.grad, wr.grad) <= REL_FRO_TOL
+
+
+def test_layer_eval_and_3d_inputs_and_bf16():
+    from flash_dropout.layers import DropoutMM
+
+    torch.manual_seed(0)
+    layer = DropoutMM(384, 256, p=0.3, variant="blockwise[cuda]", block_size=(64, 64)).cuda().bfloat16()
+    x = torch.randn(8, 256, 384, device="cuda", dtype=torch.bfloat16)
+    layer.eval()
+    assert torch.equal(layer(x), torch.nn.functional.linear(x, layer.weight))
+    layer.train()
+    torch.cuda.manual_seed(9)
+    state = torch.cuda.get_rng_state()
+    y = layer(x)
+    assert y.shape == (8, 256, 256) and y.dtype == torch.bfloat16
+    torch.cuda.set_rng_state(state)
+    mask = (torch.rand(32, 6, device="cuda") < 0.3).cpu().numpy()
+    ref = O.dsd_forward(to_np(x.reshape(-1, 384)), to_np(layer.weight), mask, 64, 0.3, np.float32)
+    assert rel_fro(y.reshape(-1, 256), ref) <= REL_FRO_TOL
+
+
+def test_autocast_contract():
+    import flash_dropout.functional as F
+
+    torch.manual_seed(1)
+    x = torch.randn(256, 256, device="cuda", requires_grad=True)
+    w = torch.randn(128, 256, device="cuda", requires_grad=True)
+    mask = torch.rand(4, 4, device="cuda") < 0.5
+    with pytest.raises(TypeError, match="float16 or bfloat16"):
+        F.hip_blockwise_dropout_matmul_mask(x, mask, 64, 0.5, w)
+    for dt in (torch.float16, torch.bfloat16):
+        x.grad = w.grad = None
+        with torch.autocast("cuda", dtype=dt):
+            y = F.hip_blockwise_dropout_matmul_mask(x, mask, 64, 0.5, w)
+        assert y.dtype == dt
+        y.float().sum().backward()
+        assert x.grad.dtype == torch.float32 and w.grad.dtype == torch.float32
+        ref = O.dsd_forward(to_np(x.to(dt)), to_np(w.to(dt)), mask.cpu().numpy(), 64, 0.5, np.float32)
+        assert rel_fro(y, ref) <= REL_FRO_TOL
+        ones = np.ones((256, 128), dtype=np.float32)
+        assert rel_fro(x.grad, O.sdd_dx(ones, to_np(w.to(dt)), mask.cpu().numpy(), 64, 0.5, np.float32)) <= REL_FRO_TOL
+        assert rel_fro(w.grad, O.dsd_dw(ones, to_np(x.to(dt)), mask.cpu().numpy(), 64, 0.5, np.float32)) <= REL_FRO_TOL
+
+
+def test_public_names_and_p_range():
+    import flash_dropout.functional as F
+
+    for name in ("cuda_blockwise_dropout_matmul", "triton_blockwise_dropout_matmul", "im2col_conv2d",
+                 "naive_blockwise_dropout_matmul", "vanilla_dropout_matmul"):
+        assert callable(getattr(F, name))
+    x = torch.randn(128, 128, device="cuda", dtype=torch.float16)
+    with pytest.raises(ValueError, match=r"\[0, 1\)"):
+        F.cuda_blockwise_dropout_matmul(x, x, 64, 1.0)
+    y = F.cuda_blockwise_dropout_matmul(x, x, 64, 0.0)
+    assert rel_fro(y, to_np(x) @ to_np(x).T) <= REL_FRO_TOL
+    # statistical sanity of the fresh mask: about p of the blocks are dropped
+    big = torch.ones(4096, 4096, device="cuda", dtype=torch.float16)
+    eye = torch.eye(4096, device="cuda", dtype=torch.float16)
+    torch.cuda.manual_seed(0)
+    out = F.cuda_blockwise_dropout_matmul(big, eye, 64, 0.25)
+    frac_dropped = (out == 0).float().mean().item()
+    assert abs(frac_dropped - 0.25) < 0.03
+    assert torch.all((out == 0) | (out == torch.tensor(1 / 0.75, dtype=torch.float16, device="cuda")))

@@ -1,0 +1,263 @@
+"""Kernels (b)(c)(d) through the C ABI: gemm / gemm_dsd / gemm_sdd against the CPU oracle.
+
+Mirrors the structure of the reference's own parity test (test/test_cuda.py:23-57): same shape grid,
+same p grid, one mask tensor handed to both sides, three outputs (C, dA, dB) checked — with the
+tolerance the north star states (relative Frobenius error <= 1e-2 against the fp32 oracle on the
+fp16-rounded inputs) in addition to the reference's own assert_close(atol=0.2, rtol=0.01).
+"""
+from itertools import product
+
+import numpy as np
+import pytest
+import torch
+
+from _util import REL_FRO_TOL, cpu_mask, make_operand, rel_fro, to_np
+from oracle import sparsedrop_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _three_products(A, B, dC, mask, bs, p):
+    """The three calls exactly as the reference's autograd function issues them."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    s = 1 / (1 - p)
+    C = ext.gemm_dsd(A, B, mask, bs, s)
+    dA = ext.gemm_sdd(dC, B.T, mask, bs, s)
+    dB = ext.gemm_dsd(A.T, dC.T, mask.T, bs, s).T
+    return C, dA, dB
+
+
+def _oracle_products(A, B, dC, mask, bs, p, dtype=np.float32):
+    a, b, dc, mk = to_np(A, dtype), to_np(B, dtype), to_np(dC, dtype), mask.cpu().numpy()
+    return (O.dsd_forward(a, b, mk, bs, p, dtype), O.sdd_dx(dc, b, mk, bs, p, dtype),
+            O.dsd_dw(dc, a, mk, bs, p, dtype))
+
+
+def _check(got, ref, what, atol=0.2, rtol=0.01):
+    err = rel_fro(got, ref)
+    assert err <= REL_FRO_TOL, f"{what}: relative Frobenius error {err:.3e}"
+    torch.testing.assert_close(got.float().cpu(), torch.from_numpy(np.asarray(ref, dtype=np.float32)),
+                               atol=atol, rtol=rtol)
+
+
+# the reference's grid (test/test_cuda.py:12-20)
+REF_MNKS = [(128, 128, 128), (512, 512, 512), (1024, 1024, 1024), (2048, 2048, 2048)]
+REF_PS = [0.0, 0.1, 0.2, 0.5, 0.9, 0.99, 0.999]
+
+
+@pytest.mark.parametrize("mnk,block_size,p", list(product(REF_MNKS, [128], REF_PS)))
+def test_reference_grid(mnk, block_size, p):
+    M, N, K = mnk
+    gen = torch.Generator().manual_seed(0)
+    A = make_operand(M, K, torch.float16, "cuda", gen=gen)
+    B = make_operand(N, K, torch.float16, "cuda", gen=gen)
+    dC = make_operand(M, N, torch.float16, "cuda", gen=gen)
+    mask = cpu_mask((M // block_size, K // block_size), p, gen).cuda()
+    C, dA, dB = _three_products(A, B, dC, mask, block_size, p)
+    rC, rdA, rdB = _oracle_products(A, B, dC, mask, block_size, p)
+    # p = 0.999 scales by 1000: the absolute tolerance scales with it, as values do
+    atol = 0.2 * max(1.0, (1 / (1 - p)) / 10)
+    _check(C, rC, "C", atol)
+    _check(dB, rdB, "dB", atol)
+    _check(dA, rdA, "dA", atol)
+    keep = O.expand_keep(mask.cpu().numpy(), block_size, M, K)
+    assert (dA.cpu().numpy()[~keep] == 0).all(), "dropped dX tiles must be exactly zero"
+
+
+@pytest.mark.parametrize("mnk", [(256, 256, 256), (1024, 1024, 1024), (2048, 2048, 2048)])
+@pytest.mark.parametrize("p", [0.0, 0.25, 0.5, 0.75])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_block64_square(mnk, p, dtype):
+    M, N, K = mnk
+    if dtype == torch.bfloat16 and M > 1024:
+        pytest.skip("bf16 covered at the smaller sizes")
+    bs = 64
+    gen = torch.Generator().manual_seed(1)
+    A = make_operand(M, K, dtype, "cuda", gen=gen)
+    B = make_operand(N, K, dtype, "cuda", scale=K ** -0.5, gen=gen)
+    dC = make_operand(M, N, dtype, "cuda", gen=gen)
+    mask = cpu_mask((M // bs, K // bs), p, gen).cuda()
+    C, dA, dB = _three_products(A, B, dC, mask, bs, p)
+    rC, rdA, rdB = _oracle_products(A, B, dC, mask, bs, p)
+    for got, ref, what in ((C, rC, "C"), (dA, rdA, "dA"), (dB, rdB, "dB")):
+        assert rel_fro(got, ref) <= REL_FRO_TOL, what
+
+
+LAYOUTS = list(product([True, False], repeat=3))  # A row-major?, B row-major?, mask row-major?
+
+
+@pytest.mark.parametrize("a_rm,b_rm,m_rm", LAYOUTS)
+@pytest.mark.parametrize("out_t", [False, True])
+def test_all_majorness_combinations(a_rm, b_rm, m_rm, out_t):
+    """The four operand layouts of the reference's manual script (binding_gemm.py:88-99) x mask layout
+    x output layout, for dense, DSD and SDD."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    M, N, K, bs, p = 256, 384, 512, 64, 0.4
+    gen = torch.Generator().manual_seed(2)
+    A = make_operand(M, K, torch.float16, "cuda", row_major=a_rm, gen=gen)
+    B = make_operand(N, K, torch.float16, "cuda", row_major=b_rm, gen=gen)
+    a, b = to_np(A), to_np(B)
+    got = ext.gemm(A, B, transposed_out=out_t)
+    assert got.shape == (M, N) and (got.stride(0) == 1) == out_t
+    assert rel_fro(got, a @ b.T) <= REL_FRO_TOL
+    mk = cpu_mask((M // bs, K // bs), p, gen)
+    mask = mk.cuda() if m_rm else mk.t().contiguous().cuda().t()
+    got = ext.gemm_dsd(A, B, mask, bs, 1 / (1 - p), transposed_out=out_t)
+    assert rel_fro(got, O.gemm_dsd(a, b, mk.numpy(), bs, 1 / (1 - p), np.float32)) <= REL_FRO_TOL
+    mk = cpu_mask((M // bs, N // bs), p, gen)
+    mask = mk.cuda() if m_rm else mk.t().contiguous().cuda().t()
+    got = ext.gemm_sdd(A, B, mask, bs, 1 / (1 - p), transposed_out=out_t)
+    ref = O.gemm_sdd(a, b, mk.numpy(), bs, 1 / (1 - p), np.float32)
+    assert rel_fro(got, ref) <= REL_FRO_TOL
+    assert (got.cpu().numpy()[ref == 0] == 0).all()
+
+
+@pytest.mark.parametrize("M,N,K,bs", [
+    (4096, 1024, 784, 64),   # MLP layer 1: K tail 784 = 12*64 + 16
+    (4096, 10, 1024, 64),    # MLP layer 3: N tail 10 (dY leading dimension 10: unaligned loads)
+    (1000, 130, 200, 64),    # tails everywhere
+    (100, 70, 50, 64),       # smaller than one block
+    (16384, 1536, 384, 64),  # transformer MLP up-projection
+    (16384, 384, 1536, 64),  # transformer MLP down-projection
+    (512, 512, 512, 256),    # large block
+    (300, 200, 500, 128),
+])
+@pytest.mark.parametrize("p", [0.5])
+def test_tails_and_model_shapes(M, N, K, bs, p):
+    gen = torch.Generator().manual_seed(3)
+    A = make_operand(M, K, torch.float16, "cuda", gen=gen)
+    B = make_operand(N, K, torch.float16, "cuda", scale=K ** -0.5, gen=gen)
+    dC = make_operand(M, N, torch.float16, "cuda", gen=gen)
+    mask = cpu_mask(O.mask_shape(M, K, bs), p, gen).cuda()
+    C, dA, dB = _three_products(A, B, dC, mask, bs, p)
+    rC, rdA, rdB = _oracle_products(A, B, dC, mask, bs, p)
+    for got, ref, what in ((C, rC, "C"), (dA, rdA, "dA"), (dB, rdB, "dB")):
+        assert rel_fro(got, ref) <= REL_FRO_TOL, what
+    keep = O.expand_keep(mask.cpu().numpy(), bs, M, K)
+    assert (dA.cpu().numpy()[~keep] == 0).all()
+
+
+def test_degenerate_masks():
+    M, N, K, bs = 256, 128, 320, 64
+    gen = torch.Generator().manual_seed(4)
+    A = make_operand(M, K, torch.float16, "cuda", gen=gen)
+    B = make_operand(N, K, torch.float16, "cuda", gen=gen)
+    dC = make_operand(M, N, torch.float16, "cuda", gen=gen)
+    masks = {
+        "row_dropped": torch.zeros(4, 5, dtype=torch.bool),
+        "col_dropped": torch.zeros(4, 5, dtype=torch.bool),
+        "all_dropped": torch.ones(4, 5, dtype=torch.bool),
+        "none_dropped": torch.zeros(4, 5, dtype=torch.bool),
+        "last_row_dropped": torch.zeros(4, 5, dtype=torch.bool),
+    }
+    masks["row_dropped"][1, :] = True
+    masks["col_dropped"][:, 2] = True
+    masks["last_row_dropped"][3, :] = True
+    for name, mk in masks.items():
+        C, dA, dB = _three_products(A, B, dC, mk.cuda(), bs, 0.5)
+        rC, rdA, rdB = _oracle_products(A, B, dC, mk, bs, 0.5)
+        for got, ref, what in ((C, rC, "C"), (dA, rdA, "dA"), (dB, rdB, "dB")):
+            assert rel_fro(got, ref) <= REL_FRO_TOL, (name, what)
+    C, dA, dB = _three_products(A, B, dC, masks["all_dropped"].cuda(), bs, 0.5)
+    assert (C == 0).all() and (dA == 0).all() and (dB == 0).all()
+    C, _, _ = _three_products(A, B, dC, masks["row_dropped"].cuda(), bs, 0.5)
+    assert (C[64:128] == 0).all()
+
+
+def test_lists_entry_points_match_mask_entry_points():
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    M, N, K, bs, p = 512, 256, 384, 64, 0.5
+    gen = torch.Generator().manual_seed(5)
+    A = make_operand(M, K, torch.float16, "cuda", gen=gen)
+    B = make_operand(N, K, torch.float16, "cuda", gen=gen)
+    dC = make_operand(M, N, torch.float16, "cuda", gen=gen)
+    mask = cpu_mask((M // bs, K // bs), p, gen).cuda()
+    lists = ext.build_lists(mask)
+    s = 1 / (1 - p)
+    assert torch.equal(ext.gemm_dsd_lists(A, B, lists, bs, s), ext.gemm_dsd(A, B, mask, bs, s))
+    assert torch.equal(ext.gemm_sdd_lists(dC, B.T, lists, bs, s), ext.gemm_sdd(dC, B.T, mask, bs, s))
+    dW = ext.gemm_dsd_lists(A.T, dC.T, lists.transposed(), bs, s, transposed_out=True).T
+    assert dW.is_contiguous()
+    assert torch.equal(dW, ext.gemm_dsd(A.T, dC.T, mask.T, bs, s).T)
+
+
+def test_errors_through_the_shim():
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    A = torch.randn(128, 128, device="cuda", dtype=torch.float16)
+    mask = torch.zeros(2, 2, dtype=torch.bool, device="cuda")
+    with pytest.raises(TypeError, match="float16 or bfloat16"):
+        ext.gemm_dsd(A.float(), A.float(), mask, 64, 1.0)
+    with pytest.raises(TypeError, match="Mask must be bool"):
+        ext.gemm_dsd(A, A, mask.to(torch.uint8), 64, 1.0)
+    with pytest.raises(ValueError, match="mask shape"):
+        ext.gemm_dsd(A, A, torch.zeros(1, 2, dtype=torch.bool, device="cuda"), 64, 1.0)
+    with pytest.raises(ValueError, match="row or column major"):
+        ext.gemm(A[::2, ::2], A[:64, :64])
+    with pytest.raises(NotImplementedError, match="multiples of 64"):
+        ext.gemm_dsd(A, A, torch.zeros(3, 3, dtype=torch.bool, device="cuda"), 48, 1.0)
+    with pytest.raises(ValueError, match="reduction dims"):
+        ext.gemm(A, A[:, :64])
+
+
+def test_runs_on_the_current_stream():
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(6)
+    A = make_operand(512, 512, torch.float16, "cuda", gen=gen)
+    B = make_operand(512, 512, torch.float16, "cuda", gen=gen)
+    mask = cpu_mask((8, 8), 0.5, gen).cuda()
+    ref = ext.gemm_dsd(A, B, mask, 64, 2.0)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        got = ext.gemm_dsd(A, B, mask, 64, 2.0)
+    side.synchronize()
+    assert torch.equal(got, ref)
+
+
+@pytest.mark.parametrize("p", [0.0, 0.5])
+def test_full_size_8192_sampled_against_oracle(p):
+    """Headline size: the oracle is evaluated on sampled row/column blocks only (it is linear in rows
+    of A and of B, so any sub-block of the output is an independent oracle problem)."""
+    M = N = K = 8192
+    bs = 64
+    gen = torch.Generator().manual_seed(8)
+    A = make_operand(M, K, torch.float16, "cuda", gen=gen)
+    B = make_operand(N, K, torch.float16, "cuda", scale=K ** -0.5, gen=gen)
+    dC = make_operand(M, N, torch.float16, "cuda", gen=gen)
+    mask = cpu_mask((M // bs, K // bs), p, gen).cuda()
+    C, dA, dB = _three_products(A, B, dC, mask, bs, p)
+    mk = mask.cpu().numpy()
+    rows = np.r_[0:64, 4032:4160, 8128:8192]       # row blocks 0, 63, 64, 127
+    cols = np.r_[64:128, 5000:5100, 8100:8192]
+    a, b, dc = to_np(A), to_np(B), to_np(dC)
+    s = np.float32(1 / (1 - p))
+    keep = O.expand_keep(mk, bs, M, K)
+    # Y[rows, cols]
+    ref = (np.where(keep[rows], a[rows], 0) @ b[cols].T) * s
+    assert rel_fro(C.cpu().numpy()[np.ix_(rows, cols)], ref) <= REL_FRO_TOL
+    # dX[rows, cols]
+    ref = np.where(keep[np.ix_(rows, cols)], (dc[rows] @ b[:, cols]) * s, 0)
+    got = dA.cpu().numpy()[np.ix_(rows, cols)]
+    assert rel_fro(got, ref) <= REL_FRO_TOL
+    assert (dA.cpu().numpy()[~keep] == 0).all()
+    # dW[rows (of N), cols (of K)]
+    ref = (dc[:, rows].T @ np.where(keep[:, cols], a[:, cols], 0)) * s
+    assert rel_fro(dB.cpu().numpy()[np.ix_(rows, cols)], ref) <= REL_FRO_TOL
+    if p == 0.0:
+        from flash_dropout.hip import GEMM
+
+        # size-independent property: with nothing dropped DSD/SDD are the dense product (the kernels
+        # may sum in a different order, so to rounding rather than bit for bit)
+        ext = GEMM()
+        assert rel_fro(C, ext.gemm(A, B).float()) <= 1e-3
+        assert rel_fro(dA, ext.gemm(dC, B.T).float()) <= 1e-3

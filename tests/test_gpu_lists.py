@@ -1,0 +1,89 @@
+"""Kernel (a): block mask -> compacted kept-block lists, through the C ABI.  Bit-exact contract."""
+import json
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import sparsedrop_oracle as O
+
+pytestmark = pytest.mark.gpu
+GOLDEN = Path(__file__).parent / "golden"
+CASES = json.loads((GOLDEN / "compaction_cases.json").read_text())
+
+
+def _lists_np(lists):
+    nnz = lists.nnz()
+    return (lists.row_ptr.cpu().numpy(), lists.col_idx[:nnz].cpu().numpy(),
+            lists.col_ptr.cpu().numpy(), lists.row_idx[:nnz].cpu().numpy())
+
+
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_known_answers(name):
+    from flash_dropout.hip import GEMM
+
+    c = CASES[name]
+    g = GEMM()
+    mask = torch.tensor(c["mask"], dtype=torch.bool, device="cuda")
+    lists = g.build_lists(mask)
+    rp, ci, cp, ri = _lists_np(lists)
+    assert rp.dtype == np.int32 and ci.dtype == np.int32
+    assert rp.tolist() == c["row_ptr"] and ci.tolist() == c["col_idx"]
+    assert cp.tolist() == c["col_ptr"] and ri.tolist() == c["row_idx"]
+    table, row_indices, row_widths = g.increment_table(lists, c["block_k"])
+    assert table.dtype == torch.int64
+    assert table.cpu().tolist() == c["table"]
+    assert row_indices.cpu().tolist() == c["row_indices"]
+    assert row_widths.cpu().tolist() == c["row_widths"]
+
+
+@pytest.mark.parametrize("shape,p", [((16, 16), 0.5), ((128, 128), 0.5), ((128, 128), 0.0), ((128, 128), 1.0),
+                                     ((64, 13), 0.5), ((256, 6), 0.3), ((2048, 9), 0.5), ((1, 1), 0.0),
+                                     ((1, 300), 0.7), ((300, 1), 0.7), ((65, 129), 0.25), ((1000, 700), 0.9)])
+@pytest.mark.parametrize("col_major", [False, True])
+def test_random_masks_bit_exact(shape, p, col_major):
+    import flash_dropout.functional as F
+
+    gen = torch.Generator().manual_seed(shape[0] * 1000 + shape[1])
+    mask_cpu = torch.rand(*shape, generator=gen) < p
+    mask = mask_cpu.t().contiguous().cuda().t() if col_major else mask_cpu.cuda()
+    assert tuple(mask.shape) == shape
+    lists = F.kept_block_lists(mask)
+    rp, ci, cp, ri = _lists_np(lists)
+    erp, eci = O.compact_csr(mask_cpu.numpy())
+    ecp, eri = O.compact_csc(mask_cpu.numpy())
+    assert np.array_equal(rp, erp) and np.array_equal(ci, eci)
+    assert np.array_equal(cp, ecp) and np.array_equal(ri, eri)
+    # the library identity the reference relies on (blockwise_dropout_matmul_triton.py:48)
+    nz = torch.nonzero(~mask, as_tuple=False)
+    assert torch.equal(F.kept_block_table(mask), nz)
+    # transposed view swaps CSR and CSC
+    t = lists.transposed()
+    assert t.shape == (shape[1], shape[0]) and t.row_ptr is lists.col_ptr
+
+
+def test_large_mask_uses_multi_launch_path():
+    import flash_dropout.functional as F
+
+    gen = torch.Generator().manual_seed(7)
+    mask_cpu = torch.rand(1500, 400, generator=gen) < 0.6  # 600k entries > fused limit
+    lists = F.kept_block_lists(mask_cpu.cuda())
+    rp, ci, cp, ri = _lists_np(lists)
+    erp, eci = O.compact_csr(mask_cpu.numpy())
+    ecp, eri = O.compact_csc(mask_cpu.numpy())
+    assert np.array_equal(rp, erp) and np.array_equal(ci, eci)
+    assert np.array_equal(cp, ecp) and np.array_equal(ri, eri)
+
+
+@pytest.mark.parametrize("shape,p,bk", [((16, 16), 0.5, 64), ((40, 70), 0.8, 128), ((9, 3), 0.95, 16)])
+def test_increment_table_vs_oracle(shape, p, bk):
+    import flash_dropout.functional as F
+
+    gen = torch.Generator().manual_seed(11)
+    mask_cpu = torch.rand(*shape, generator=gen) < p
+    table, ri, rw = F.mask_to_increment_table(mask_cpu.cuda(), bk)
+    et, eri, erw = O.mask_to_increment_table(mask_cpu.numpy(), bk)
+    assert np.array_equal(table.cpu().numpy(), et)
+    assert np.array_equal(ri.cpu().numpy(), eri)
+    assert np.array_equal(rw.cpu().numpy(), erw)

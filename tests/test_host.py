@@ -1,0 +1,158 @@
+"""CPU-side checks: the C-ABI library loads and exports what include/sparsedrop.h declares, host-side
+argument validation (which runs before any GPU call), and the layer/host logic."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def _declared_symbols():
+    text = (ROOT / "include" / "sparsedrop.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sd_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from flash_dropout.hip import _loader
+
+    lib = _loader.load()
+    declared = _declared_symbols()
+    assert len(declared) >= 12
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in include/sparsedrop.h but not exported"
+    # and the ctypes table covers exactly the header
+    assert sorted(_loader.SIGNATURES) == declared
+    assert lib.sd_version() >= 100
+
+
+def test_workspace_bytes():
+    from flash_dropout.hip import _loader
+
+    lib = _loader.load()
+    assert lib.sd_workspace_bytes(128, 128) >= (129 + 128 * 128) * 4
+    assert lib.sd_workspace_bytes(1, 1) >= 12
+    assert lib.sd_workspace_bytes(-1, 4) == 0
+
+
+def test_host_validation_rejects_bad_arguments_without_touching_the_gpu():
+    from flash_dropout.hip import _loader
+
+    lib = _loader.load()
+    fake = ctypes.c_void_p(0x1000)
+    # neither stride is 1
+    rc = lib.sd_gemm(fake, 2, 2, fake, 8, 1, fake, 8, 1, 8, 8, 8, 0, None)
+    assert rc == 1 and b"row or column major" in lib.sd_last_error()
+    # bad dtype
+    rc = lib.sd_gemm(fake, 8, 1, fake, 8, 1, fake, 8, 1, 8, 8, 8, 7, None)
+    assert rc == 1 and b"dtype" in lib.sd_last_error()
+    # row stride shorter than the row
+    rc = lib.sd_gemm(fake, 4, 1, fake, 8, 1, fake, 8, 1, 8, 8, 8, 0, None)
+    assert rc == 1 and b"row stride" in lib.sd_last_error()
+    # unsupported block size
+    rc = lib.sd_gemm_dsd_lists(fake, 96, 1, fake, 96, 1, fake, 96, 1, fake, fake, 96, 96, 96, 48, 1.0, 0, None)
+    assert rc == 2 and b"multiples of 64" in lib.sd_last_error()
+    # workspace too small
+    rc = lib.sd_gemm_dsd(fake, 128, 1, fake, 128, 1, fake, 128, 1, fake, 2, 1, 128, 128, 128, 64, 2.0, 0, fake, 8, None)
+    assert rc == 1 and b"workspace too small" in lib.sd_last_error()
+    # null list
+    rc = lib.sd_gemm_sdd_lists(fake, 128, 1, fake, 128, 1, fake, 128, 1, None, None, 128, 128, 128, 64, 2.0, 0, None)
+    assert rc == 1 and b"null list" in lib.sd_last_error()
+    # build_lists argument checks
+    rc = lib.sd_build_lists(fake, 4, 4, 4, 1, None, None, None, None, None)
+    assert rc == 1 and b"nothing to build" in lib.sd_last_error()
+    rc = lib.sd_build_lists(fake, 0, 4, 4, 1, fake, fake, None, None, None)
+    assert rc == 1 and b"non-empty" in lib.sd_last_error()
+    # conv geometry
+    rc = lib.sd_im2col(fake, 1, 1, 1, 1, fake, 4, 1, 1, 2, 2, 3, 3, 0, 0, 1, 1, 1, 1, None, None, 0, 0, None)
+    assert rc == 1 and b"does not fit" in lib.sd_last_error()
+    rc = lib.sd_im2col(fake, 1, 1, 1, 1, fake, 4, 1, 1, 4, 4, 3, 3, 0, 0, 1, 1, 1, 1, None, None, 0, 0, None)
+    assert rc == 1 and b"cols_ld" in lib.sd_last_error()
+
+
+def test_python_shim_rejects_cpu_and_fp32_operands():
+    from flash_dropout.hip import GEMM
+
+    g = GEMM()
+    a = torch.randn(64, 64, dtype=torch.float16)
+    with pytest.raises(ValueError, match="GPU"):
+        g.gemm(a, a)
+    with pytest.raises(ValueError, match="GPU"):
+        g.build_lists(torch.zeros(2, 2, dtype=torch.bool))
+
+
+def test_block_size_int_or_equal_pair():
+    from flash_dropout.hip.binding_gemm import _block_size
+
+    assert _block_size(64) == 64
+    assert _block_size((128, 128)) == 128
+    with pytest.raises(ValueError):
+        _block_size((64, 128))
+    with pytest.raises(ValueError):
+        _block_size(0)
+
+
+def test_mask_helper_matches_reference_definition():
+    import flash_dropout.functional as F
+
+    x = torch.empty(3, 784, 100)
+    torch.manual_seed(5)
+    m = F.blockwise_dropout_mask(x, 64, 0.5)
+    torch.manual_seed(5)
+    again = torch.rand(3, 13, 2) < 0.5
+    assert m.dtype == torch.bool and torch.equal(m, again)
+    assert not F.blockwise_dropout_mask(x, (64, 64), 0.0).any()
+
+
+def test_dropout_mm_layer_host_logic():
+    from flash_dropout.layers import DropoutMM
+
+    torch.manual_seed(0)
+    layer = DropoutMM(16, 8, p=0.5, variant="blockwise[naive]", block_size=4)
+    assert layer.weight.shape == (8, 16) and not hasattr(layer, "bias")
+    x = torch.randn(2, 3, 16)
+    layer.eval()
+    assert torch.allclose(layer(x), torch.nn.functional.linear(x, layer.weight))
+    layer.train()
+    y = layer(x)
+    assert y.shape == (2, 3, 8)
+    for variant in ("none", "vanilla"):
+        assert DropoutMM(16, 8, variant=variant)(x).shape == (2, 3, 8)
+    bad = DropoutMM(16, 8, variant="nope")
+    with pytest.raises(ValueError, match="Unknown variant"):
+        bad(x)
+    # p = 0 block dropout is a plain linear
+    l0 = DropoutMM(16, 8, p=0.0, variant="blockwise[naive]", block_size=4)
+    assert torch.allclose(l0(x), torch.nn.functional.linear(x, l0.weight), atol=1e-6)
+
+
+def test_naive_variant_matches_oracle_with_tails():
+    import numpy as np
+
+    import flash_dropout.functional as F
+    from oracle import sparsedrop_oracle as O
+
+    torch.manual_seed(0)
+    x, w = torch.randn(10, 14, dtype=torch.float64), torch.randn(5, 14, dtype=torch.float64)
+    mask = torch.rand(3, 4) < 0.5
+    y = F.naive_blockwise_dropout_matmul_mask(x, mask, 4, 0.25, w)
+    np.testing.assert_allclose(y.numpy(), O.dsd_forward(x.numpy(), w.numpy(), mask.numpy(), 4, 0.25), rtol=1e-12)
+
+
+def test_dropout_conv_layer_host_logic():
+    from flash_dropout.layers import DropoutConv2d
+
+    torch.manual_seed(0)
+    x = torch.randn(2, 3, 8, 8)
+    conv = DropoutConv2d(3, 4, (3, 3), padding=(1, 1), p=0.0, variant="blockwise[naive]", block_size=4)
+    ref = torch.nn.functional.conv2d(x, conv.weight, padding=(1, 1))
+    assert torch.allclose(conv(x), ref, atol=1e-5)
+    conv.eval()
+    assert torch.allclose(conv(x), ref, atol=1e-6)
+    for variant in ("none", "vanilla", "vanilla_2d"):
+        assert DropoutConv2d(3, 4, (3, 3), padding=(1, 1), variant=variant)(x).shape == (2, 4, 8, 8)
+    with pytest.raises(ValueError, match="Unknown variant"):
+        DropoutConv2d(3, 4, (3, 3), variant="nope")(x)
