@@ -82,7 +82,11 @@ def test_cfg4_transformer_mlp(p):
 
 def test_cfg3_mlp_on_28x28_images_through_layers():
     """X[4096x784] uniform[0,1]; 784->1024->1024->10 with ReLU; block dropout p=0.5 on each hidden
-    input (layers 2 and 3) and, to exercise the K tail 784 = 12*64+16, on layer 1 as well."""
+    input (layers 2 and 3) and, to exercise the K tail 784 = 12*64+16, on layer 1 as well.
+
+    Parity is judged layer by layer on identical inputs: each layer's fp16 input and upstream gradient
+    are taken from the GPU run and handed to the oracle, so the 1e-2 bar applies to every product and
+    is not blurred by fp16 rounding accumulating through three layers and two ReLUs."""
     from flash_dropout.layers import DropoutMM
 
     torch.manual_seed(3)
@@ -91,38 +95,30 @@ def test_cfg3_mlp_on_28x28_images_through_layers():
     x = torch.rand(4096, 784).half()
     dy = torch.randn(4096, 10).half()
     mods = [l.cuda().half() for l in layers]
-    xg = x.cuda().requires_grad_()
 
-    # run the HIP layers with a fixed generator state so the masks can be re-drawn for the oracle
+    # fixed generator state so that the masks the layers draw can be re-drawn for the oracle
     torch.cuda.manual_seed(123)
     state = torch.cuda.get_rng_state()
-    h = xg
+    ins, outs = [], []
+    h = x.cuda().requires_grad_()
     for i, l in enumerate(mods):
+        h.retain_grad()
+        ins.append(h)
         h = l(h)
+        h.retain_grad()
+        outs.append(h)
         if i < 2:
             h = torch.relu(h)
     h.backward(dy.cuda())
 
     torch.cuda.set_rng_state(state)
-    masks = []
-    for i in range(3):
-        masks.append((torch.rand(64, -(-dims[i] // 64), device="cuda") < 0.5).cpu())
-
-    def expand(mask, m, k):
-        return torch.from_numpy(O.expand_keep(mask.numpy(), 64, m, k)).float()
-
-    xr = x.float().requires_grad_()
-    ws = [l.weight.detach().float().cpu().requires_grad_() for l in mods]
-    hr = xr
-    for i in range(3):
-        hr = torch.nn.functional.linear(hr * expand(masks[i], 4096, dims[i]) * 2.0, ws[i])
-        if i < 2:
-            hr = torch.relu(hr)
-    hr.backward(dy.float())
-    assert rel_fro(h, hr) <= REL_FRO_TOL
-    assert rel_fro(xg.grad, xr.grad) <= REL_FRO_TOL
-    for l, wr in zip(mods, ws):
-        assert rel_fro(l.weight.grad, wr.grad) <= REL_FRO_TOL
+    masks = [(torch.rand(64, -(-dims[i] // 64), device="cuda") < 0.5).cpu().numpy() for i in range(3)]
+    for i, l in enumerate(mods):
+        a, g, w = to_np(ins[i]), to_np(outs[i].grad), to_np(l.weight)
+        assert rel_fro(outs[i], O.dsd_forward(a, w, masks[i], 64, 0.5, np.float32)) <= REL_FRO_TOL, f"Y{i}"
+        assert rel_fro(ins[i].grad, O.sdd_dx(g, w, masks[i], 64, 0.5, np.float32)) <= REL_FRO_TOL, f"dX{i}"
+        assert rel_fro(l.weight.grad, O.dsd_dw(g, a, masks[i], 64, 0.5, np.float32)) <= REL_FRO_TOL, f"dW{i}"
+        assert l.weight.grad.shape == l.weight.shape
 
 
 def test_layer_eval_and_3d_inputs_and_bf16():
