@@ -15,6 +15,15 @@
 // which makes the MFMA fragment reads (ds_read_b128, 32 rows x one chunk per half-wave) hit all
 // 64 LDS banks; the swizzle is applied on the global side (which chunk a lane fetches), because the
 // LDS side of a direct load is fixed at lane*16.
+//
+// ---- DSD, both operands reduction-strided (the weight gradient dW = s*dY^T.(keep.X)) ------------
+// Same walk with the roles renamed: the "row blocks" are K blocks of X (rows of X^T), the list is the
+// CSC list (kept row blocks of X per K block), the reduction runs over M.  Tiles arrive in memory
+// order [reduction][64 or 256 contiguous columns] and the MFMA fragments (8 consecutive reduction
+// elements of one column per lane) are formed by ds_read_b64_tr_b16, two per fragment.  That read
+// takes, per 16-lane group, 4 reduction rows x 32 bytes; the chunk swizzles below put those on
+// distinct banks.  The MFMA operands are swapped so that lanes run along K, the contiguous index of
+// the row-major dW the kernel writes.
 #include "common.h"
 
 namespace sd {
@@ -59,9 +68,21 @@ __device__ inline void tile_of_block(int bid, int tiles_m, int tiles_n, int& tm,
   tn = in_group / gm;
 }
 
-template <typename T>
-__global__ __launch_bounds__(THREADS) void dsd_nt_kernel(GemmArgs g, int tiles_m, int tiles_n,
-                                                         int Mb, int Kb) {
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+
+// 4 reduction-consecutive halfs of one column, gathered from 4 LDS rows (see the file comment)
+__device__ inline u32x2 lds_read_tr(const char* p) {
+  s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p);
+  return __builtin_bit_cast(u32x2, v);
+}
+
+// TRANS = false: A[row][red], B[col][red] with the reduction index contiguous (forward / dense)
+// TRANS = true : A and B are given as transposed views, the reduction index is the strided one (dW)
+// In both cases "Mb" counts the row blocks of A (of X^T for dW) and "Kb" the reduction blocks.
+template <typename T, bool TRANS>
+__global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, int tiles_n,
+                                                      int Mb, int Kb) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   uint16_t* step_kb = reinterpret_cast<uint16_t*>(smem + SMEM_STEPS);
   uint8_t* step_fl = reinterpret_cast<uint8_t*>(smem + SMEM_FLAGS);
@@ -112,39 +133,81 @@ __global__ __launch_bounds__(THREADS) void dsd_nt_kernel(GemmArgs g, int tiles_m
   const int nsteps = *nsteps_p;
 
   // ---- per-lane constants ---------------------------------------------------------------------
-  // loads: a wave-wide load covers 8 tile rows; lane -> (row lane/8, physical chunk lane%8)
-  const int ld_row = lane / 8;
-  const int ld_pch = lane % 8;
-  // fragment reads: lane -> tile row lane%32 (+32*tile), logical chunk 2*ks + lane/32
-  const int fr_row = lane % 32;
-  const int fr_sw = (lane >> 1) & 7;
-  int koff[4];
+  // fragment reads
+  int a_off[4], b_off[4];  // byte offsets inside an X tile / the W tile, per 16-wide reduction step
+  if (!TRANS) {
+    // rows of 128 B; lane -> tile row lane%32 (+32*tile), logical 16 B chunk 2*ks + lane/32,
+    // physical chunk = logical ^ ((row>>1)&7)
+    const int fr_row = lane % 32;
+    const int fr_sw = (lane >> 1) & 7;
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks) koff[ks] = ((2 * ks + lane / 32) ^ fr_sw) * 16;
+    for (int ks = 0; ks < 4; ++ks) {
+      const int ko = ((2 * ks + lane / 32) ^ fr_sw) * 16;
+      a_off[ks] = fr_row * 128 + ko;
+      b_off[ks] = (ns * 64 + fr_row) * 128 + ko;
+    }
+  } else {
+    // rows are reduction indices.  16-lane group b = lane/16, lane = 16b + 4e + j reads 8 bytes of
+    // row (8*(b/2) + e) [+16*ks, +4 for the second half], columns 16*(b%2) + 4j .. +3 [+32*tile].
+    const int b4 = lane / 16, e = (lane % 16) / 4, j = lane % 4;
+    const int row = 8 * (b4 / 2) + e;
+    const int colchunk = 2 * (b4 % 2) + j / 2;  // 16 B chunk inside a 32-column tile
+    // X tile rows are 128 B (8 chunks): physical chunk = logical ^ (((row>>1)&1)<<2)
+    const int a_ch = colchunk ^ (((e >> 1) & 1) << 2);
+    // W tile rows are 512 B (32 chunks): physical chunk = logical ^ ((row&3)<<2)
+    const int b_ch = (ns * 8 + colchunk) ^ (e << 2);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      a_off[ks] = (16 * ks + row) * 128 + a_ch * 16 + (j % 2) * 8;
+      b_off[ks] = (16 * ks + row) * 512 + b_ch * 16 + (j % 2) * 8;
+    }
+  }
 
-  const uint16_t* a_base = g.a.ptr + (int64_t)rb0 * BS * g.a.sr;
-  const uint16_t* b_base = g.b.ptr + n0 * g.b.sr;
-
+  // global -> LDS: every wave-wide load fills 1 KB of LDS in lane order
   auto issue_loads = [&](int step, int stage) {
     const int kb = step_kb[step];
     const uint32_t fl = step_fl[step];
     char* st = smem + stage * STAGE;
-    // W tile: 32 row-octets, 4 per wave
+    if (!TRANS) {
+      // 8 tile rows per load; lane -> (row lane/8, physical chunk lane%8)
+      const int ld_row = lane / 8, ld_pch = lane % 8;
+      const uint16_t* a_base = g.a.ptr + (int64_t)rb0 * BS * g.a.sr + kb * BS;
+      const uint16_t* b_base = g.b.ptr + n0 * g.b.sr + kb * BS;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int oct = wave * 4 + j;
-      const int row = oct * 8 + ld_row;
-      const int ch = ld_pch ^ ((row >> 1) & 7);
-      load16_to_lds(b_base + (int64_t)row * g.b.sr + kb * BS + ch * 8, st + oct * 1024);
-    }
-    // X tiles of the row blocks that keep this K block: 8 row-octets each, one per wave
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      if (fl & (1u << r)) {
-        const int row = wave * 8 + ld_row;
+      for (int jj = 0; jj < 4; ++jj) {
+        const int oct = wave * 4 + jj;
+        const int row = oct * 8 + ld_row;
         const int ch = ld_pch ^ ((row >> 1) & 7);
-        load16_to_lds(a_base + (int64_t)(r * BS + row) * g.a.sr + kb * BS + ch * 8,
-                      st + A_OFF + r * TILE + wave * 1024);
+        load16_to_lds(b_base + (int64_t)row * g.b.sr + ch * 8, st + oct * 1024);
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        if (fl & (1u << r)) {
+          const int row = wave * 8 + ld_row;
+          const int ch = ld_pch ^ ((row >> 1) & 7);
+          load16_to_lds(a_base + (int64_t)(r * BS + row) * g.a.sr + ch * 8,
+                        st + A_OFF + r * TILE + wave * 1024);
+        }
+      }
+    } else {
+      // W tile: 2 reduction rows of 512 B per load; X tiles: 8 reduction rows of 128 B per load
+      const uint16_t* a_base = g.a.ptr + (int64_t)rb0 * BS + (int64_t)kb * BS * g.a.sc;
+      const uint16_t* b_base = g.b.ptr + n0 + (int64_t)kb * BS * g.b.sc;
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const int seg = wave * 4 + jj;
+        const int row = seg * 2 + lane / 32;
+        const int ch = (lane % 32) ^ ((row & 3) << 2);
+        load16_to_lds(b_base + (int64_t)row * g.b.sc + ch * 8, st + seg * 1024);
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        if (fl & (1u << r)) {
+          const int row = wave * 8 + lane / 8;
+          const int ch = (lane % 8) ^ (((row >> 1) & 1) << 2);
+          load16_to_lds(a_base + (int64_t)row * g.a.sc + r * BS + ch * 8,
+                        st + A_OFF + r * TILE + wave * 1024);
+        }
       }
     }
   };
@@ -173,8 +236,16 @@ __global__ __launch_bounds__(THREADS) void dsd_nt_kernel(GemmArgs g, int tiles_m
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
-          bf[nt][ks] = *reinterpret_cast<const u32x4*>(st + (ns * 64 + nt * 32 + fr_row) * 128 + koff[ks]);
+        for (int ks = 0; ks < 4; ++ks) {
+          if (!TRANS) {
+            bf[nt][ks] = *reinterpret_cast<const u32x4*>(st + b_off[ks] + nt * 32 * 128);
+          } else {
+            // the column tile toggles bit 2 of the chunk index, i.e. 64 bytes, under the XOR swizzle
+            const char* p = st + (b_off[ks] ^ (nt * 64));
+            const u32x2 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * 512);
+            bf[nt][ks] = u32x4{lo.x, lo.y, hi.x, hi.y};
+          }
+        }
 #pragma unroll
       for (int rr = 0; rr < 2; ++rr) {
         if (mine & (1u << rr)) {
@@ -183,15 +254,23 @@ __global__ __launch_bounds__(THREADS) void dsd_nt_kernel(GemmArgs g, int tiles_m
 #pragma unroll
           for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
-              af[mt][ks] = *reinterpret_cast<const u32x4*>(at + (mt * 32 + fr_row) * 128 + koff[ks]);
+            for (int ks = 0; ks < 4; ++ks) {
+              if (!TRANS) {
+                af[mt][ks] = *reinterpret_cast<const u32x4*>(at + a_off[ks] + mt * 32 * 128);
+              } else {
+                const char* p = at + (a_off[ks] ^ (mt * 64));
+                const u32x2 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * 128);
+                af[mt][ks] = u32x4{lo.x, lo.y, hi.x, hi.y};
+              }
+            }
 #pragma unroll
           for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
               for (int nt = 0; nt < 2; ++nt)
-                acc[rr][mt][nt] = T::mfma32(af[mt][ks], bf[nt][ks], acc[rr][mt][nt]);
+                acc[rr][mt][nt] = TRANS ? T::mfma32(bf[nt][ks], af[mt][ks], acc[rr][mt][nt])
+                                        : T::mfma32(af[mt][ks], bf[nt][ks], acc[rr][mt][nt]);
         }
       }
     }
@@ -199,7 +278,9 @@ __global__ __launch_bounds__(THREADS) void dsd_nt_kernel(GemmArgs g, int tiles_m
     __syncthreads();
   }
 
-  // ---- epilogue: scale, round once, store (row-major C) -----------------------------------------
+  // ---- epilogue: scale, round once, store ---------------------------------------------------------
+  // accumulator register v of lane l is element (8*(v/4) + 4*(l/32) + v%4, l%32) of the 32x32 product
+  // (first MFMA operand's rows) x (second operand's rows); lanes run along C's contiguous index.
 #pragma unroll
   for (int rr = 0; rr < 2; ++rr) {
     const int rb = rb0 + 2 * rh + rr;
@@ -210,30 +291,31 @@ __global__ __launch_bounds__(THREADS) void dsd_nt_kernel(GemmArgs g, int tiles_m
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const int row = mt * 32 + 8 * (v / 4) + 4 * (lane / 32) + (v % 4);
-          const int64_t m = (int64_t)rb * BS + row;
-          const int64_t n = n0 + ns * 64 + nt * 32 + (lane % 32);
-          g.c[m * g.c_sr + n] = T::from_float(acc[rr][mt][nt][v] * g.scale);
+          const int reg_i = 8 * (v / 4) + 4 * (lane / 32) + (v % 4);
+          const int lane_i = lane % 32;
+          const int64_t m = (int64_t)rb * BS + mt * 32 + (TRANS ? lane_i : reg_i);
+          const int64_t n = n0 + ns * 64 + nt * 32 + (TRANS ? reg_i : lane_i);
+          g.c[m * g.c_sr + n * g.c_sc] = T::from_float(acc[rr][mt][nt][v] * g.scale);
         }
   }
 }
 
 bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
 
-template <typename T>
-int launch_dsd_nt(const GemmArgs& g, hipStream_t stream) {
+template <typename T, bool TRANS>
+int launch_dsd(const GemmArgs& g, hipStream_t stream) {
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dsd_nt_kernel<T>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dsd_kernel<T, TRANS>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
     if (e != hipSuccess) return fail(SD_ERR_RUNTIME, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     configured = true;
   }
   const int Mb = (int)(g.M / BS), Kb = (int)(g.K / BS);
   const int tiles_m = (Mb + R - 1) / R, tiles_n = (int)(g.N / BN);
-  hipLaunchKernelGGL(dsd_nt_kernel<T>, dim3((unsigned)(tiles_m * tiles_n)), dim3(THREADS), SMEM_BYTES,
-                     stream, g, tiles_m, tiles_n, Mb, Kb);
-  return check_launch("dsd_nt_kernel");
+  hipLaunchKernelGGL((dsd_kernel<T, TRANS>), dim3((unsigned)(tiles_m * tiles_n)), dim3(THREADS),
+                     SMEM_BYTES, stream, g, tiles_m, tiles_n, Mb, Kb);
+  return check_launch("dsd_kernel");
 }
 
 }  // namespace
@@ -241,14 +323,18 @@ int launch_dsd_nt(const GemmArgs& g, hipStream_t stream) {
 int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   if (mode == kSdd) return SD_ERR_UNSUPPORTED;
   if (mode == kDsd && g.bs != BS) return SD_ERR_UNSUPPORTED;
-  // both operands reduction-contiguous, C row-major, everything tile-aligned and 16-byte aligned
-  const bool layout_ok = g.a.sc == 1 && g.b.sc == 1 && g.c_sc == 1;
+  // everything tile-aligned and 16-byte aligned; the three matrices agree on which index is contiguous
+  const bool nt = g.a.sc == 1 && g.b.sc == 1 && g.c_sc == 1;  // reduction-contiguous, C row-major
+  const bool tn = !nt && g.a.sr == 1 && g.b.sr == 1 && g.c_sr == 1;  // reduction-strided, C column-major
   const bool shape_ok = g.M > 0 && g.M % BS == 0 && g.N > 0 && g.N % BN == 0 && g.K > 0 &&
                         g.K % BS == 0 && g.K / BS <= MAX_STEPS;
-  const bool align_ok = aligned16(g.a.ptr) && aligned16(g.b.ptr) && g.a.sr % 8 == 0 && g.b.sr % 8 == 0;
+  const int64_t lda = nt ? g.a.sr : g.a.sc, ldb = nt ? g.b.sr : g.b.sc;
+  const bool align_ok = aligned16(g.a.ptr) && aligned16(g.b.ptr) && lda % 8 == 0 && ldb % 8 == 0;
   const int64_t tiles = ((g.M / BS + R - 1) / R) * (g.N / BN);
-  if (!(layout_ok && shape_ok && align_ok) || tiles > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
-  return dtype == SD_BF16 ? launch_dsd_nt<BF16>(g, stream) : launch_dsd_nt<F16>(g, stream);
+  if (!(nt || tn) || !shape_ok || !align_ok || tiles > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
+  if (nt)
+    return dtype == SD_BF16 ? launch_dsd<BF16, false>(g, stream) : launch_dsd<F16, false>(g, stream);
+  return dtype == SD_BF16 ? launch_dsd<BF16, true>(g, stream) : launch_dsd<F16, true>(g, stream);
 }
 
 }  // namespace sd
