@@ -24,6 +24,15 @@
 // takes, per 16-lane group, 4 reduction rows x 32 bytes; the chunk swizzles below put those on
 // distinct banks.  The MFMA operands are swapped so that lanes run along K, the contiguous index of
 // the row-major dW the kernel writes.
+//
+// ---- SDD (the input gradient dX = s*(dY.W) (.) keep) ----------------------------------------------
+// A workgroup owns a 4x4 patch of 64x64 output tiles and computes only the kept ones; the reduction
+// (over N) is dense.  Per 64-wide reduction step it loads the dY tiles of the row blocks that have
+// anything kept in the patch (reduction-contiguous, swizzled as in the forward) and the W tiles of the
+// column blocks that have anything kept (reduction-strided, read with ds_read_b64_tr_b16 as in dW).
+// Waves are (32x32 quadrant of every tile = wave%4) x (row-block pair = wave/4), so the two waves of a
+// SIMD together issue 4 MFMAs per kept tile per step: MFMA work follows the kept count and stays
+// balanced over the SIMDs.  Dropped tiles of the patch are written as zeros by the same workgroup.
 #include "common.h"
 
 namespace sd {
@@ -300,6 +309,162 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
   }
 }
 
+// A = dY [M, red] reduction-contiguous; B = W^T [cols, red] given with the reduction index strided
+// (b.sr == 1); C row-major.  Mb x Cb is the block grid of the output (and of the mask).
+template <typename T>
+__global__ __launch_bounds__(THREADS) void sdd_kernel(GemmArgs g, int tiles_m, int tiles_n, int Mb,
+                                                      int Cb) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  uint32_t* kept_p = reinterpret_cast<uint32_t*>(smem + 2 * STAGE);
+
+  int tm, tn;
+  tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int tid = threadIdx.x;
+  const int lane = tid % 64;
+  const int wave = tid / 64;
+  const int quad = wave % 4, mq = quad / 2, nq = quad % 2;
+  const int rh = wave / 4;
+  const int rb0 = tm * R, cb0 = tn * R;
+
+  // ---- which of the 16 tiles are kept: bit r*4 + c ------------------------------------------------
+  if (tid == 0) *kept_p = 0;
+  __syncthreads();
+  if (wave < R && rb0 + wave < Mb) {
+    const int beg = g.row_ptr[rb0 + wave], end = g.row_ptr[rb0 + wave + 1];
+    uint32_t bits = 0;
+    for (int i = beg + lane; i < end; i += 64) {
+      const int c = g.col_idx[i] - cb0;
+      if (c >= 0 && c < R) bits |= 1u << (wave * 4 + c);
+    }
+    if (bits) atomicOr(kept_p, bits);
+  }
+  __syncthreads();
+  const uint32_t kept = *kept_p;
+  uint32_t rowmask = 0, colmask = 0;  // row / column blocks with anything kept
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+    if ((kept >> (4 * r)) & 0xfu) rowmask |= 1u << r;
+#pragma unroll
+  for (int c = 0; c < R; ++c)
+    if (kept & (0x1111u << c)) colmask |= 1u << c;
+
+  // ---- zeros for the dropped tiles of the patch ---------------------------------------------------
+  {
+    const int row = tid / 8, ch = tid % 8;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    for (int r = 0; r < R; ++r) {
+      if (rb0 + r >= Mb) break;
+      for (int c = 0; c < R; ++c) {
+        if (cb0 + c >= Cb) break;
+        if (!((kept >> (4 * r + c)) & 1u))
+          *reinterpret_cast<u32x4*>(g.c + ((int64_t)(rb0 + r) * BS + row) * g.c_sr +
+                                    (int64_t)(cb0 + c) * BS + ch * 8) = z;
+      }
+    }
+  }
+  if (kept == 0) return;
+
+  // ---- per-lane constants ---------------------------------------------------------------------
+  int a_off[4], b_off[4];
+  {
+    const int fr_sw = (lane >> 1) & 7;
+    const int b4 = lane / 16, e = (lane % 16) / 4, j = lane % 4;
+    const int row = 8 * (b4 / 2) + e;
+    const int b_ch = (nq * 4 + 2 * (b4 % 2) + j / 2) ^ (((e >> 1) & 1) << 2);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      a_off[ks] = (mq * 32 + lane % 32) * 128 + ((2 * ks + lane / 32) ^ fr_sw) * 16;
+      b_off[ks] = (16 * ks + row) * 128 + b_ch * 16 + (j % 2) * 8;
+    }
+  }
+
+  const int nsteps = (int)(g.K / BS);
+  auto issue_loads = [&](int step, int stage) {
+    char* st = smem + stage * STAGE;
+    const int row = wave * 8 + lane / 8;
+    const int pch = lane % 8;
+    // dY tiles: [64 rows][64 red], chunk swizzle (row>>1)&7
+    const uint16_t* a_base = g.a.ptr + ((int64_t)rb0 * BS + row) * g.a.sr + step * BS +
+                             (pch ^ ((row >> 1) & 7)) * 8;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (rowmask & (1u << r))
+        load16_to_lds(a_base + (int64_t)r * BS * g.a.sr, st + r * TILE + wave * 1024);
+    // W tiles: [64 red][64 cols], chunk swizzle ((red>>1)&1)<<2
+    const uint16_t* b_base = g.b.ptr + (int64_t)cb0 * BS + ((int64_t)step * BS + row) * g.b.sc +
+                             (pch ^ (((row >> 1) & 1) << 2)) * 8;
+#pragma unroll
+    for (int c = 0; c < R; ++c)
+      if (colmask & (1u << c))
+        load16_to_lds(b_base + c * BS, st + A_OFF + c * TILE + wave * 1024);
+  };
+
+  f32x16 acc[2][R];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int c = 0; c < R; ++c)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[a][c][v] = 0.f;
+
+  const uint32_t mine = (kept >> (8 * rh)) & 0xffu;  // bit rr*4 + c
+  const uint32_t mycols = (mine | (mine >> 4)) & 0xfu;
+
+  issue_loads(0, 0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  for (int step = 0; step < nsteps; ++step) {
+    const int stage = step & 1;
+    if (step + 1 < nsteps) issue_loads(step + 1, stage ^ 1);
+    if (mine) {
+      const char* st = smem + stage * STAGE;
+      u32x4 af[2][4];
+#pragma unroll
+      for (int rr = 0; rr < 2; ++rr)
+        if ((mine >> (4 * rr)) & 0xfu) {
+#pragma unroll
+          for (int ks = 0; ks < 4; ++ks)
+            af[rr][ks] = *reinterpret_cast<const u32x4*>(st + (2 * rh + rr) * TILE + a_off[ks]);
+        }
+#pragma unroll
+      for (int c = 0; c < R; ++c) {
+        if (mycols & (1u << c)) {
+          const char* bt = st + A_OFF + c * TILE;
+          u32x4 bf[4];
+#pragma unroll
+          for (int ks = 0; ks < 4; ++ks) {
+            const u32x2 lo = lds_read_tr(bt + b_off[ks]), hi = lds_read_tr(bt + b_off[ks] + 4 * 128);
+            bf[ks] = u32x4{lo.x, lo.y, hi.x, hi.y};
+          }
+#pragma unroll
+          for (int rr = 0; rr < 2; ++rr)
+            if (mine & (1u << (4 * rr + c))) {
+#pragma unroll
+              for (int ks = 0; ks < 4; ++ks) acc[rr][c] = T::mfma32(af[rr][ks], bf[ks], acc[rr][c]);
+            }
+        }
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+
+  // ---- epilogue -----------------------------------------------------------------------------------
+#pragma unroll
+  for (int rr = 0; rr < 2; ++rr)
+#pragma unroll
+    for (int c = 0; c < R; ++c) {
+      if (!(mine & (1u << (4 * rr + c)))) continue;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int64_t m = (int64_t)(rb0 + 2 * rh + rr) * BS + mq * 32 + 8 * (v / 4) + 4 * (lane / 32) + (v % 4);
+        const int64_t n = (int64_t)(cb0 + c) * BS + nq * 32 + (lane % 32);
+        g.c[m * g.c_sr + n] = T::from_float(acc[rr][c][v] * g.scale);
+      }
+    }
+}
+
 bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
 
 template <typename T, bool TRANS>
@@ -318,10 +483,37 @@ int launch_dsd(const GemmArgs& g, hipStream_t stream) {
   return check_launch("dsd_kernel");
 }
 
+template <typename T>
+int launch_sdd(const GemmArgs& g, hipStream_t stream) {
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sdd_kernel<T>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
+    if (e != hipSuccess) return fail(SD_ERR_RUNTIME, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  const int Mb = (int)(g.M / BS), Cb = (int)(g.N / BS);
+  const int tiles_m = (Mb + R - 1) / R, tiles_n = (Cb + R - 1) / R;
+  hipLaunchKernelGGL(sdd_kernel<T>, dim3((unsigned)(tiles_m * tiles_n)), dim3(THREADS), SMEM_BYTES,
+                     stream, g, tiles_m, tiles_n, Mb, Cb);
+  return check_launch("sdd_kernel");
+}
+
+int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
+  if (g.bs != BS) return SD_ERR_UNSUPPORTED;
+  const bool layout_ok = g.a.sc == 1 && g.b.sr == 1 && g.b.sc != 1 && g.c_sc == 1;
+  const bool shape_ok = g.M > 0 && g.M % BS == 0 && g.N > 0 && g.N % BS == 0 && g.K > 0 && g.K % BS == 0;
+  const bool align_ok = aligned16(g.a.ptr) && aligned16(g.b.ptr) && aligned16(g.c) && g.a.sr % 8 == 0 &&
+                        g.b.sc % 8 == 0 && g.c_sr % 8 == 0;
+  const int64_t tiles = ((g.M / BS + R - 1) / R) * ((g.N / BS + R - 1) / R);
+  if (!layout_ok || !shape_ok || !align_ok || tiles > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
+  return dtype == SD_BF16 ? launch_sdd<BF16>(g, stream) : launch_sdd<F16>(g, stream);
+}
+
 }  // namespace
 
 int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
-  if (mode == kSdd) return SD_ERR_UNSUPPORTED;
+  if (mode == kSdd) return try_sdd(g, dtype, stream);
   if (mode == kDsd && g.bs != BS) return SD_ERR_UNSUPPORTED;
   // everything tile-aligned and 16-byte aligned; the three matrices agree on which index is contiguous
   const bool nt = g.a.sc == 1 && g.b.sc == 1 && g.c_sc == 1;  // reduction-contiguous, C row-major
