@@ -30,15 +30,29 @@ PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA peak
 METRIC = "fwd+bwd ms & effective TFLOP/s vs p (0–0.75) at 8192³ fp16; % of MFMA peak"
 
 
+LD_PAD = 0  # extra elements in every leading dimension (--ld-pad; 0 = dense row-major tensors)
+
+
+def _padded(t, dev):
+    import torch
+
+    if LD_PAD == 0:
+        return t.to(dev)
+    buf = torch.empty(t.shape[0], t.shape[1] + LD_PAD, dtype=t.dtype, device=dev)
+    view = buf[:, : t.shape[1]]
+    view.copy_(t)
+    return view
+
+
 def make_problem(size: int, p: float, bs: int, seed: int = 0):
     import torch
 
     gen = torch.Generator().manual_seed(seed)
     M = N = K = size
     dev = torch.device("cuda:0")
-    x = torch.randn(M, K, generator=gen).half().to(dev)
-    w = (torch.randn(N, K, generator=gen) / K ** 0.5).half().to(dev)
-    dy = torch.randn(M, N, generator=gen).half().to(dev)
+    x = _padded(torch.randn(M, K, generator=gen).half(), dev)
+    w = _padded((torch.randn(N, K, generator=gen) / K ** 0.5).half(), dev)
+    dy = _padded(torch.randn(M, N, generator=gen).half(), dev)
     mask = (torch.rand(M // bs, K // bs, generator=gen) < p).to(dev)  # CPU generator: device independent
     return x, w, dy, mask
 
@@ -56,9 +70,9 @@ class Step:
         self.scale = 1.0 / (1.0 - p)
         M, K = x.shape
         N = w.shape[0]
-        self.y = torch.empty(M, N, dtype=x.dtype, device=x.device)
-        self.dx = torch.empty(M, K, dtype=x.dtype, device=x.device)
-        self.dw_t = torch.empty(N, K, dtype=x.dtype, device=x.device).t()  # [K, N] view of row-major [N, K]
+        self.y = torch.empty(M, N + LD_PAD, dtype=x.dtype, device=x.device)[:, :N]
+        self.dx = torch.empty(M, K + LD_PAD, dtype=x.dtype, device=x.device)[:, :K]
+        self.dw_t = torch.empty(N, K + LD_PAD, dtype=x.dtype, device=x.device)[:, :K].t()  # [K, N] view of [N, K]
         self.lists = self.ext.build_lists(mask)
         kept = int((~mask).sum().item())
         self.kept_area = kept * bs * bs
@@ -154,8 +168,14 @@ def main() -> int:
     ap.add_argument("--block-size", type=int, default=64)
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--cpu-size", type=int, default=4096)
+    ap.add_argument("--cpu-size", type=int, default=8192)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 128 MiB device copy 3 times (known traffic, for scaling rocprof's FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--ld-pad", type=int, default=0,
+                    help="pad every leading dimension by this many elements (experiment: power-of-two row strides)")
     args = ap.parse_args()
+    global LD_PAD
+    LD_PAD = args.ld_pad
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
               "(the path has no collectives; sharding is described in DESIGN.md)", file=sys.stderr)
@@ -168,6 +188,14 @@ def main() -> int:
     entry.ensure_built()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     size, bs = args.size, args.block_size
+
+    if args.copy_calibration:
+        src = torch.empty(64 << 20, dtype=torch.float16, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- headline: K timed steps at p -----------------------------------------------------
     step = Step(*make_problem(size, args.p, bs), bs, args.p)

@@ -33,6 +33,8 @@
 // Waves are (32x32 quadrant of every tile = wave%4) x (row-block pair = wave/4), so the two waves of a
 // SIMD together issue 4 MFMAs per kept tile per step: MFMA work follows the kept count and stays
 // balanced over the SIMDs.  Dropped tiles of the patch are written as zeros by the same workgroup.
+#include <type_traits>
+
 #include "common.h"
 
 namespace sd {
@@ -52,11 +54,16 @@ constexpr int SMEM_SCRATCH = SMEM_FLAGS + MAX_STEPS;    // uint32 per K block wh
 constexpr int SMEM_BYTES = SMEM_SCRATCH + 4 * MAX_STEPS + 16;
 
 typedef __attribute__((address_space(3))) void lds_void;
-typedef const __attribute__((address_space(1))) void glb_void;
 
-// one wave-wide 1 KB direct load: lane i's 16 bytes land at lds_dst + 16*i
+// One wave-wide 1 KB direct global->LDS load: lane i's 16 bytes land at lds_dst + 16*i (lds_dst is
+// wave-uniform and goes through M0).  Issued as inline assembly on purpose: when the compiler sees a
+// direct-to-LDS load in flight it stops counting LDS reads precisely (every wait becomes
+// lgkmcnt(0), and transpose reads get a vmcnt(0) in front), which serialises the fragment reads with
+// the MFMAs.  Written this way the loads are invisible to its counters; the kernels wait for them
+// themselves with s_waitcnt vmcnt(0) before the barrier that publishes a stage.
 __device__ inline void load16_to_lds(const void* g, char* lds_dst) {
-  __builtin_amdgcn_global_load_lds((glb_void*)g, (lds_void*)lds_dst, 16, 0, 0);
+  const uint32_t a = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_void*)lds_dst);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(a) : "memory");
 }
 
 // Maps the launch index to an output tile so that the workgroups resident on one XCD (the hardware
@@ -172,53 +179,54 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
     }
   }
 
-  // global -> LDS: every wave-wide load fills 1 KB of LDS in lane order
-  auto issue_loads = [&](int step, int stage) {
-    const int kb = step_kb[step];
-    const uint32_t fl = step_fl[step];
-    char* st = smem + stage * STAGE;
-    if (!TRANS) {
-      // 8 tile rows per load; lane -> (row lane/8, physical chunk lane%8)
-      const int ld_row = lane / 8, ld_pch = lane % 8;
-      const uint16_t* a_base = g.a.ptr + (int64_t)rb0 * BS * g.a.sr + kb * BS;
-      const uint16_t* b_base = g.b.ptr + n0 * g.b.sr + kb * BS;
+  // global -> LDS: every wave-wide load fills 1 KB of LDS in lane order.  Per-lane byte offsets are
+  // fixed for the whole kernel; per step only a wave-uniform base moves.
+  uint32_t b_lane[4], a_lane;
+  const char* a_tile0;  // first X tile of the patch at reduction block 0
+  const char* b_tile0;  // W tile at reduction block 0
+  int64_t red_stride;   // bytes between consecutive reduction blocks
+  uint32_t a_rstride;   // bytes between consecutive row blocks of the patch
+  if (!TRANS) {
+    // 8 tile rows per load; lane -> (row lane/8, physical chunk lane%8)
+    const int ld_row = lane / 8, ld_pch = lane % 8;
 #pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const int oct = wave * 4 + jj;
-        const int row = oct * 8 + ld_row;
-        const int ch = ld_pch ^ ((row >> 1) & 7);
-        load16_to_lds(b_base + (int64_t)row * g.b.sr + ch * 8, st + oct * 1024);
-      }
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        if (fl & (1u << r)) {
-          const int row = wave * 8 + ld_row;
-          const int ch = ld_pch ^ ((row >> 1) & 7);
-          load16_to_lds(a_base + (int64_t)(r * BS + row) * g.a.sr + ch * 8,
-                        st + A_OFF + r * TILE + wave * 1024);
-        }
-      }
-    } else {
-      // W tile: 2 reduction rows of 512 B per load; X tiles: 8 reduction rows of 128 B per load
-      const uint16_t* a_base = g.a.ptr + (int64_t)rb0 * BS + (int64_t)kb * BS * g.a.sc;
-      const uint16_t* b_base = g.b.ptr + n0 + (int64_t)kb * BS * g.b.sc;
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const int seg = wave * 4 + jj;
-        const int row = seg * 2 + lane / 32;
-        const int ch = (lane % 32) ^ ((row & 3) << 2);
-        load16_to_lds(b_base + (int64_t)row * g.b.sc + ch * 8, st + seg * 1024);
-      }
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        if (fl & (1u << r)) {
-          const int row = wave * 8 + lane / 8;
-          const int ch = (lane % 8) ^ (((row >> 1) & 1) << 2);
-          load16_to_lds(a_base + (int64_t)row * g.a.sc + r * BS + ch * 8,
-                        st + A_OFF + r * TILE + wave * 1024);
-        }
-      }
+    for (int jj = 0; jj < 4; ++jj) {
+      const int row = (wave * 4 + jj) * 8 + ld_row;
+      b_lane[jj] = (uint32_t)(row * g.b.sr + (ld_pch ^ ((row >> 1) & 7)) * 8) * 2u;
     }
+    const int row = wave * 8 + ld_row;
+    a_lane = (uint32_t)(row * g.a.sr + (ld_pch ^ ((row >> 1) & 7)) * 8) * 2u;
+    a_tile0 = reinterpret_cast<const char*>(g.a.ptr + (int64_t)rb0 * BS * g.a.sr);
+    b_tile0 = reinterpret_cast<const char*>(g.b.ptr + n0 * g.b.sr);
+    red_stride = BS * 2;
+    a_rstride = (uint32_t)(BS * g.a.sr) * 2u;
+  } else {
+    // W tile: 2 reduction rows of 512 B per load; X tiles: 8 reduction rows of 128 B per load
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const int row = (wave * 4 + jj) * 2 + lane / 32;
+      b_lane[jj] = (uint32_t)(row * g.b.sc + ((lane % 32) ^ ((row & 3) << 2)) * 8) * 2u;
+    }
+    const int row = wave * 8 + lane / 8;
+    a_lane = (uint32_t)(row * g.a.sc + ((lane % 8) ^ (((row >> 1) & 1) << 2)) * 8) * 2u;
+    a_tile0 = reinterpret_cast<const char*>(g.a.ptr + (int64_t)rb0 * BS);
+    b_tile0 = reinterpret_cast<const char*>(g.b.ptr + n0);
+    red_stride = (int64_t)BS * g.a.sc * 2;  // == BS * g.b.sc * 2 only if the leading dimensions agree
+    a_rstride = BS * 2;
+  }
+  const int64_t b_red_stride = TRANS ? (int64_t)BS * g.b.sc * 2 : (int64_t)BS * 2;
+
+  auto issue_loads = [&](int step, int stage) {
+    const int kb = __builtin_amdgcn_readfirstlane((int)step_kb[step]);
+    const uint32_t fl = __builtin_amdgcn_readfirstlane((uint32_t)step_fl[step]);
+    char* st = smem + stage * STAGE;
+    const char* bp = b_tile0 + kb * b_red_stride;
+    const char* ap = a_tile0 + kb * red_stride;
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) load16_to_lds(bp + b_lane[jj], st + (wave * 4 + jj) * 1024);
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (fl & (1u << r)) load16_to_lds(ap + r * a_rstride + a_lane, st + A_OFF + r * TILE + wave * 1024);
   };
 
   f32x16 acc[2][2][2];  // [row block of the pair][m tile][n tile]
@@ -231,6 +239,65 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[a][b][c][v] = 0.f;
 
+  // fragment reads for one 16-wide reduction step ks: both 32-row tiles of an X tile / of the W slice
+  auto read_a = [&](const char* at, int ks, u32x4 (&dst)[2]) {
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+      if (!TRANS) {
+        dst[mt] = *reinterpret_cast<const u32x4*>(at + a_off[ks] + mt * 32 * 128);
+      } else {
+        // the 32-column tile toggles bit 2 of the chunk index, i.e. 64 bytes, under the XOR swizzle
+        const char* p = at + (a_off[ks] ^ (mt * 64));
+        const u32x2 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * 128);
+        dst[mt] = u32x4{lo.x, lo.y, hi.x, hi.y};
+      }
+    }
+  };
+  auto read_b = [&](const char* st, int ks, u32x4 (&dst)[2][4]) {
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      if (!TRANS) {
+        dst[nt][ks] = *reinterpret_cast<const u32x4*>(st + b_off[ks] + nt * 32 * 128);
+      } else {
+        const char* p = st + (b_off[ks] ^ (nt * 64));
+        const u32x2 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * 512);
+        dst[nt][ks] = u32x4{lo.x, lo.y, hi.x, hi.y};
+      }
+    }
+  };
+
+  // One step of MFMA work for this wave, specialised on which of its two row blocks keep the K block
+  // (MINE = 1, 2 or 3).  The work is a chain of units (row block, ks); the LDS reads of unit u+1 are
+  // issued before the MFMAs of unit u so that their latency hides behind 4 MFMAs (128 cycles).  The W
+  // fragments are read during the first row block's units and stay in registers for the second.
+  auto compute = [&](auto mine_c, const char* st) {
+    constexpr int MINE = decltype(mine_c)::value;
+    constexpr int NR = (MINE == 3) ? 2 : 1;
+    constexpr int R0 = (MINE == 2) ? 1 : 0;
+    u32x4 bf[2][4];
+    u32x4 af[2][2];
+    const char* at0 = st + A_OFF + (2 * rh + R0) * TILE;
+    read_b(st, 0, bf);
+    read_a(at0, 0, af[0]);
+#pragma unroll
+    for (int u = 0; u < NR * 4; ++u) {
+      const int rr = R0 + u / 4, ks = u % 4;
+      if (u + 1 < NR * 4) {
+        const int ks1 = (u + 1) % 4;
+        if (u + 1 < 4) read_b(st, ks1, bf);
+        read_a(at0 + ((u + 1) / 4) * TILE, ks1, af[(u + 1) & 1]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+          acc[rr][mt][nt] = TRANS ? T::mfma32(bf[nt][ks], af[u & 1][mt], acc[rr][mt][nt])
+                                  : T::mfma32(af[u & 1][mt], bf[nt][ks], acc[rr][mt][nt]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
   if (nsteps > 0) issue_loads(0, 0);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
@@ -238,51 +305,11 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
   for (int step = 0; step < nsteps; ++step) {
     const int stage = step & 1;
     if (step + 1 < nsteps) issue_loads(step + 1, stage ^ 1);
-    const uint32_t mine = (step_fl[step] >> (2 * rh)) & 3u;
-    if (mine) {
-      const char* st = smem + stage * STAGE;
-      u32x4 bf[2][4];
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-          if (!TRANS) {
-            bf[nt][ks] = *reinterpret_cast<const u32x4*>(st + b_off[ks] + nt * 32 * 128);
-          } else {
-            // the column tile toggles bit 2 of the chunk index, i.e. 64 bytes, under the XOR swizzle
-            const char* p = st + (b_off[ks] ^ (nt * 64));
-            const u32x2 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * 512);
-            bf[nt][ks] = u32x4{lo.x, lo.y, hi.x, hi.y};
-          }
-        }
-#pragma unroll
-      for (int rr = 0; rr < 2; ++rr) {
-        if (mine & (1u << rr)) {
-          const char* at = st + A_OFF + (2 * rh + rr) * TILE;
-          u32x4 af[2][4];
-#pragma unroll
-          for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-              if (!TRANS) {
-                af[mt][ks] = *reinterpret_cast<const u32x4*>(at + a_off[ks] + mt * 32 * 128);
-              } else {
-                const char* p = at + (a_off[ks] ^ (mt * 64));
-                const u32x2 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * 128);
-                af[mt][ks] = u32x4{lo.x, lo.y, hi.x, hi.y};
-              }
-            }
-#pragma unroll
-          for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-            for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-              for (int nt = 0; nt < 2; ++nt)
-                acc[rr][mt][nt] = TRANS ? T::mfma32(bf[nt][ks], af[mt][ks], acc[rr][mt][nt])
-                                        : T::mfma32(af[mt][ks], bf[nt][ks], acc[rr][mt][nt]);
-        }
-      }
-    }
+    const uint32_t mine = (__builtin_amdgcn_readfirstlane((uint32_t)step_fl[step]) >> (2 * rh)) & 3u;
+    const char* st = smem + stage * STAGE;
+    if (mine == 3u) compute(std::integral_constant<int, 3>{}, st);
+    else if (mine == 1u) compute(std::integral_constant<int, 1>{}, st);
+    else if (mine == 2u) compute(std::integral_constant<int, 2>{}, st);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   }
@@ -521,7 +548,8 @@ int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   const bool shape_ok = g.M > 0 && g.M % BS == 0 && g.N > 0 && g.N % BN == 0 && g.K > 0 &&
                         g.K % BS == 0 && g.K / BS <= MAX_STEPS;
   const int64_t lda = nt ? g.a.sr : g.a.sc, ldb = nt ? g.b.sr : g.b.sc;
-  const bool align_ok = aligned16(g.a.ptr) && aligned16(g.b.ptr) && lda % 8 == 0 && ldb % 8 == 0;
+  const bool align_ok = aligned16(g.a.ptr) && aligned16(g.b.ptr) && lda % 8 == 0 && ldb % 8 == 0 &&
+                        lda < (1 << 22) && ldb < (1 << 22);  // per-lane byte offsets are 32-bit
   const int64_t tiles = ((g.M / BS + R - 1) / R) * (g.N / BN);
   if (!(nt || tn) || !shape_ok || !align_ok || tiles > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
   if (nt)
