@@ -406,24 +406,31 @@ __global__ __launch_bounds__(THREADS) void sdd_kernel(GemmArgs g, int tiles_m, i
   }
 
   const int nsteps = (int)(g.K / BS);
-  auto issue_loads = [&](int step, int stage) {
-    char* st = smem + stage * STAGE;
+  // per-lane source pointers of the wave's 1 KiB of a tile at reduction step 0
+  const char* a_ptr0;
+  const char* b_ptr0;
+  {
     const int row = wave * 8 + lane / 8;
     const int pch = lane % 8;
     // dY tiles: [64 rows][64 red], chunk swizzle (row>>1)&7
-    const uint16_t* a_base = g.a.ptr + ((int64_t)rb0 * BS + row) * g.a.sr + step * BS +
-                             (pch ^ ((row >> 1) & 7)) * 8;
+    a_ptr0 = reinterpret_cast<const char*>(g.a.ptr + ((int64_t)rb0 * BS + row) * g.a.sr +
+                                           (pch ^ ((row >> 1) & 7)) * 8);
+    // W tiles: [64 red][64 cols], chunk swizzle ((red>>1)&1)<<2
+    b_ptr0 = reinterpret_cast<const char*>(g.b.ptr + (int64_t)cb0 * BS + (int64_t)row * g.b.sc +
+                                           (pch ^ (((row >> 1) & 1) << 2)) * 8);
+  }
+  const uint32_t a_tile_stride = (uint32_t)(BS * g.a.sr) * 2u;
+  const int64_t b_step_stride = (int64_t)BS * g.b.sc * 2;
+  auto issue_loads = [&](int step, int stage) {
+    char* st = smem + stage * STAGE + wave * 1024;
+    const char* ap = a_ptr0 + step * (BS * 2);
+    const char* bp = b_ptr0 + step * b_step_stride;
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      if (rowmask & (1u << r))
-        load16_to_lds(a_base + (int64_t)r * BS * g.a.sr, st + r * TILE + wave * 1024);
-    // W tiles: [64 red][64 cols], chunk swizzle ((red>>1)&1)<<2
-    const uint16_t* b_base = g.b.ptr + (int64_t)cb0 * BS + ((int64_t)step * BS + row) * g.b.sc +
-                             (pch ^ (((row >> 1) & 1) << 2)) * 8;
+      if (rowmask & (1u << r)) load16_to_lds(ap + r * a_tile_stride, st + r * TILE);
 #pragma unroll
     for (int c = 0; c < R; ++c)
-      if (colmask & (1u << c))
-        load16_to_lds(b_base + c * BS, st + A_OFF + c * TILE + wave * 1024);
+      if (colmask & (1u << c)) load16_to_lds(bp + c * (BS * 2), st + A_OFF + c * TILE);
   };
 
   f32x16 acc[2][R];
@@ -446,6 +453,7 @@ __global__ __launch_bounds__(THREADS) void sdd_kernel(GemmArgs g, int tiles_m, i
     if (step + 1 < nsteps) issue_loads(step + 1, stage ^ 1);
     if (mine) {
       const char* st = smem + stage * STAGE;
+      // this wave's 32-row slice of the dY tiles of its two row blocks, all four 16-wide sub-steps
       u32x4 af[2][4];
 #pragma unroll
       for (int rr = 0; rr < 2; ++rr)
@@ -454,23 +462,30 @@ __global__ __launch_bounds__(THREADS) void sdd_kernel(GemmArgs g, int tiles_m, i
           for (int ks = 0; ks < 4; ++ks)
             af[rr][ks] = *reinterpret_cast<const u32x4*>(st + (2 * rh + rr) * TILE + a_off[ks]);
         }
+      // W fragments of column block c+1 are read before the MFMAs of column block c
+      u32x4 bf[2][4];
+      auto read_b = [&](int c) {
+        const char* bt = st + A_OFF + c * TILE;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+          const u32x2 lo = lds_read_tr(bt + b_off[ks]), hi = lds_read_tr(bt + b_off[ks] + 4 * 128);
+          bf[c & 1][ks] = u32x4{lo.x, lo.y, hi.x, hi.y};
+        }
+      };
+      if (mycols & 1u) read_b(0);
 #pragma unroll
       for (int c = 0; c < R; ++c) {
+        if (c + 1 < R && (mycols & (1u << (c + 1)))) read_b(c + 1);
+        __builtin_amdgcn_sched_barrier(0);
         if (mycols & (1u << c)) {
-          const char* bt = st + A_OFF + c * TILE;
-          u32x4 bf[4];
-#pragma unroll
-          for (int ks = 0; ks < 4; ++ks) {
-            const u32x2 lo = lds_read_tr(bt + b_off[ks]), hi = lds_read_tr(bt + b_off[ks] + 4 * 128);
-            bf[ks] = u32x4{lo.x, lo.y, hi.x, hi.y};
-          }
 #pragma unroll
           for (int rr = 0; rr < 2; ++rr)
             if (mine & (1u << (4 * rr + c))) {
 #pragma unroll
-              for (int ks = 0; ks < 4; ++ks) acc[rr][c] = T::mfma32(af[rr][ks], bf[ks], acc[rr][c]);
+              for (int ks = 0; ks < 4; ++ks) acc[rr][c] = T::mfma32(af[rr][ks], bf[c & 1][ks], acc[rr][c]);
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
