@@ -27,6 +27,16 @@ for _p in (ROOT, ROOT / "sparse-dropout_amd"):
         sys.path.insert(0, str(_p))
 
 PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA peak
+
+# HBM/fabric bytes per launch of the three GEMM kernels at the headline workload (M=N=K=8192, p=0.5),
+# from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a 128 MiB device copy in the same run
+# (profiles/bench_8192_p50_pmc.txt: read factor 2.0, write factor 1.0).  Only reported when the
+# benchmark runs that workload; a counter run cannot be made from inside this process.
+MEASURED_TRAFFIC_BYTES = {
+    "dsd_forward": int((1585.0 + 129.1) * 2**20),
+    "sdd_dx": int((4709.3 + 128.0) * 2**20),
+    "dsd_dw": int((1531.9 + 141.4) * 2**20),
+}
 METRIC = "fwd+bwd ms & effective TFLOP/s vs p (0–0.75) at 8192³ fp16; % of MFMA peak"
 
 
@@ -220,7 +230,8 @@ def main() -> int:
         "peak": PEAK_FP16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": round(achieved / PEAK_FP16_TFLOPS, 4),
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC_BYTES.get(dominant) if (size == 8192 and args.p == 0.5 and bs == 64 and LD_PAD == 0) else None,
+        "traffic_unit": "bytes per launch (HBM/fabric reads + writes, rocprofv3 FETCH_SIZE/WRITE_SIZE, see profiles/)",
         "flops_per_launch": step.flops_fwd,
         "avg_launch_ms": round(kern_ms[dominant], 4),
         "all_kernels_ms": {k: round(v, 4) for k, v in kern_ms.items()},
@@ -287,7 +298,7 @@ def main() -> int:
         "roofline": roofline,
     }
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(args.cpu_size, bs, args.p, reps=3)
+        out["cpu_baseline"] = cpu_baseline(args.cpu_size, bs, args.p, reps=4)
     print(json.dumps(out))
     return 0
 

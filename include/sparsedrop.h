@@ -85,13 +85,23 @@ int sd_increment_table(const int32_t* row_ptr, const int32_t* col_idx, int64_t m
 /* Bytes of workspace the mask-taking GEMM entry points need for an mb x kb mask. */
 int64_t sd_workspace_bytes(int64_t mb, int64_t kb);
 
+/* Optional split-K scratch.  When the output has too few tiles to fill the GPU and the reduction is long
+ * (the weight gradient of a tall activation matrix), sd_gemm and the DSD entry points split the reduction
+ * over several workgroups and need fp32 scratch for the partial tiles: this returns how many bytes
+ * (0 = no split wanted) for C[M,N] with reduction length K; sparse = 0 for sd_gemm, 1 for DSD.
+ * Passing less (or NULL) is always allowed and only costs speed.  The mask-taking sd_gemm_dsd takes it
+ * appended to its list workspace: workspace_bytes >= round16(sd_workspace_bytes) + this.
+ * No counterpart in the reference (its kernels never split the reduction). */
+int64_t sd_splitk_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t block_size, int sparse);
+
 /* ---------------------------------------------------------------------------------------------
  * dense C[M,N] = A[M,K] * B[N,K]^T            replaces gemm()      gemm_binding.cu:47-54
  * ------------------------------------------------------------------------------------------- */
 int sd_gemm(const void* A, int64_t a_stride_r, int64_t a_stride_c,
             const void* B, int64_t b_stride_r, int64_t b_stride_c,
             void* C, int64_t c_stride_r, int64_t c_stride_c,
-            int64_t M, int64_t N, int64_t K, int dtype, void* stream);
+            int64_t M, int64_t N, int64_t K, int dtype,
+            void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * (b)/(d) DSD: C[M,N] = scale * sum over kept K-blocks of A's row-block of A_blk * B_blk^T
@@ -125,7 +135,7 @@ int sd_gemm_dsd_lists(const void* A, int64_t a_stride_r, int64_t a_stride_c,
                       void* C, int64_t c_stride_r, int64_t c_stride_c,
                       const int32_t* row_ptr, const int32_t* col_idx,
                       int64_t M, int64_t N, int64_t K, int64_t block_size, float scale, int dtype,
-                      void* stream);
+                      void* workspace, int64_t workspace_bytes, void* stream);
 
 int sd_gemm_sdd_lists(const void* A, int64_t a_stride_r, int64_t a_stride_c,
                       const void* B, int64_t b_stride_r, int64_t b_stride_c,

@@ -72,7 +72,8 @@ int run(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
 
 GemmArgs make_args(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc,
                    void* C, int64_t csr, int64_t csc, int64_t M, int64_t N, int64_t K, int64_t bs,
-                   float scale, const int32_t* row_ptr, const int32_t* col_idx) {
+                   float scale, const int32_t* row_ptr, const int32_t* col_idx, void* ws = nullptr,
+                   int64_t ws_bytes = 0) {
   GemmArgs g;
   g.a = Mat{(const uint16_t*)A, asr, asc};
   g.b = Mat{(const uint16_t*)B, bsr, bsc};
@@ -86,6 +87,10 @@ GemmArgs make_args(const void* A, int64_t asr, int64_t asc, const void* B, int64
   g.scale = scale;
   g.row_ptr = row_ptr;
   g.col_idx = col_idx;
+  // split-K scratch is optional: unusable pointers just mean "no split"
+  const bool ws_ok = ws != nullptr && ws_bytes > 0 && reinterpret_cast<uintptr_t>(ws) % 16 == 0;
+  g.ws = ws_ok ? static_cast<float*>(ws) : nullptr;
+  g.ws_bytes = ws_ok ? ws_bytes : 0;
   return g;
 }
 
@@ -127,20 +132,30 @@ int sd_increment_table(const int32_t* row_ptr, const int32_t* col_idx, int64_t m
   return increment_table(row_ptr, col_idx, mb, block_k, table, row_indices, row_widths, (hipStream_t)stream);
 }
 
+int64_t sd_splitk_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t block_size, int sparse) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  const int splits = generic_splits(M, N, K, sparse ? block_size : 0, sparse ? kDsd : kDense);
+  return splits > 1 ? (int64_t)splits * M * N * 4 : 0;
+}
+
 int sd_gemm(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc, void* C,
-            int64_t csr, int64_t csc, int64_t M, int64_t N, int64_t K, int dtype, void* stream) {
+            int64_t csr, int64_t csc, int64_t M, int64_t N, int64_t K, int dtype, void* workspace,
+            int64_t workspace_bytes, void* stream) {
   if (int rc = check_common(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, dtype)) return rc;
-  GemmArgs g = make_args(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, 0, 1.0f, nullptr, nullptr);
+  GemmArgs g = make_args(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, 0, 1.0f, nullptr, nullptr,
+                         workspace, workspace_bytes);
   return run(g, kDense, dtype, (hipStream_t)stream);
 }
 
 int sd_gemm_dsd_lists(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc,
                       void* C, int64_t csr, int64_t csc, const int32_t* row_ptr, const int32_t* col_idx,
-                      int64_t M, int64_t N, int64_t K, int64_t bs, float scale, int dtype, void* stream) {
+                      int64_t M, int64_t N, int64_t K, int64_t bs, float scale, int dtype,
+                      void* workspace, int64_t workspace_bytes, void* stream) {
   if (int rc = check_common(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, dtype)) return rc;
   if (int rc = check_sparse(bs, scale)) return rc;
   SD_REQUIRE(row_ptr && col_idx, "gemm_dsd: null list");
-  GemmArgs g = make_args(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, bs, scale, row_ptr, col_idx);
+  GemmArgs g = make_args(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, bs, scale, row_ptr, col_idx,
+                         workspace, workspace_bytes);
   return run(g, kDsd, dtype, (hipStream_t)stream);
 }
 
@@ -180,8 +195,11 @@ int sd_gemm_dsd(const void* A, int64_t asr, int64_t asc, const void* B, int64_t 
   if (int rc = lists_in_workspace(mask, msr, msc, ceil_div(M, bs), ceil_div(K, bs), workspace,
                                   workspace_bytes, &row_ptr, &col_idx, stream))
     return rc;
+  // whatever the caller provided beyond the lists serves as split-K scratch
+  const int64_t used = (sd_workspace_bytes(ceil_div(M, bs), ceil_div(K, bs)) + 15) / 16 * 16;
   return sd_gemm_dsd_lists(A, asr, asc, B, bsr, bsc, C, csr, csc, row_ptr, col_idx, M, N, K, bs, scale,
-                           dtype, stream);
+                           dtype, workspace_bytes > used ? (char*)workspace + used : nullptr,
+                           workspace_bytes > used ? workspace_bytes - used : 0, stream);
 }
 
 int sd_gemm_sdd(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc, void* C,

@@ -104,12 +104,17 @@ struct GemmArgs {
   float scale;
   const int32_t* row_ptr;  // CSR of the mask (DSD: over A; SDD: over C); null for dense
   const int32_t* col_idx;
+  float* ws;         // optional split-K workspace (fp32 partial tiles), may be null
+  int64_t ws_bytes;
 };
 
 enum Mode { kDense = 0, kDsd = 1, kSdd = 2 };
 
 // launchers (one per translation unit)
 int launch_generic(const GemmArgs& g, int mode, int dtype, hipStream_t stream);
+// number of reduction splits the generic kernel would like for this problem (1 = none); it needs
+// splits * M * N * 4 bytes of workspace for that
+int generic_splits(int64_t M, int64_t N, int64_t K, int64_t bs, int mode);
 // returns SD_ERR_UNSUPPORTED (without setting an error message) when the fast path does not apply
 int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream);
 

@@ -567,6 +567,12 @@ int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
                         lda < (1 << 22) && ldb < (1 << 22);  // per-lane byte offsets are 32-bit
   const int64_t tiles = ((g.M / BS + R - 1) / R) * (g.N / BN);
   if (!(nt || tn) || !shape_ok || !align_ok || tiles > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
+  // a long reduction over few output tiles (weight gradient of a tall matrix) is better served by the
+  // generic kernel's split-K when the caller gave it a workspace
+  if (tiles < 128 && g.ws != nullptr) {
+    const int splits = generic_splits(g.M, g.N, g.K, g.bs, mode);
+    if (splits > 1 && g.ws_bytes >= (int64_t)splits * g.M * g.N * 4) return SD_ERR_UNSUPPORTED;
+  }
   if (nt)
     return dtype == SD_BF16 ? launch_dsd<BF16, false>(g, stream) : launch_dsd<F16, false>(g, stream);
   return dtype == SD_BF16 ? launch_dsd<BF16, true>(g, stream) : launch_dsd<F16, true>(g, stream);

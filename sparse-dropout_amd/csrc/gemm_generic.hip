@@ -12,6 +12,10 @@
 //        tile lies in, so dropped blocks cost neither loads nor MFMAs.
 //   SDD (matmul_sdd.cuh:44-65): a wave whose 32x64 piece lies in a dropped output block skips its
 //        MFMAs and stores zeros; a workgroup with nothing kept skips the K loop altogether.
+//   Split-K: when the output has too few tiles to fill the chip and the reduction is long (the weight
+//        gradient of a tall activation matrix: dW[N,K] summed over M = 131072 rows for the conv
+//        configuration), blockIdx.y splits the reduction (for DSD: the row block's kept list); partial
+//        tiles go to an fp32 workspace and a second kernel sums, scales, rounds once and stores.
 #include "common.h"
 
 namespace sd {
@@ -97,18 +101,22 @@ struct KWalk {
   int64_t bs, K;
   int64_t k, kend;
   bool listed;
-  __device__ inline void init_dense(int64_t K_) {
+  // split s of S takes an equal share of the BK-steps (dense) or of the list entries (listed)
+  __device__ inline void init_dense(int64_t K_, int s, int S) {
     listed = false;
     K = K_;
-    k = 0;
-    kend = K_;
+    const int64_t steps = (K_ + BK - 1) / BK;
+    k = steps * s / S * BK;
+    kend = steps * (s + 1) / S * BK;
+    if (kend > K_) kend = K_;
   }
   __device__ inline void init_list(const int32_t* col_idx, int32_t beg, int32_t end_, int64_t bs_,
-                                   int64_t K_) {
+                                   int64_t K_, int s, int S) {
     listed = true;
     idx = col_idx;
-    pos = beg;
-    end = end_;
+    const int64_t len = end_ - beg;
+    pos = beg + (int32_t)(len * s / S);
+    end = beg + (int32_t)(len * (s + 1) / S);
     bs = bs_;
     K = K_;
     k = 0;
@@ -140,7 +148,7 @@ __device__ inline bool list_contains(const int32_t* idx, int32_t beg, int32_t en
   return false;
 }
 
-template <typename T, int MODE, bool TRANS_OUT>
+template <typename T, int MODE, bool TRANS_OUT, bool SPLIT>
 __global__ __launch_bounds__(THREADS) void gemm_generic_kernel(GemmArgs g, int tiles_n, bool a_kc,
                                                                bool b_kc, bool a_vec, bool b_vec) {
   __shared__ __attribute__((aligned(16))) uint16_t sA[BM * LDS_LD];
@@ -159,9 +167,10 @@ __global__ __launch_bounds__(THREADS) void gemm_generic_kernel(GemmArgs g, int t
   bool any_kept = true;
   if (MODE == kDsd) {
     const int64_t rb = m0 / g.bs;
-    walk.init_list(g.col_idx, g.row_ptr[rb], g.row_ptr[rb + 1], g.bs, g.K);
+    walk.init_list(g.col_idx, g.row_ptr[rb], g.row_ptr[rb + 1], g.bs, g.K, SPLIT ? blockIdx.y : 0,
+                   SPLIT ? gridDim.y : 1);
   } else {
-    walk.init_dense(g.K);
+    walk.init_dense(g.K, SPLIT ? blockIdx.y : 0, SPLIT ? gridDim.y : 1);
     if (MODE == kSdd) {
       const int64_t rb = m0 / g.bs;
       const int32_t beg = g.row_ptr[rb], end = g.row_ptr[rb + 1];
@@ -213,7 +222,8 @@ __global__ __launch_bounds__(THREADS) void gemm_generic_kernel(GemmArgs g, int t
     }
   }
 
-  // epilogue: scale in fp32, round once, predicated store.
+  // epilogue: scale in fp32, round once, predicated store (or the raw fp32 partial tile when the
+  // reduction is split).
   // MFMA result layout: register v of lane l is element (row 8*(v/4) + 4*(l/32) + v%4, col l%32)
   // of D = (first operand rows) x (second operand rows).
 #pragma unroll
@@ -224,9 +234,31 @@ __global__ __launch_bounds__(THREADS) void gemm_generic_kernel(GemmArgs g, int t
       const int lane_i = lane % 32;
       const int64_t m = m0 + wm * 32 + (TRANS_OUT ? lane_i : reg_i);
       const int64_t n = n0 + wn * 64 + j * 32 + (TRANS_OUT ? reg_i : lane_i);
-      if (m < g.M && n < g.N) g.c[m * g.c_sr + n * g.c_sc] = T::from_float(acc[j][v] * g.scale);
+      if (m < g.M && n < g.N) {
+        if (SPLIT) {
+          // workspace layout follows C's contiguous index so that lanes stay coalesced
+          const int64_t e = TRANS_OUT ? n * g.M + m : m * g.N + n;
+          g.ws[(int64_t)blockIdx.y * g.M * g.N + e] = acc[j][v];
+        } else {
+          g.c[m * g.c_sr + n * g.c_sc] = T::from_float(acc[j][v] * g.scale);
+        }
+      }
     }
   }
+}
+
+// C = scale * sum over splits of the fp32 partial tiles; one thread per element, lanes along C's
+// contiguous index (the workspace is laid out the same way).
+template <typename T>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs g, int splits, bool trans) {
+  const int64_t total = g.M * g.N;
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  float acc = 0.f;
+  for (int s = 0; s < splits; ++s) acc += g.ws[(int64_t)s * total + e];
+  const int64_t m = trans ? e % g.M : e / g.N;
+  const int64_t n = trans ? e / g.M : e % g.N;
+  g.c[m * g.c_sr + n * g.c_sc] = T::from_float(acc * g.scale);
 }
 
 template <typename T, int MODE>
@@ -241,12 +273,28 @@ int launch_t(const GemmArgs& g, hipStream_t stream) {
   };
   const bool a_vec = vec_ok(g.a), b_vec = vec_ok(g.b);
   const bool trans_out = (g.c_sr == 1 && g.c_sc != 1);
-  dim3 grid((unsigned)(tiles_m * tiles_n)), block(THREADS);
+  int splits = (MODE == kSdd) ? 1 : generic_splits(g.M, g.N, g.K, g.bs, MODE);
+  if (splits > 1 && (g.ws == nullptr || g.ws_bytes < (int64_t)splits * g.M * g.N * 4)) splits = 1;
+  dim3 block(THREADS);
+  if (splits > 1) {
+    dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)splits);
+    if (trans_out)
+      hipLaunchKernelGGL((gemm_generic_kernel<T, MODE, true, true>), grid, block, 0, stream, g,
+                         (int)tiles_n, a_kc, b_kc, a_vec, b_vec);
+    else
+      hipLaunchKernelGGL((gemm_generic_kernel<T, MODE, false, true>), grid, block, 0, stream, g,
+                         (int)tiles_n, a_kc, b_kc, a_vec, b_vec);
+    if (int rc = check_launch("gemm_generic (split)")) return rc;
+    hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)ceil_div(g.M * g.N, 256)), dim3(256), 0,
+                       stream, g, splits, trans_out);
+    return check_launch("splitk_reduce");
+  }
+  dim3 grid((unsigned)(tiles_m * tiles_n));
   if (trans_out)
-    hipLaunchKernelGGL((gemm_generic_kernel<T, MODE, true>), grid, block, 0, stream, g,
+    hipLaunchKernelGGL((gemm_generic_kernel<T, MODE, true, false>), grid, block, 0, stream, g,
                        (int)tiles_n, a_kc, b_kc, a_vec, b_vec);
   else
-    hipLaunchKernelGGL((gemm_generic_kernel<T, MODE, false>), grid, block, 0, stream, g,
+    hipLaunchKernelGGL((gemm_generic_kernel<T, MODE, false, false>), grid, block, 0, stream, g,
                        (int)tiles_n, a_kc, b_kc, a_vec, b_vec);
   return check_launch("gemm_generic");
 }
@@ -262,6 +310,21 @@ int launch_mode(const GemmArgs& g, int mode, hipStream_t stream) {
 }
 
 }  // namespace
+
+// Split the reduction when the output tiles alone cannot fill the 256 CUs and each tile has a long
+// reduction: aim for about two workgroups per CU, keep at least 8 K-steps (two 64-blocks) per split.
+int generic_splits(int64_t M, int64_t N, int64_t K, int64_t bs, int mode) {
+  if (mode == kSdd || M <= 0 || N <= 0) return 1;
+  const int64_t tiles = ceil_div(M, BM) * ceil_div(N, BN);
+  if (tiles >= 192 || K < 2048) return 1;
+  const int64_t units = (mode == kDsd && bs > 0) ? ceil_div(K, bs) : ceil_div(K, 64);
+  int64_t want = ceil_div(512, tiles);
+  if (want > units / 2) want = units / 2;
+  if (want > 128) want = 128;
+  // the product must stay a sane workspace: 256 MiB at most
+  while (want > 1 && want * M * N * 4 > (256LL << 20)) --want;
+  return want < 2 ? 1 : (int)want;
+}
 
 int launch_generic(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   if (g.M == 0 || g.N == 0) return SD_OK;

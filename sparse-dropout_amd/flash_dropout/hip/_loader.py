@@ -23,13 +23,14 @@ SIGNATURES = {
                                c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sd_increment_table": (c_int, [c_void_p, c_void_p, c_int64, c_int64,
                                    c_void_p, c_void_p, c_void_p, c_void_p]),
-    "sd_gemm": (c_int, [*_mat, *_mat, *_mat, c_int64, c_int64, c_int64, c_int, c_void_p]),
+    "sd_splitk_workspace_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int64, c_int]),
+    "sd_gemm": (c_int, [*_mat, *_mat, *_mat, c_int64, c_int64, c_int64, c_int, c_void_p, c_int64, c_void_p]),
     "sd_gemm_dsd": (c_int, [*_mat, *_mat, *_mat, *_mat, c_int64, c_int64, c_int64, c_int64,
                             c_float, c_int, c_void_p, c_int64, c_void_p]),
     "sd_gemm_sdd": (c_int, [*_mat, *_mat, *_mat, *_mat, c_int64, c_int64, c_int64, c_int64,
                             c_float, c_int, c_void_p, c_int64, c_void_p]),
     "sd_gemm_dsd_lists": (c_int, [*_mat, *_mat, *_mat, c_void_p, c_void_p, c_int64, c_int64,
-                                  c_int64, c_int64, c_float, c_int, c_void_p]),
+                                  c_int64, c_int64, c_float, c_int, c_void_p, c_int64, c_void_p]),
     "sd_gemm_sdd_lists": (c_int, [*_mat, *_mat, *_mat, c_void_p, c_void_p, c_int64, c_int64,
                                   c_int64, c_int64, c_float, c_int, c_void_p]),
     "sd_im2col": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64,

@@ -148,10 +148,21 @@ class GEMM:
         """Dense ``A @ B.T`` (reference: binding_gemm.py:26-27)."""
         self._check_pair(A, B)
         C = self._out(A, B, out, transposed_out)
+        if A.shape[0] == 0 or B.shape[0] == 0:
+            return C
+        ws, ws_ptr, ws_bytes = self._splitk_scratch(A, B, 0, 0)
         with torch.cuda.device(A.device):
             self._call(self.lib.sd_gemm, *_mat(A), *_mat(B), *_mat(C), A.shape[0], B.shape[0],
-                       A.shape[1], _DTYPES[A.dtype], self._stream(A))
+                       A.shape[1], _DTYPES[A.dtype], ws_ptr, ws_bytes, self._stream(A))
         return C
+
+    def _splitk_scratch(self, A, B, bs, sparse):
+        """fp32 scratch for a split reduction, when the library wants one for this shape."""
+        nbytes = self.lib.sd_splitk_workspace_bytes(A.shape[0], B.shape[0], A.shape[1], bs, sparse)
+        if nbytes <= 0:
+            return None, None, 0
+        ws = torch.empty(nbytes // 4, dtype=torch.float32, device=A.device)
+        return ws, ws.data_ptr(), nbytes
 
     def _masked(self, fn, mask_cols, A, B, mask, block_size, scale, out, transposed_out):
         self._check_pair(A, B)
@@ -162,7 +173,9 @@ class GEMM:
         C = self._out(A, B, out, transposed_out)
         if M == 0 or N == 0:
             return C
-        ws_bytes = self.lib.sd_workspace_bytes(mb, cb)
+        ws_bytes = (self.lib.sd_workspace_bytes(mb, cb) + 15) // 16 * 16
+        if mask_cols == "K":
+            ws_bytes += self.lib.sd_splitk_workspace_bytes(M, N, K, bs, 1)
         ws = torch.empty((ws_bytes + 3) // 4, dtype=torch.int32, device=A.device)
         with torch.cuda.device(A.device):
             self._call(fn, *_mat(A), *_mat(B), *_mat(C), mask.data_ptr(), *_mask_strides(mask),
@@ -225,10 +238,14 @@ class GEMM:
         C = self._out(A, B, out, transposed_out)
         if M == 0 or N == 0:
             return C
+        extra = ()
+        if mask_cols == "K":  # DSD may split a long reduction
+            ws, ws_ptr, ws_bytes = self._splitk_scratch(A, B, bs, 1)
+            extra = (ws_ptr, ws_bytes)
         with torch.cuda.device(A.device):
             self._call(fn, *_mat(A), *_mat(B), *_mat(C), lists.row_ptr.data_ptr(),
                        lists.col_idx.data_ptr(), M, N, K, bs, float(scale), _DTYPES[A.dtype],
-                       self._stream(A))
+                       *extra, self._stream(A))
         return C
 
     def gemm_dsd_lists(self, A, B, lists: KeptLists, block_size, scale, out=None, transposed_out=False):

@@ -33,6 +33,10 @@ def test_workspace_bytes():
     from flash_dropout.hip import _loader
 
     lib = _loader.load()
+    # split-K scratch: wanted for a long reduction over few tiles, not for a square problem
+    assert lib.sd_splitk_workspace_bytes(576, 128, 131072, 64, 1) >= 2 * 576 * 128 * 4
+    assert lib.sd_splitk_workspace_bytes(8192, 8192, 8192, 64, 1) == 0
+    assert lib.sd_splitk_workspace_bytes(64, 64, 512, 64, 0) == 0
     assert lib.sd_workspace_bytes(128, 128) >= (129 + 128 * 128) * 4
     assert lib.sd_workspace_bytes(1, 1) >= 12
     assert lib.sd_workspace_bytes(-1, 4) == 0
@@ -44,16 +48,16 @@ def test_host_validation_rejects_bad_arguments_without_touching_the_gpu():
     lib = _loader.load()
     fake = ctypes.c_void_p(0x1000)
     # neither stride is 1
-    rc = lib.sd_gemm(fake, 2, 2, fake, 8, 1, fake, 8, 1, 8, 8, 8, 0, None)
+    rc = lib.sd_gemm(fake, 2, 2, fake, 8, 1, fake, 8, 1, 8, 8, 8, 0, None, 0, None)
     assert rc == 1 and b"row or column major" in lib.sd_last_error()
     # bad dtype
-    rc = lib.sd_gemm(fake, 8, 1, fake, 8, 1, fake, 8, 1, 8, 8, 8, 7, None)
+    rc = lib.sd_gemm(fake, 8, 1, fake, 8, 1, fake, 8, 1, 8, 8, 8, 7, None, 0, None)
     assert rc == 1 and b"dtype" in lib.sd_last_error()
     # row stride shorter than the row
-    rc = lib.sd_gemm(fake, 4, 1, fake, 8, 1, fake, 8, 1, 8, 8, 8, 0, None)
+    rc = lib.sd_gemm(fake, 4, 1, fake, 8, 1, fake, 8, 1, 8, 8, 8, 0, None, 0, None)
     assert rc == 1 and b"row stride" in lib.sd_last_error()
     # unsupported block size
-    rc = lib.sd_gemm_dsd_lists(fake, 96, 1, fake, 96, 1, fake, 96, 1, fake, fake, 96, 96, 96, 48, 1.0, 0, None)
+    rc = lib.sd_gemm_dsd_lists(fake, 96, 1, fake, 96, 1, fake, 96, 1, fake, fake, 96, 96, 96, 48, 1.0, 0, None, 0, None)
     assert rc == 2 and b"multiples of 64" in lib.sd_last_error()
     # workspace too small
     rc = lib.sd_gemm_dsd(fake, 128, 1, fake, 128, 1, fake, 128, 1, fake, 2, 1, 128, 128, 128, 64, 2.0, 0, fake, 8, None)
