@@ -20,32 +20,38 @@ struct ConvGeom {
 };
 
 constexpr int TILE = 64;
-constexpr int TLD = TILE + 2;  // 33 words per LDS row: conflict-free turned reads
+constexpr int TLD = TILE + 2;  // 33 words per LDS row: both the 2-byte column writes and the 4-byte row reads are conflict-free
 
 __global__ __launch_bounds__(256) void im2col_kernel(const uint16_t* __restrict__ x,
                                                      uint16_t* __restrict__ cols, int64_t ld,
                                                      ConvGeom g, const int32_t* row_ptr,
                                                      const int32_t* col_idx, int bs) {
-  __shared__ uint16_t tile[TILE * TLD];
+  __shared__ __attribute__((aligned(4))) uint16_t tile[TILE * TLD];  // [row][col]
   const int t = threadIdx.x;
+  const int lane = t % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(t / 64);
   const int64_t rows = (int64_t)g.n * g.p * g.q;
   const int ncols = g.c * g.r * g.s;
   const int64_t r0 = (int64_t)blockIdx.x * TILE;
 
-  // this thread's row while gathering (fixed: 256 % 64 == 0)
-  const int64_t grow = r0 + (t % TILE);
+  // gather phase: lane = row of the tile, so a wave reads consecutive pixels of an image row
+  const int64_t grow = r0 + lane;
   const bool row_ok = grow < rows;
-  int n_i = 0, h_base = 0, w_base = 0;
+  int h_base = 0, w_base = 0;
+  const uint16_t* xrow = x;
   if (row_ok) {
     const int pq = (int)(grow % ((int64_t)g.p * g.q));
-    n_i = (int)(grow / ((int64_t)g.p * g.q));
+    const int n_i = (int)(grow / ((int64_t)g.p * g.q));
     h_base = (pq / g.q) * g.str_h - g.pad_h;
     w_base = (pq % g.q) * g.str_w - g.pad_w;
+    xrow = x + (int64_t)n_i * g.xs_n + (int64_t)h_base * g.xs_h + (int64_t)w_base * g.xs_w;
   }
-  const uint16_t* xn = x + (int64_t)n_i * g.xs_n;
+  // write phase: 32 lanes x 4 bytes cover the 128 bytes of one tile row; needs even, 4-byte aligned columns
+  const bool pair_ok = (ld % 2 == 0) && (reinterpret_cast<uintptr_t>(cols) % 4 == 0);
 
   const int sub_per_block = bs / TILE;  // 64-column tiles per mask block
   const int ntiles = (ncols + TILE - 1) / TILE;
+  const int rs_n = g.r * g.s;
   int32_t pos = 0, end = 0;
   if (row_ptr) {
     const int64_t rb = r0 / bs;
@@ -64,30 +70,150 @@ __global__ __launch_bounds__(256) void im2col_kernel(const uint16_t* __restrict_
       if (++ct >= ntiles) break;
     }
     const int c0 = ct * TILE;
-    // gather: lanes along rows (q fastest)
+    // gather: wave w takes columns w, w+4, ...; the column's (c, r, s) is wave-uniform
 #pragma unroll 4
-    for (int i = 0; i < TILE * TILE / 256; ++i) {
-      const int col_l = t / TILE + i * (256 / TILE);
+    for (int i = 0; i < TILE / 4; ++i) {
+      const int col_l = wave + 4 * i;
       const int col = c0 + col_l;
       uint16_t v = 0;
-      if (row_ok && col < ncols) {
-        const int ci = col / (g.r * g.s);
-        const int rs = col % (g.r * g.s);
-        const int hh = h_base + (rs / g.s) * g.dil_h;
-        const int ww = w_base + (rs % g.s) * g.dil_w;
-        if (hh >= 0 && hh < g.h && ww >= 0 && ww < g.w)
-          v = xn[(int64_t)ci * g.xs_c + (int64_t)hh * g.xs_h + (int64_t)ww * g.xs_w];
+      if (col < ncols) {
+        const int ci = col / rs_n;
+        const int rs = col - ci * rs_n;
+        const int dh = (rs / g.s) * g.dil_h;
+        const int dw = (rs % g.s) * g.dil_w;
+        const int hh = h_base + dh, ww = w_base + dw;
+        if (row_ok && hh >= 0 && hh < g.h && ww >= 0 && ww < g.w)
+          v = xrow[(int64_t)ci * g.xs_c + (int64_t)dh * g.xs_h + (int64_t)dw * g.xs_w];
       }
-      tile[col_l * TLD + (t % TILE)] = v;
+      tile[lane * TLD + col_l] = v;
     }
     __syncthreads();
-    // write: lanes along columns
+    // write: 4 bytes per lane, a full 128-byte line per half wave
+    if (pair_ok) {
 #pragma unroll 4
-    for (int i = 0; i < TILE * TILE / 256; ++i) {
-      const int row_l = t / TILE + i * (256 / TILE);
-      const int col_l = t % TILE;
-      const int64_t row = r0 + row_l;
-      if (row < rows && c0 + col_l < ncols) cols[row * ld + c0 + col_l] = tile[col_l * TLD + row_l];
+      for (int i = 0; i < TILE * TILE / 2 / 256; ++i) {
+        const int row_l = t / 32 + i * 8;
+        const int cp = (t % 32) * 2;
+        const int64_t row = r0 + row_l;
+        if (row < rows) {
+          const uint32_t two = *reinterpret_cast<const uint32_t*>(&tile[row_l * TLD + cp]);
+          uint16_t* dst = cols + row * ld + c0 + cp;
+          if (c0 + cp + 1 < ncols) *reinterpret_cast<uint32_t*>(dst) = two;
+          else if (c0 + cp < ncols) *dst = (uint16_t)two;
+        }
+      }
+    } else {
+#pragma unroll 4
+      for (int i = 0; i < TILE * TILE / 256; ++i) {
+        const int row_l = t / TILE + i * (256 / TILE);
+        const int col_l = t % TILE;
+        const int64_t row = r0 + row_l;
+        if (row < rows && c0 + col_l < ncols) cols[row * ld + c0 + col_l] = tile[row_l * TLD + col_l];
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// Patch-staged variant for the common case that the 64 rows of a workgroup lie in one image
+// ((P*Q) % 64 == 0): per 64-column tile the (at most 64/(R*S) + 2) input channels it touches are copied
+// once into LDS as a zero-padded patch [channel][input row][padded input column]; every output element
+// is then an LDS read with no bounds check, and a thread assembles 8 consecutive columns of one row
+// into a single 16-byte store.  Global reads drop to the unique bytes, global writes are full lines.
+constexpr int PATCH_MAX_BYTES = 48 * 1024;
+
+__global__ __launch_bounds__(256) void im2col_patch_kernel(const uint16_t* __restrict__ x,
+                                                           uint16_t* __restrict__ cols, int64_t ld,
+                                                           ConvGeom g, const int32_t* row_ptr,
+                                                           const int32_t* col_idx, int bs, int hp,
+                                                           int wp, int max_ch) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t patch[];  // [max_ch][hp][wp]
+  __shared__ int col_off[TILE];  // patch offset of each column of the tile (0 past the last column: never stored)
+  const int t = threadIdx.x;
+  const int ncols = g.c * g.r * g.s;
+  const int rs_n = g.r * g.s;
+  const int pq = g.p * g.q;
+  const int64_t r0 = (int64_t)blockIdx.x * TILE;
+  const int n_i = (int)(r0 / pq);
+  const int pq0 = (int)(r0 % pq);
+  const int p_lo = pq0 / g.q;
+  const int h_lo = p_lo * g.str_h - g.pad_h;  // input row of patch row 0
+  const uint16_t* xn = x + (int64_t)n_i * g.xs_n;
+
+  // per-thread output rows (two per tile): patch offset of their top-left tap
+  int row_off[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row_l = t / 8 + 32 * i;
+    const int pql = pq0 + row_l;
+    row_off[i] = ((pql / g.q - p_lo) * g.str_h) * wp + (pql % g.q) * g.str_w;
+  }
+
+  const int sub_per_block = bs / TILE;
+  const int ntiles = (ncols + TILE - 1) / TILE;
+  int32_t pos = 0, end = 0;
+  if (row_ptr) {
+    const int64_t rb = r0 / bs;
+    pos = row_ptr[rb];
+    end = row_ptr[rb + 1];
+  }
+  int sub = 0, ct = -1;
+  for (;;) {
+    if (row_ptr) {
+      if (pos >= end) break;
+      ct = col_idx[pos] * sub_per_block + sub;
+      if (++sub == sub_per_block) { sub = 0; ++pos; }
+      if (ct >= ntiles) continue;
+    } else {
+      if (++ct >= ntiles) break;
+    }
+    const int c0 = ct * TILE;
+    const int ch_lo = c0 / rs_n;
+    const int last = (c0 + TILE - 1 < ncols ? c0 + TILE - 1 : ncols - 1);
+    const int nch = last / rs_n - ch_lo + 1;
+    // stage the patch: lanes along the padded input column
+    const int per_ch = hp * wp;
+    for (int e = t; e < nch * per_ch; e += 256) {
+      const int ci = e / per_ch, rem = e - ci * per_ch;
+      const int hh = h_lo + rem / wp, ww = rem % wp - g.pad_w;
+      uint16_t v = 0;
+      if (hh >= 0 && hh < g.h && ww >= 0 && ww < g.w)
+        v = xn[(int64_t)(ch_lo + ci) * g.xs_c + (int64_t)hh * g.xs_h + (int64_t)ww * g.xs_w];
+      patch[e] = v;
+    }
+    if (t < TILE) {
+      const int col = c0 + t;
+      int off = 0;
+      if (col < ncols) {
+        const int ci = col / rs_n, rs = col - ci * rs_n;
+        off = ((ci - ch_lo) * hp + (rs / g.s) * g.dil_h) * wp + (rs % g.s) * g.dil_w;
+      }
+      col_off[t] = off;
+    }
+    __syncthreads();
+    const int ch8 = (t % 8) * 8;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int row_l = t / 8 + 32 * i;
+      uint16_t e[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int off = col_off[ch8 + j];
+        e[j] = patch[off + row_off[i]];
+      }
+      uint16_t* dst = cols + (r0 + row_l) * ld + c0 + ch8;
+      if (c0 + ch8 + 8 <= ncols) {
+        u32x4 v;
+        v.x = e[0] | ((uint32_t)e[1] << 16);
+        v.y = e[2] | ((uint32_t)e[3] << 16);
+        v.z = e[4] | ((uint32_t)e[5] << 16);
+        v.w = e[6] | ((uint32_t)e[7] << 16);
+        *reinterpret_cast<u32x4*>(dst) = v;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (c0 + ch8 + j < ncols) dst[j] = e[j];
+      }
     }
     __syncthreads();
   }
@@ -164,6 +290,20 @@ int im2col(const void* x, int64_t sn, int64_t sc, int64_t sh, int64_t sw, void* 
   const int64_t rows = n * g.p * g.q;
   const int64_t blocks = ceil_div(rows, TILE);
   SD_REQUIRE(blocks <= 0x7fffffffLL, "im2col: too many rows");
+  // patch-staged kernel: workgroup rows inside one image, 16-byte aligned stores, patch fits in LDS
+  const int64_t pq = (int64_t)g.p * g.q;
+  const int rows_p = (int)((TILE + g.q - 2) / g.q + 1);  // output rows p a 64-row group can touch
+  const int hp = (rows_p - 1) * g.str_h + (g.r - 1) * g.dil_h + 1;
+  const int wp = (g.q - 1) * g.str_w + (g.s - 1) * g.dil_w + 1;
+  const int max_ch = (int)((TILE + r * s - 2) / (r * s) + 1);
+  const int64_t patch_bytes = (int64_t)max_ch * hp * wp * 2;
+  if (pq % TILE == 0 && ld % 8 == 0 && reinterpret_cast<uintptr_t>(cols) % 16 == 0 &&
+      patch_bytes <= PATCH_MAX_BYTES) {
+    hipLaunchKernelGGL(im2col_patch_kernel, dim3((unsigned)blocks), dim3(256), (size_t)patch_bytes, stream,
+                       (const uint16_t*)x, (uint16_t*)cols, ld, g, row_ptr, col_idx,
+                       row_ptr ? (int)bs : TILE, hp, wp, max_ch);
+    return check_launch("im2col_patch");
+  }
   hipLaunchKernelGGL(im2col_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
                      (const uint16_t*)x, (uint16_t*)cols, ld, g, row_ptr, col_idx,
                      row_ptr ? (int)bs : TILE);

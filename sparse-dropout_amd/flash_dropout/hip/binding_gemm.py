@@ -263,9 +263,11 @@ class GEMM:
         return p, q
 
     def im2col(self, x: torch.Tensor, kernel_size, padding=(0, 0), stride=(1, 1), dilation=(1, 1),
-               lists: KeptLists | None = None, block_size=None) -> torch.Tensor:
+               lists: KeptLists | None = None, block_size=None,
+               out: torch.Tensor | None = None) -> torch.Tensor:
         """[N*P*Q, C*R*S] patch matrix in F.unfold column order.  With ``lists`` (over the block mask
-        of that matrix) only kept blocks are written; the rest of the buffer is uninitialised."""
+        of that matrix) only kept blocks are written; the rest of the buffer is left as it was
+        (uninitialised for a fresh one).  ``out`` may be any 2D view with unit column stride."""
         if x.dim() != 4 or not x.is_cuda or x.dtype not in _DTYPES:
             raise ValueError("x must be a 4D float16/bfloat16 tensor on the GPU")
         n, c, h, w = x.shape
@@ -273,7 +275,14 @@ class GEMM:
         p, q = self.conv_out_hw(h, w, r, s, padding, stride, dilation)
         if p <= 0 or q <= 0:
             raise ValueError("kernel does not fit the padded image")
-        cols = torch.empty((n * p * q, c * r * s), dtype=x.dtype, device=x.device)
+        if out is None:
+            cols = torch.empty((n * p * q, c * r * s), dtype=x.dtype, device=x.device)
+        else:
+            cols = out
+            if (tuple(cols.shape) != (n * p * q, c * r * s) or cols.dtype != x.dtype
+                    or cols.device != x.device or cols.stride(1) != 1):
+                raise ValueError(f"out must be a [{n * p * q}, {c * r * s}] {x.dtype} view on {x.device} "
+                                 "with unit column stride")
         rp = ci = None
         bs = 0
         if lists is not None:

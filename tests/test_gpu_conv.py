@@ -14,6 +14,12 @@ GEOMS = [
     dict(n=4, c=64, h=16, w=16, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)),
     dict(n=2, c=16, h=10, w=10, r=1, s=1, padding=(0, 0), stride=(1, 1), dilation=(1, 1)),
     dict(n=1, c=8, h=12, w=12, r=5, s=5, padding=(2, 2), stride=(2, 2), dilation=(1, 1)),
+    # P*Q a multiple of 64 and C*R*S a multiple of 8: the patch-staged im2col kernel
+    dict(n=2, c=24, h=24, w=24, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)),   # 216 columns: ragged tile
+    dict(n=2, c=8, h=32, w=32, r=3, s=3, padding=(1, 1), stride=(2, 2), dilation=(1, 1)),
+    dict(n=1, c=16, h=16, w=16, r=3, s=3, padding=(2, 2), stride=(1, 1), dilation=(2, 2)),
+    dict(n=2, c=8, h=16, w=16, r=5, s=5, padding=(2, 2), stride=(1, 1), dilation=(1, 1)),
+    dict(n=1, c=32, h=8, w=128, r=1, s=7, padding=(0, 3), stride=(1, 1), dilation=(1, 1)),   # a 64-row group inside one image row
 ]
 
 
@@ -38,23 +44,29 @@ def test_im2col_bit_exact(cfg, channels_last, dtype):
     assert np.array_equal(cols.float().cpu().numpy(), ref)  # a gather: bit exact
 
 
-@pytest.mark.parametrize("cfg", GEOMS[2:3])
-def test_im2col_writes_only_kept_blocks(cfg):
+@pytest.mark.parametrize("cfg", [
+    GEOMS[2],                                                                                   # patch-staged kernel
+    dict(n=4, c=64, h=12, w=12, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)),      # P*Q = 144: tile-turning kernel
+    dict(n=4, c=24, h=16, w=16, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)),      # 216 columns: ragged last block
+])
+@pytest.mark.parametrize("bs", [64, 128])
+def test_im2col_writes_only_kept_blocks(cfg, bs):
     from flash_dropout.hip import GEMM
 
     ext = GEMM()
     gen = torch.Generator().manual_seed(1)
     x = torch.randn(cfg["n"], cfg["c"], cfg["h"], cfg["w"], generator=gen).half().cuda()
-    rows, ncols = cfg["n"] * 16 * 16, cfg["c"] * 9
-    mask = cpu_mask(O.mask_shape(rows, ncols, 64), 0.5, gen)
+    ks = (cfg["r"], cfg["s"])
+    p_, q_ = O.conv_out_hw(cfg["h"], cfg["w"], *ks, **_geo(cfg))
+    rows, ncols = cfg["n"] * p_ * q_, cfg["c"] * cfg["r"] * cfg["s"]
+    mask = cpu_mask(O.mask_shape(rows, ncols, bs), 0.5, gen)
     lists = ext.build_lists(mask.cuda())
-    full = ext.im2col(x, (3, 3), **_geo(cfg))
-    # poison the allocator's next block so untouched entries are recognisable
-    poison = torch.full((rows, ncols), 7.0, dtype=torch.float16, device="cuda")
-    del poison
-    part = ext.im2col(x, (3, 3), lists=lists, block_size=64, **_geo(cfg))
-    keep = torch.from_numpy(O.expand_keep(mask.numpy(), 64, rows, ncols)).cuda()
+    full = ext.im2col(x, ks, **_geo(cfg))
+    part = torch.full((rows, ncols), 7.0, dtype=torch.float16, device="cuda")
+    ext.im2col(x, ks, lists=lists, block_size=bs, out=part, **_geo(cfg))
+    keep = torch.from_numpy(O.expand_keep(mask.numpy(), bs, rows, ncols)).cuda()
     assert torch.equal(part[keep], full[keep])
+    assert bool((part[~keep] == 7.0).all())  # dropped blocks are not touched
 
 
 @pytest.mark.parametrize("cfg", GEOMS)
