@@ -75,6 +75,29 @@ int sd_build_lists(const uint8_t* mask, int64_t mb, int64_t kb, int64_t mask_str
                    int64_t mask_stride_c, int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr,
                    int32_t* row_idx, void* stream);
 
+/* Block splitting: the same lists for the mask with every entry repeated split x split times, cropped
+ * to out_mb x out_kb ((mb-1)*split < out_mb <= mb*split, likewise out_kb); capacities out_mb*out_kb.
+ * A mask drawn at block size 64*split over an [M,K] operand is listed with out_mb = ceil(M/64),
+ * out_kb = ceil(K/64) and then drives the 64-block kernels (block_size 64 in the *_lists calls), which
+ * compute the same product: the repeated mask expands to the same element mask
+ * (flash_dropout/functional/naive.py:18-23 zeroes whole block_size x block_size tiles).  The reference
+ * fixes block_size = 128 = its tile (matmul_dsd.cuh:92-93) and has no counterpart. */
+int sd_build_lists_split(const uint8_t* mask, int64_t mb, int64_t kb, int64_t mask_stride_r,
+                         int64_t mask_stride_c, int64_t split, int64_t out_mb, int64_t out_kb,
+                         int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx,
+                         void* stream);
+
+/* Draws the mask on the device and lists it in the same launch: replaces
+ * blockwise_dropout_mask, flash_dropout/functional/utils.py:11-16 (torch.rand(mb, kb) < p, True =
+ * dropped) followed by the compaction above.  Entry e = i*kb + j is dropped iff
+ * (w >> 8) * 2^-24 < p (compared in fp32), w = word e%4 of Philox4x32-10 with counter
+ * (lo32(e/4), hi32(e/4), lo32(offset), hi32(offset)) and key (lo32(seed), hi32(seed)): a pure function
+ * of (seed, offset, e), not torch's generator stream.  mask_out receives the mb x kb mask as row-major
+ * bytes (the autograd context and parity tests keep it); split / out_mb / out_kb as above. */
+int sd_random_lists(uint64_t seed, uint64_t offset, float p, int64_t mb, int64_t kb, uint8_t* mask_out,
+                    int64_t split, int64_t out_mb, int64_t out_kb, int32_t* row_ptr, int32_t* col_idx,
+                    int32_t* col_ptr, int32_t* row_idx, void* stream);
+
 /* Pointer-increment table of flash_dropout/functional/utils.py:19-69 from a CSR list:
  * table[i] = col_idx[i]*block_k for the first kept block of a row, else (col_idx[i]-col_idx[i-1])*block_k;
  * row_indices[r] = row_ptr[r]; row_widths[r] = row_ptr[r+1]-row_ptr[r].
@@ -82,7 +105,10 @@ int sd_build_lists(const uint8_t* mask, int64_t mb, int64_t kb, int64_t mask_str
 int sd_increment_table(const int32_t* row_ptr, const int32_t* col_idx, int64_t mb, int64_t block_k,
                        int64_t* table, int64_t* row_indices, int64_t* row_widths, void* stream);
 
-/* Bytes of workspace the mask-taking GEMM entry points need for an mb x kb mask. */
+/* Bytes of workspace the mask-taking GEMM entry points need for an mb x kb mask.  For a block size that
+ * is a larger multiple of 64, a workspace sized for the 64-granular grid instead
+ * (sd_workspace_bytes(ceil(rows/64), ceil(cols/64)) of the masked matrix) makes them split the mask and
+ * run the 64-block kernels; the smaller size is accepted and runs the generic kernel. */
 int64_t sd_workspace_bytes(int64_t mb, int64_t kb);
 
 /* Optional split-K scratch.  When the output has too few tiles to fill the GPU and the reduction is long

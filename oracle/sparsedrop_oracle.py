@@ -23,6 +23,14 @@ Parity status of each function (what pins it is in tests/test_oracle.py):
                                            single-kept-block closed form, torch autograd of the
                                            literal naive.py restatement (oracle/naive_torch.py)
   im2col / col2im / conv2d_blockdrop       pinned: torch F.unfold / F.fold / F.conv2d library routines
+  philox4x32_10 / random_mask              pinned: the Random123 known-answer vectors for Philox4x32-10
+                                           (zeros, all ones, digits of pi); the mask on top of it is the
+                                           reference's definition ``uniform < p`` (utils.py:15) on a 24-bit
+                                           uniform, checked for polarity, p=0 and the empirical rate.  The
+                                           reference draws from torch's generator instead: equality of the
+                                           random STREAM is not part of the contract (parity is defined for
+                                           a given mask), only the distribution is
+  split_mask                               pinned: expand_keep identity (same element mask at both sizes)
 No function here is "parity unpinned".
 """
 from __future__ import annotations
@@ -38,6 +46,9 @@ __all__ = [
     "compact_csc",
     "kept_table",
     "mask_to_increment_table",
+    "philox4x32_10",
+    "random_mask",
+    "split_mask",
     "gemm_dsd",
     "gemm_sdd",
     "dsd_forward",
@@ -53,6 +64,61 @@ __all__ = [
 # --------------------------------------------------------------------------------------
 # mask + compaction (integer work; bit-exact contract)
 # --------------------------------------------------------------------------------------
+_PHILOX_M0, _PHILOX_M1 = 0xD2511F53, 0xCD9E8D57
+_PHILOX_W0, _PHILOX_W1 = 0x9E3779B9, 0xBB67AE85
+
+
+def philox4x32_10(counter, key) -> np.ndarray:
+    """Philox4x32 with 10 rounds (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as
+    1, 2, 3", SC'11, the generator family torch uses on GPUs).  ``counter`` is [..., 4] and ``key``
+    [..., 2] (broadcast), uint32 words; returns [..., 4] uint32.
+
+    One round: (hi0, lo0) = M0*c0, (hi1, lo1) = M1*c2 as 64-bit products;
+    c <- (hi1 ^ c1 ^ k0, lo1, hi0 ^ c3 ^ k1, lo0); the key is bumped by (W0, W1) between rounds.
+    """
+    c = np.array(counter, dtype=np.uint64) & 0xFFFFFFFF
+    k = np.array(key, dtype=np.uint64) & 0xFFFFFFFF
+    c0, c1, c2, c3 = (c[..., i] for i in range(4))
+    k0, k1 = k[..., 0], k[..., 1]
+    for _ in range(10):
+        p0 = _PHILOX_M0 * c0  # < 2^64: fits uint64 exactly
+        p1 = _PHILOX_M1 * c2
+        c0, c1, c2, c3 = ((p1 >> 32) ^ c1 ^ k0, p1 & 0xFFFFFFFF, (p0 >> 32) ^ c3 ^ k1, p0 & 0xFFFFFFFF)
+        k0 = (k0 + _PHILOX_W0) & 0xFFFFFFFF
+        k1 = (k1 + _PHILOX_W1) & 0xFFFFFFFF
+    return np.stack(np.broadcast_arrays(c0, c1, c2, c3), axis=-1).astype(np.uint32)
+
+
+def random_mask(shape: tuple[int, int], p: float, seed: int, offset: int = 0) -> np.ndarray:
+    """The block mask the library draws for (seed, offset): bool [mb, kb], True = dropped with
+    probability p — the reference's ``torch.rand(mb, kb) < p`` (utils.py:15) on a counter-based stream.
+
+    Entry e = i*kb + j takes word e % 4 of philox4x32_10(counter=(lo32(e//4), hi32(e//4),
+    lo32(offset), hi32(offset)), key=(lo32(seed), hi32(seed))); its top 24 bits make a uniform in
+    [0, 1) (exact in float32), compared with float32(p)."""
+    mb, kb = shape
+    e = np.arange(mb * kb, dtype=np.uint64)
+    blk = e >> np.uint64(2)
+    ctr = np.stack([blk & 0xFFFFFFFF, blk >> np.uint64(32),
+                    np.full_like(blk, offset & 0xFFFFFFFF), np.full_like(blk, (offset >> 32) & 0xFFFFFFFF)], axis=-1)
+    words = philox4x32_10(ctr, [seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF])
+    w = words[np.arange(mb * kb), (e & np.uint64(3)).astype(np.int64)]
+    u = (w >> np.uint32(8)).astype(np.float32) * np.float32(2.0 ** -24)
+    return (u < np.float32(p)).reshape(mb, kb)
+
+
+def split_mask(mask: np.ndarray, split: int, grid: tuple[int, int] | None = None) -> np.ndarray:
+    """Block splitting: every entry repeated split x split times, cropped to ``grid``.  A mask at
+    block size bs*split over an [m, k] matrix and its split at block size bs with
+    grid = mask_shape(m, k, bs) expand to the same element mask (naive.py:18-23 zeroes whole tiles)."""
+    mask = np.asarray(mask, dtype=bool)
+    out = np.repeat(np.repeat(mask, split, axis=0), split, axis=1)
+    if grid is not None:
+        assert (mask.shape[0] - 1) * split < grid[0] <= mask.shape[0] * split, (mask.shape, split, grid)
+        assert (mask.shape[1] - 1) * split < grid[1] <= mask.shape[1] * split, (mask.shape, split, grid)
+        out = out[: grid[0], : grid[1]]
+    return out
+
 def mask_shape(m: int, k: int, block_size: int) -> tuple[int, int]:
     """Shape of the block mask of an [m, k] matrix (utils.py:13-14: ceil on both axes)."""
     return (math.ceil(m / block_size), math.ceil(k / block_size))

@@ -11,9 +11,12 @@ char* last_error_buf() {
   return buf;
 }
 
-int build_lists(const uint8_t* mask, int64_t mb, int64_t kb, int64_t msr, int64_t msc,
-                int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx,
-                hipStream_t stream);
+int build_lists(const uint8_t* mask, int64_t msr, int64_t msc, int64_t stored_kb, int64_t split,
+                int64_t mb, int64_t kb, int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr,
+                int32_t* row_idx, hipStream_t stream);
+int random_lists(uint64_t seed, uint64_t offset, float p, int64_t stored_mb, int64_t stored_kb,
+                 uint8_t* mask_out, int64_t split, int64_t mb, int64_t kb, int32_t* row_ptr,
+                 int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx, hipStream_t stream);
 int increment_table(const int32_t* row_ptr, const int32_t* col_idx, int64_t mb, int64_t block_k,
                     int64_t* table, int64_t* row_indices, int64_t* row_widths, hipStream_t stream);
 int im2col(const void* x, int64_t sn, int64_t sc, int64_t sh, int64_t sw, void* cols, int64_t ld,
@@ -112,17 +115,46 @@ int64_t sd_workspace_bytes(int64_t mb, int64_t kb) {
   return ptr_bytes + mb * kb * 4;
 }
 
-int sd_build_lists(const uint8_t* mask, int64_t mb, int64_t kb, int64_t msr, int64_t msc,
-                   int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx,
-                   void* stream) {
-  SD_REQUIRE(mask != nullptr, "build_lists: null mask");
+static int check_list_grid(int64_t mb, int64_t kb, int64_t split, int64_t out_mb, int64_t out_kb,
+                           const int32_t* row_ptr, const int32_t* col_idx, const int32_t* col_ptr,
+                           const int32_t* row_idx) {
   SD_REQUIRE(mb > 0 && kb > 0, "build_lists: mask must be non-empty (got %lld x %lld)", (long long)mb, (long long)kb);
-  SD_REQUIRE(mb * kb < kMaxDim, "build_lists: mask too large for 32-bit lists");
-  SD_REQUIRE(msr >= 1 && msc >= 1 && (msr == 1 || msc == 1), "build_lists: mask must be row or column major");
+  SD_REQUIRE(split >= 1 && split < (1 << 16), "build_lists: split must be >= 1 (got %lld)", (long long)split);
+  // the listed grid is the mask repeated split x split, cropped inside its last row / column of entries
+  SD_REQUIRE(out_mb > (mb - 1) * split && out_mb <= mb * split && out_kb > (kb - 1) * split && out_kb <= kb * split,
+             "build_lists: a %lld x %lld grid does not match a %lld x %lld mask split by %lld", (long long)out_mb,
+             (long long)out_kb, (long long)mb, (long long)kb, (long long)split);
+  SD_REQUIRE(out_mb * out_kb < kMaxDim, "build_lists: mask too large for 32-bit lists");
   SD_REQUIRE((row_ptr == nullptr) == (col_idx == nullptr), "build_lists: pass both CSR arrays or neither");
   SD_REQUIRE((col_ptr == nullptr) == (row_idx == nullptr), "build_lists: pass both CSC arrays or neither");
   SD_REQUIRE(row_ptr || col_ptr, "build_lists: nothing to build");
-  return build_lists(mask, mb, kb, msr, msc, row_ptr, col_idx, col_ptr, row_idx, (hipStream_t)stream);
+  return SD_OK;
+}
+
+int sd_build_lists_split(const uint8_t* mask, int64_t mb, int64_t kb, int64_t msr, int64_t msc,
+                         int64_t split, int64_t out_mb, int64_t out_kb, int32_t* row_ptr,
+                         int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx, void* stream) {
+  SD_REQUIRE(mask != nullptr, "build_lists: null mask");
+  if (int rc = check_list_grid(mb, kb, split, out_mb, out_kb, row_ptr, col_idx, col_ptr, row_idx)) return rc;
+  SD_REQUIRE(msr >= 1 && msc >= 1 && (msr == 1 || msc == 1), "build_lists: mask must be row or column major");
+  return build_lists(mask, msr, msc, kb, split, out_mb, out_kb, row_ptr, col_idx, col_ptr, row_idx,
+                     (hipStream_t)stream);
+}
+
+int sd_build_lists(const uint8_t* mask, int64_t mb, int64_t kb, int64_t msr, int64_t msc,
+                   int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx,
+                   void* stream) {
+  return sd_build_lists_split(mask, mb, kb, msr, msc, 1, mb, kb, row_ptr, col_idx, col_ptr, row_idx, stream);
+}
+
+int sd_random_lists(uint64_t seed, uint64_t offset, float p, int64_t mb, int64_t kb, uint8_t* mask_out,
+                    int64_t split, int64_t out_mb, int64_t out_kb, int32_t* row_ptr, int32_t* col_idx,
+                    int32_t* col_ptr, int32_t* row_idx, void* stream) {
+  SD_REQUIRE(p >= 0.f && p < 1.f, "random_lists: p must be in [0, 1) (got %g)", (double)p);
+  SD_REQUIRE(mask_out != nullptr, "random_lists: null mask_out");
+  if (int rc = check_list_grid(mb, kb, split, out_mb, out_kb, row_ptr, col_idx, col_ptr, row_idx)) return rc;
+  return random_lists(seed, offset, p, mb, kb, mask_out, split, out_mb, out_kb, row_ptr, col_idx, col_ptr,
+                      row_idx, (hipStream_t)stream);
 }
 
 int sd_increment_table(const int32_t* row_ptr, const int32_t* col_idx, int64_t mb, int64_t block_k,
@@ -169,18 +201,32 @@ int sd_gemm_sdd_lists(const void* A, int64_t asr, int64_t asc, const void* B, in
   return run(g, kSdd, dtype, (hipStream_t)stream);
 }
 
-static int lists_in_workspace(const uint8_t* mask, int64_t msr, int64_t msc, int64_t mb, int64_t kb,
-                              void* workspace, int64_t workspace_bytes, int32_t** row_ptr,
-                              int32_t** col_idx, void* stream) {
+// Builds the CSR list of a [rows x cols] operand's mask at the head of the workspace.  When the block
+// size is a larger multiple of 64 and the workspace holds the finer list, the mask is listed at 64
+// granularity (each entry repeated) so that the 64-block kernels apply; *bs and *used report the choice.
+static int lists_in_workspace(const uint8_t* mask, int64_t msr, int64_t msc, int64_t rows, int64_t cols,
+                              int64_t* bs, void* workspace, int64_t workspace_bytes, int32_t** row_ptr,
+                              int32_t** col_idx, int64_t* used, void* stream) {
   SD_REQUIRE(mask != nullptr, "null mask");
+  const int64_t mb = ceil_div(rows, *bs), kb = ceil_div(cols, *bs);
   SD_REQUIRE(mb > 0 && kb > 0, "empty mask");
-  const int64_t need = sd_workspace_bytes(mb, kb);
+  int64_t split = 1, out_mb = mb, out_kb = kb;
+  if (*bs > 64 && *bs % 64 == 0 && ceil_div(rows, 64) * ceil_div(cols, 64) < kMaxDim &&
+      workspace_bytes >= sd_workspace_bytes(ceil_div(rows, 64), ceil_div(cols, 64))) {
+    split = *bs / 64;
+    out_mb = ceil_div(rows, 64);
+    out_kb = ceil_div(cols, 64);
+    *bs = 64;
+  }
+  const int64_t need = sd_workspace_bytes(out_mb, out_kb);
   SD_REQUIRE(workspace != nullptr && workspace_bytes >= need, "workspace too small: need %lld bytes, got %lld",
              (long long)need, (long long)workspace_bytes);
   SD_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, "workspace must be 16-byte aligned");
   *row_ptr = (int32_t*)workspace;
-  *col_idx = (int32_t*)((char*)workspace + ((mb + 1) * 4 + 15) / 16 * 16);
-  return sd_build_lists(mask, mb, kb, msr, msc, *row_ptr, *col_idx, nullptr, nullptr, stream);
+  *col_idx = (int32_t*)((char*)workspace + ((out_mb + 1) * 4 + 15) / 16 * 16);
+  *used = (need + 15) / 16 * 16;
+  return sd_build_lists_split(mask, mb, kb, msr, msc, split, out_mb, out_kb, *row_ptr, *col_idx, nullptr,
+                              nullptr, stream);
 }
 
 int sd_gemm_dsd(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc, void* C,
@@ -192,11 +238,11 @@ int sd_gemm_dsd(const void* A, int64_t asr, int64_t asc, const void* B, int64_t 
   if (M == 0 || N == 0) return SD_OK;
   SD_REQUIRE(K > 0, "gemm_dsd: K must be positive");
   int32_t *row_ptr, *col_idx;
-  if (int rc = lists_in_workspace(mask, msr, msc, ceil_div(M, bs), ceil_div(K, bs), workspace,
-                                  workspace_bytes, &row_ptr, &col_idx, stream))
+  int64_t used;
+  if (int rc = lists_in_workspace(mask, msr, msc, M, K, &bs, workspace, workspace_bytes, &row_ptr, &col_idx,
+                                  &used, stream))
     return rc;
   // whatever the caller provided beyond the lists serves as split-K scratch
-  const int64_t used = (sd_workspace_bytes(ceil_div(M, bs), ceil_div(K, bs)) + 15) / 16 * 16;
   return sd_gemm_dsd_lists(A, asr, asc, B, bsr, bsc, C, csr, csc, row_ptr, col_idx, M, N, K, bs, scale,
                            dtype, workspace_bytes > used ? (char*)workspace + used : nullptr,
                            workspace_bytes > used ? workspace_bytes - used : 0, stream);
@@ -210,8 +256,9 @@ int sd_gemm_sdd(const void* A, int64_t asr, int64_t asc, const void* B, int64_t 
   if (int rc = check_sparse(bs, scale)) return rc;
   if (M == 0 || N == 0) return SD_OK;
   int32_t *row_ptr, *col_idx;
-  if (int rc = lists_in_workspace(mask, msr, msc, ceil_div(M, bs), ceil_div(N, bs), workspace,
-                                  workspace_bytes, &row_ptr, &col_idx, stream))
+  int64_t used;
+  if (int rc = lists_in_workspace(mask, msr, msc, M, N, &bs, workspace, workspace_bytes, &row_ptr, &col_idx,
+                                  &used, stream))
     return rc;
   return sd_gemm_sdd_lists(A, asr, asc, B, bsr, bsc, C, csr, csc, row_ptr, col_idx, M, N, K, bs, scale,
                            dtype, stream);

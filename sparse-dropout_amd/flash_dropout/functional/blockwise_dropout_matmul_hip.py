@@ -8,37 +8,41 @@ Counterpart of the reference's ``BlockwiseDropoutMatmulCUDA``
               dW = gemm_dsd(X.T, dY.T, mask.T).T   (:49-51)
 
 Differences that matter to a caller: the kept-block lists are built once on the GPU in forward and
-reused by both backward products (no per-iteration mask reads, no host sync); dW comes back as a
-contiguous [N, K] tensor instead of a transposed view; bf16 works as well as fp16; shapes need not
-be multiples of anything; launches go to torch's current stream.
+reused by both backward products (no per-iteration mask reads, no host sync); without a given mask
+the Bernoulli draw happens inside the list-building launch; dW comes back as a contiguous [N, K]
+tensor instead of a transposed view; bf16 works as well as fp16; shapes need not be multiples of
+anything; block sizes that are multiples of 64 all run on the 64-block kernels; launches go to
+torch's current stream.
 """
 from __future__ import annotations
 
 import torch
 
 from ..hip.binding_gemm import GEMM, KeptLists, _block_size
-from .utils import blockwise_dropout_mask
 
 
 class BlockwiseDropoutMatmulHIP(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, input: torch.Tensor, weight: torch.Tensor, mask: torch.Tensor, block_size: int,
-                p: float):
+    def forward(ctx, input: torch.Tensor, weight: torch.Tensor, mask: torch.Tensor | None,
+                block_size: int, p: float, seed: int | None = None):
         ext = GEMM()
         scale = 1.0 / (1.0 - p)
-        lists = ext.build_lists(mask)
+        # mask given, or drawn in the list-building launch (reference: blockwise_dropout_mask, …_cuda.py:24)
+        mask, lists, kernel_bs = ext.kept_lists(input.shape[0], input.shape[1], block_size, mask, p, seed,
+                                                input.device)
         # C (M N) = A (M K sparse) * B (N K)
-        out = ext.gemm_dsd_lists(input, weight, lists, block_size, scale)
+        out = ext.gemm_dsd_lists(input, weight, lists, kernel_bs, scale)
         ctx.save_for_backward(input, weight, mask, lists.row_ptr, lists.col_idx, lists.col_ptr,
                               lists.row_idx)
-        ctx.block_size = block_size
+        ctx.block_size = kernel_bs
+        ctx.list_shape = lists.shape
         ctx.scale = scale
         return out
 
     @staticmethod
     def backward(ctx, grad_output: torch.Tensor):
         input, weight, mask, row_ptr, col_idx, col_ptr, row_idx = ctx.saved_tensors
-        lists = KeptLists(row_ptr, col_idx, col_ptr, row_idx, tuple(mask.shape))
+        lists = KeptLists(row_ptr, col_idx, col_ptr, row_idx, ctx.list_shape)
         ext = GEMM()
         if grad_output.dtype != input.dtype:
             grad_output = grad_output.to(input.dtype)
@@ -52,7 +56,7 @@ class BlockwiseDropoutMatmulHIP(torch.autograd.Function):
             # dB.T (K N) = A.T (K M sparse) * dC.T (N M), written straight into a row-major [N, K]
             grad_weight = ext.gemm_dsd_lists(input.t(), grad_output.t(), lists.transposed(),
                                              ctx.block_size, ctx.scale, transposed_out=True).t()
-        return grad_input, grad_weight, None, None, None
+        return grad_input, grad_weight, None, None, None, None
 
 
 def _prepare(input: torch.Tensor, weight: torch.Tensor):
@@ -83,9 +87,16 @@ def blockwise_dropout_matmul_mask(input: torch.Tensor, mask: torch.Tensor, block
         return BlockwiseDropoutMatmulHIP.apply(input, weight, mask, bs, float(p))
 
 
-def blockwise_dropout_matmul(input: torch.Tensor, weight: torch.Tensor, block_size, p: float) -> torch.Tensor:
-    """``(keep ⊙ input)/(1-p) @ weight.T`` with a fresh block mask (reference: …_cuda.py:56-59)."""
+def blockwise_dropout_matmul(input: torch.Tensor, weight: torch.Tensor, block_size, p: float,
+                             seed: int | None = None) -> torch.Tensor:
+    """``(keep ⊙ input)/(1-p) @ weight.T`` with a fresh block mask (reference: …_cuda.py:56-59).
+
+    The mask is drawn on the device inside the list-building launch; ``seed`` pins it (the same mask
+    comes back from ``GEMM().random_lists(mask_shape, p, seed)``), otherwise a seed is taken from
+    torch's default generator."""
     if not 0 <= p < 1:
         raise ValueError("Dropout probability must be in [0, 1)")
-    mask = blockwise_dropout_mask(input, block_size, p)
-    return blockwise_dropout_matmul_mask(input, mask, block_size, p, weight)
+    bs = _block_size(block_size)
+    input, weight = _prepare(input, weight)
+    with torch.autocast("cuda", enabled=False):
+        return BlockwiseDropoutMatmulHIP.apply(input, weight, None, bs, float(p), seed)

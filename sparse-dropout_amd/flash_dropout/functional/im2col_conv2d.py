@@ -35,30 +35,32 @@ def _to_matrix_grad(grad_output: torch.Tensor, dtype) -> torch.Tensor:
 
 class _Im2colConv2d(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, input, kernel, mask, block_size, p, padding, stride, dilation):
+    def forward(ctx, input, kernel, mask, block_size, p, padding, stride, dilation, seed=None):
         ext = GEMM()
         n, c, h, w = input.shape
         k, _, r, s = kernel.shape
         po, qo = ext.conv_out_hw(h, w, r, s, padding, stride, dilation)
         w2 = kernel.reshape(k, c * r * s)
-        lists = None
-        if mask is not None:
-            lists = ext.build_lists(mask)
-            cols = ext.im2col(input, (r, s), padding, stride, dilation, lists, block_size)
-            y2 = ext.gemm_dsd_lists(cols, w2, lists, block_size, 1.0 / (1.0 - p))
+        kernel_bs = block_size
+        if block_size:  # block dropout: mask given, or drawn in the list-building launch
+            mask, lists, kernel_bs = ext.kept_lists(n * po * qo, c * r * s, block_size, mask, p, seed,
+                                                    input.device)
+            cols = ext.im2col(input, (r, s), padding, stride, dilation, lists, kernel_bs)
+            y2 = ext.gemm_dsd_lists(cols, w2, lists, kernel_bs, 1.0 / (1.0 - p))
             ctx.save_for_backward(cols, w2, mask, lists.row_ptr, lists.col_idx, lists.col_ptr, lists.row_idx)
+            ctx.list_shape = lists.shape
         else:
             cols = ext.im2col(input, (r, s), padding, stride, dilation)
             y2 = ext.gemm(cols, w2)
             ctx.save_for_backward(cols, w2)
-        ctx.geom = (tuple(input.shape), tuple(kernel.shape), padding, stride, dilation, block_size, p,
+        ctx.geom = (tuple(input.shape), tuple(kernel.shape), padding, stride, dilation, block_size, kernel_bs, p,
                     input.is_contiguous(memory_format=torch.channels_last) and not input.is_contiguous())
         return y2.view(n, po * qo, k).permute(0, 2, 1).view(n, k, po, qo)
 
     @staticmethod
     def backward(ctx, grad_output):
         ext = GEMM()
-        x_shape, k_shape, padding, stride, dilation, block_size, p, ch_last = ctx.geom
+        x_shape, k_shape, padding, stride, dilation, block_size, kernel_bs, p, ch_last = ctx.geom
         r, s = k_shape[2], k_shape[3]
         saved = ctx.saved_tensors
         cols, w2 = saved[0], saved[1]
@@ -66,13 +68,13 @@ class _Im2colConv2d(torch.autograd.Function):
         dx = dk = None
         if len(saved) > 2:
             mask = saved[2]
-            lists = KeptLists(saved[3], saved[4], saved[5], saved[6], tuple(mask.shape))
+            lists = KeptLists(saved[3], saved[4], saved[5], saved[6], ctx.list_shape)
             scale = 1.0 / (1.0 - p)
             if ctx.needs_input_grad[0]:
-                dcols = ext.gemm_sdd_lists(dy2, w2.t(), lists, block_size, scale)
+                dcols = ext.gemm_sdd_lists(dy2, w2.t(), lists, kernel_bs, scale)
                 dx = ext.col2im(dcols, x_shape, (r, s), padding, stride, dilation, mask, block_size, ch_last)
             if ctx.needs_input_grad[1]:
-                dk = ext.gemm_dsd_lists(cols.t(), dy2.t(), lists.transposed(), block_size, scale,
+                dk = ext.gemm_dsd_lists(cols.t(), dy2.t(), lists.transposed(), kernel_bs, scale,
                                         transposed_out=True).t().reshape(k_shape)
         else:
             if ctx.needs_input_grad[0]:
@@ -80,7 +82,7 @@ class _Im2colConv2d(torch.autograd.Function):
                 dx = ext.col2im(dcols, x_shape, (r, s), padding, stride, dilation, channels_last=ch_last)
             if ctx.needs_input_grad[1]:
                 dk = ext.gemm(cols.t(), dy2.t(), transposed_out=True).t().reshape(k_shape)
-        return dx, dk, None, None, None, None, None, None
+        return dx, dk, None, None, None, None, None, None, None
 
 
 def _prepare(input: torch.Tensor, kernel: torch.Tensor):
@@ -123,12 +125,16 @@ def blockwise_dropout_conv2d_mask(input, mask, block_size, p: float, kernel, pad
 
 
 def blockwise_dropout_conv2d(input, kernel, block_size, p: float, padding=(0, 0), stride=(1, 1),
-                             dilation=(1, 1)) -> torch.Tensor:
-    """Block-dropout convolution with a fresh mask over the patch matrix."""
+                             dilation=(1, 1), seed: int | None = None) -> torch.Tensor:
+    """Block-dropout convolution with a fresh mask over the patch matrix, drawn on the device inside the
+    list-building launch (``seed`` pins it, as for the matmul)."""
+    if not 0 <= p < 1:
+        raise ValueError("Dropout probability must be in [0, 1)")
     bs = _block_size(block_size)
-    rows, ncols = conv_patch_matrix_shape(input.shape, kernel.shape, padding, stride, dilation)
-    mask = torch.rand(ceil(rows / bs), ceil(ncols / bs), device=input.device) < p
-    return blockwise_dropout_conv2d_mask(input, mask, bs, p, kernel, padding, stride, dilation)
+    input, kernel = _prepare(input, kernel)
+    with torch.autocast("cuda", enabled=False):
+        return _Im2colConv2d.apply(input, kernel, None, bs, float(p), _pair(padding), _pair(stride),
+                                   _pair(dilation), seed)
 
 
 def naive_blockwise_dropout_conv2d_mask(input, mask, block_size, p: float, kernel, padding=(0, 0),

@@ -6,7 +6,7 @@ no fallback: if the shared object is missing, loading raises.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_uint64, c_void_p
 from functools import lru_cache
 from pathlib import Path
 
@@ -21,6 +21,10 @@ SIGNATURES = {
     "sd_workspace_bytes": (c_int64, [c_int64, c_int64]),
     "sd_build_lists": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64,
                                c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sd_build_lists_split": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                     c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sd_random_lists": (c_int, [c_uint64, c_uint64, c_float, c_int64, c_int64, c_void_p, c_int64, c_int64,
+                                c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sd_increment_table": (c_int, [c_void_p, c_void_p, c_int64, c_int64,
                                    c_void_p, c_void_p, c_void_p, c_void_p]),
     "sd_splitk_workspace_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int64, c_int]),

@@ -173,7 +173,11 @@ class GEMM:
         C = self._out(A, B, out, transposed_out)
         if M == 0 or N == 0:
             return C
-        ws_bytes = (self.lib.sd_workspace_bytes(mb, cb) + 15) // 16 * 16
+        if bs > 64 and bs % 64 == 0:  # room for the 64-granular list: the library then splits the mask
+            ws_bytes = self.lib.sd_workspace_bytes(ceil(M / 64), ceil((K if mask_cols == "K" else N) / 64))
+        else:
+            ws_bytes = self.lib.sd_workspace_bytes(mb, cb)
+        ws_bytes = (ws_bytes + 15) // 16 * 16
         if mask_cols == "K":
             ws_bytes += self.lib.sd_splitk_workspace_bytes(M, N, K, bs, 1)
         ws = torch.empty((ws_bytes + 3) // 4, dtype=torch.int32, device=A.device)
@@ -194,24 +198,86 @@ class GEMM:
         return self._masked(self.lib.sd_gemm_sdd, "N", A, B, mask, block_size, scale, out, transposed_out)
 
     # ------------------------------------------------------------------ lists
-    def build_lists(self, mask: torch.Tensor) -> KeptLists:
-        """Mask -> CSR + CSC kept-block lists in one launch, no host synchronisation."""
+    @staticmethod
+    def _list_grid(mb, kb, split, grid):
+        split = int(split)
+        if split < 1:
+            raise ValueError(f"split must be >= 1, got {split}")
+        out_mb, out_kb = (mb * split, kb * split) if grid is None else (int(grid[0]), int(grid[1]))
+        if not ((mb - 1) * split < out_mb <= mb * split and (kb - 1) * split < out_kb <= kb * split):
+            raise ValueError(f"grid {(out_mb, out_kb)} does not match a {(mb, kb)} mask split by {split}")
+        return split, out_mb, out_kb
+
+    @staticmethod
+    def _list_buffers(out_mb, out_kb, dev):
+        # one allocation: row_ptr | col_ptr | col_idx | row_idx
+        buf = torch.empty(out_mb + 1 + out_kb + 1 + 2 * out_mb * out_kb, dtype=torch.int32, device=dev)
+        return torch.split(buf, [out_mb + 1, out_kb + 1, out_mb * out_kb, out_mb * out_kb])
+
+    def build_lists(self, mask: torch.Tensor, split: int = 1, grid=None) -> KeptLists:
+        """Mask -> CSR + CSC kept-block lists in one launch, no host synchronisation.
+
+        ``split`` > 1 lists the mask with every entry repeated split x split times, cropped to
+        ``grid`` = (rows, cols) of the finer block grid (default: uncropped): a mask drawn at block
+        size 64*split then drives the 64-block kernels."""
         if mask.dim() != 2 or mask.dtype != torch.bool or not mask.is_cuda:
             raise ValueError("mask must be a 2D bool tensor on the GPU")
         mb, kb = mask.shape
         if mb == 0 or kb == 0:
             raise ValueError("mask must be non-empty")
+        split, out_mb, out_kb = self._list_grid(mb, kb, split, grid)
         if mask.stride(0) != 1 and mask.stride(1) != 1:
             mask = mask.contiguous()
-        dev = mask.device
-        # one allocation: row_ptr | col_ptr | col_idx | row_idx
-        buf = torch.empty(mb + 1 + kb + 1 + 2 * mb * kb, dtype=torch.int32, device=dev)
-        row_ptr, col_ptr, col_idx, row_idx = torch.split(buf, [mb + 1, kb + 1, mb * kb, mb * kb])
+        row_ptr, col_ptr, col_idx, row_idx = self._list_buffers(out_mb, out_kb, mask.device)
+        with torch.cuda.device(mask.device):
+            self._call(self.lib.sd_build_lists_split, mask.data_ptr(), mb, kb, *_mask_strides(mask),
+                       split, out_mb, out_kb, row_ptr.data_ptr(), col_idx.data_ptr(), col_ptr.data_ptr(),
+                       row_idx.data_ptr(), self._stream(mask))
+        return KeptLists(row_ptr, col_idx, col_ptr, row_idx, (out_mb, out_kb))
+
+    def random_lists(self, shape, p: float, seed: int, offset: int = 0, device=None, split: int = 1,
+                     grid=None):
+        """Draws a Bernoulli(p) block mask of ``shape`` on the device (True = dropped) and lists it in
+        the same launch: (mask, lists).  The mask is a pure function of (seed, offset, shape[1]) —
+        Philox4x32-10, one 32-bit word per entry — not torch's generator stream."""
+        mb, kb = int(shape[0]), int(shape[1])
+        if mb <= 0 or kb <= 0:
+            raise ValueError("mask must be non-empty")
+        if not 0.0 <= p < 1.0:
+            raise ValueError(f"p must be in [0, 1), got {p}")
+        split, out_mb, out_kb = self._list_grid(mb, kb, split, grid)
+        dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+        mask = torch.empty((mb, kb), dtype=torch.bool, device=dev)
+        row_ptr, col_ptr, col_idx, row_idx = self._list_buffers(out_mb, out_kb, dev)
         with torch.cuda.device(dev):
-            self._call(self.lib.sd_build_lists, mask.data_ptr(), mb, kb, *_mask_strides(mask),
-                       row_ptr.data_ptr(), col_idx.data_ptr(), col_ptr.data_ptr(), row_idx.data_ptr(),
-                       self._stream(mask))
-        return KeptLists(row_ptr, col_idx, col_ptr, row_idx, (mb, kb))
+            self._call(self.lib.sd_random_lists, int(seed) & (2 ** 64 - 1), int(offset) & (2 ** 64 - 1),
+                       float(p), mb, kb, mask.data_ptr(), split, out_mb, out_kb, row_ptr.data_ptr(),
+                       col_idx.data_ptr(), col_ptr.data_ptr(), row_idx.data_ptr(), self._stream(mask))
+        return mask, KeptLists(row_ptr, col_idx, col_ptr, row_idx, (out_mb, out_kb))
+
+    def kept_lists(self, rows: int, cols: int, block_size, mask: torch.Tensor | None = None,
+                   p: float = 0.0, seed: int | None = None, device=None):
+        """Lists for a [rows, cols] matrix masked in block_size tiles -> (mask, lists, kernel block size).
+
+        The mask is the given one, or drawn on the device (Bernoulli(p), ``seed`` or a fresh seed from
+        torch's default CPU generator, so ``torch.manual_seed`` makes runs repeatable).  A block size
+        that is a larger multiple of 64 is listed at 64 granularity, which is what the fast kernels
+        take: pass the returned block size, not the logical one, to the ``*_lists`` calls."""
+        bs = _block_size(block_size)
+        shape = (ceil(rows / bs), ceil(cols / bs))
+        split, grid, kernel_bs = 1, None, bs
+        if bs > 64 and bs % 64 == 0:
+            split, grid, kernel_bs = bs // 64, (ceil(rows / 64), ceil(cols / 64)), 64
+        if mask is None:
+            if seed is None:
+                seed = int(torch.empty((), dtype=torch.int64).random_().item())
+            mask, lists = self.random_lists(shape, p, seed, 0, device, split, grid)
+        else:
+            if tuple(mask.shape) != shape:
+                raise ValueError(f"mask shape {tuple(mask.shape)} != {shape} for a [{rows}, {cols}] matrix "
+                                 f"in blocks of {bs}")
+            lists = self.build_lists(mask, split, grid)
+        return mask, lists, kernel_bs
 
     def increment_table(self, lists: KeptLists, block_k: int):
         """(table, row_indices, row_widths) of the reference's ``mask_to_increment_table``

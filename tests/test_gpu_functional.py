@@ -96,9 +96,10 @@ def test_cfg3_mlp_on_28x28_images_through_layers():
     dy = torch.randn(4096, 10).half()
     mods = [l.cuda().half() for l in layers]
 
-    # fixed generator state so that the masks the layers draw can be re-drawn for the oracle
-    torch.cuda.manual_seed(123)
-    state = torch.cuda.get_rng_state()
+    # fixed generator state so that the masks the layers draw can be re-drawn for the oracle: every
+    # call takes one 64-bit seed from torch's default CPU generator and draws its mask from that
+    torch.manual_seed(123)
+    state = torch.get_rng_state()
     ins, outs = [], []
     h = x.cuda().requires_grad_()
     for i, l in enumerate(mods):
@@ -111,8 +112,9 @@ def test_cfg3_mlp_on_28x28_images_through_layers():
             h = torch.relu(h)
     h.backward(dy.cuda())
 
-    torch.cuda.set_rng_state(state)
-    masks = [(torch.rand(64, -(-dims[i] // 64), device="cuda") < 0.5).cpu().numpy() for i in range(3)]
+    torch.set_rng_state(state)
+    seeds = [int(torch.empty((), dtype=torch.int64).random_().item()) for _ in range(3)]
+    masks = [O.random_mask((64, -(-dims[i] // 64)), 0.5, seeds[i]) for i in range(3)]
     for i, l in enumerate(mods):
         a, g, w = to_np(ins[i]), to_np(outs[i].grad), to_np(l.weight)
         assert rel_fro(outs[i], O.dsd_forward(a, w, masks[i], 64, 0.5, np.float32)) <= REL_FRO_TOL, f"Y{i}"
@@ -130,12 +132,12 @@ def test_layer_eval_and_3d_inputs_and_bf16():
     layer.eval()
     assert torch.equal(layer(x), torch.nn.functional.linear(x, layer.weight))
     layer.train()
-    torch.cuda.manual_seed(9)
-    state = torch.cuda.get_rng_state()
+    torch.manual_seed(9)
+    state = torch.get_rng_state()
     y = layer(x)
     assert y.shape == (8, 256, 256) and y.dtype == torch.bfloat16
-    torch.cuda.set_rng_state(state)
-    mask = (torch.rand(32, 6, device="cuda") < 0.3).cpu().numpy()
+    torch.set_rng_state(state)  # the layer took one 64-bit seed from the default CPU generator
+    mask = O.random_mask((32, 6), 0.3, int(torch.empty((), dtype=torch.int64).random_().item()))
     ref = O.dsd_forward(to_np(x.reshape(-1, 384)), to_np(layer.weight), mask, 64, 0.3, np.float32)
     assert rel_fro(y.reshape(-1, 256), ref) <= REL_FRO_TOL
 
@@ -177,7 +179,7 @@ def test_public_names_and_p_range():
     # statistical sanity of the fresh mask: about p of the blocks are dropped
     big = torch.ones(4096, 4096, device="cuda", dtype=torch.float16)
     eye = torch.eye(4096, device="cuda", dtype=torch.float16)
-    torch.cuda.manual_seed(0)
+    torch.manual_seed(0)
     out = F.cuda_blockwise_dropout_matmul(big, eye, 64, 0.25)
     frac_dropped = (out == 0).float().mean().item()
     assert abs(frac_dropped - 0.25) < 0.03

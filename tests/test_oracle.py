@@ -244,3 +244,52 @@ def test_conv_blockdrop_vs_autograd_composition():
     np.testing.assert_allclose(y, y_ref.detach().numpy(), rtol=1e-12, atol=1e-12)
     np.testing.assert_allclose(dx, x.grad.numpy(), rtol=1e-12, atol=1e-12)
     np.testing.assert_allclose(dk, k.grad.numpy(), rtol=1e-12, atol=1e-12)
+
+
+# ---- on-device mask draw and block splitting ---------------------------------------------------
+# Known answers of Philox4x32-10 from the Random123 distribution's kat_vectors (counter, key, output).
+PHILOX_KAT = [
+    ([0x00000000] * 4, [0x00000000] * 2, [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]),
+    ([0xFFFFFFFF] * 4, [0xFFFFFFFF] * 2, [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]),
+    ([0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344], [0xA4093822, 0x299F31D0],
+     [0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1]),
+]
+
+
+@pytest.mark.parametrize("counter,key,want", PHILOX_KAT)
+def test_philox_known_answers(counter, key, want):
+    assert O.philox4x32_10(counter, key).tolist() == want
+
+
+def test_philox_is_vectorised_consistently():
+    ctr = np.array([k[0] for k in PHILOX_KAT], dtype=np.uint64)
+    one_key = O.philox4x32_10(ctr, PHILOX_KAT[2][1])
+    assert one_key[2].tolist() == PHILOX_KAT[2][2]
+    assert one_key[0].tolist() == O.philox4x32_10(PHILOX_KAT[0][0], PHILOX_KAT[2][1]).tolist()
+
+
+def test_random_mask_definition():
+    shape = (37, 53)
+    # entry e uses word e % 4 of block e // 4: recompute a few entries by hand
+    m = O.random_mask(shape, 0.4, seed=(5 << 32) | 9, offset=(1 << 32) | 2)
+    for e in (0, 1, 5, 702, 37 * 53 - 1):
+        w = O.philox4x32_10([e // 4, 0, 2, 1], [9, 5])[e % 4]
+        assert m.reshape(-1)[e] == (np.float32(w >> 8) * np.float32(2.0 ** -24) < np.float32(0.4))
+    assert m.dtype == bool and m.shape == shape
+    assert not O.random_mask(shape, 0.0, 1).any()                 # p = 0 keeps everything
+    assert O.random_mask(shape, 1.0 - 2.0 ** -24, 1).mean() > 0.999  # True means dropped
+    big = O.random_mask((512, 512), 0.3, seed=11)
+    assert abs(big.mean() - 0.3) < 4 * (0.3 * 0.7 / big.size) ** 0.5
+    assert (O.random_mask((512, 512), 0.3, seed=12) != big).any()
+    assert (O.random_mask((512, 512), 0.3, seed=11, offset=1) != big).any()
+    # rows are independent: no visible correlation between neighbouring entries
+    assert abs(np.corrcoef(big[:, :-1].ravel(), big[:, 1:].ravel())[0, 1]) < 0.02
+
+
+@pytest.mark.parametrize("m,k,bs,split", [(256, 384, 128, 2), (200, 130, 128, 2), (70, 500, 192, 3), (64, 64, 64, 1)])
+def test_split_mask_expands_to_the_same_elements(m, k, bs, split):
+    rng = np.random.default_rng(0)
+    mask = rng.random(O.mask_shape(m, k, bs)) < 0.5
+    fine = O.split_mask(mask, split, O.mask_shape(m, k, bs // split))
+    assert fine.shape == O.mask_shape(m, k, bs // split)
+    assert np.array_equal(O.expand_keep(mask, bs, m, k), O.expand_keep(fine, bs // split, m, k))
