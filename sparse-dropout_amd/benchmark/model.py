@@ -1,0 +1,103 @@
+"""Whole-model forward + backward time as the drop rate varies (reference: benchmark/model.py:119-229).
+
+    python -m benchmark.model --model mlp vit-ffn --p 0 0.1 0.3 0.5 0.7
+
+Models are built from ``DropoutMM`` the way the reference's evaluation models are:
+  mlp      flattened 32x32 images -> [hidden]*layers -> 10 classes padded to 128, ReLU between, dropout on
+           the input of every linear but the first (eval/mlp/model.py: BasicNet); batch 1024, hidden 1024
+  vit-ffn  one transformer feed-forward block on 64x256 tokens: 384 -> 1536 -> GELU -> 384, dropout on the
+           inputs of both linears
+Each is timed with variant "none" (dense), "vanilla" (element dropout + dense) and "blockwise[hip]"."""
+from __future__ import annotations
+
+import argparse
+import statistics
+import time
+
+import torch
+from torch import nn
+
+from flash_dropout.layers import DropoutMM
+
+from .utils import FLUSH_BYTES
+
+
+class Mlp(nn.Module):
+    def __init__(self, variant, p, block_size, in_dim=1024, hidden=1024, layers=2, classes=128):
+        super().__init__()
+        dims = [in_dim] + [hidden] * layers + [classes]
+        self.linears = nn.ModuleList(
+            DropoutMM(dims[i], dims[i + 1], p=p if i else 0.0, variant=variant if i else "none",
+                      block_size=block_size) for i in range(len(dims) - 1))
+
+    def forward(self, x):
+        x = x.flatten(1)
+        for i, lin in enumerate(self.linears):
+            x = lin(x if i == 0 else torch.relu(x))
+        return x
+
+
+class VitFfn(nn.Module):
+    def __init__(self, variant, p, block_size, dim=384, hidden=1536):
+        super().__init__()
+        self.up = DropoutMM(dim, hidden, p=p, variant=variant, block_size=block_size)
+        self.down = DropoutMM(hidden, dim, p=p, variant=variant, block_size=block_size)
+
+    def forward(self, x):
+        return self.down(nn.functional.gelu(self.up(x)))
+
+
+MODELS = {
+    "mlp": (Mlp, lambda: torch.rand(1024, 1, 32, 32)),
+    "vit-ffn": (VitFfn, lambda: torch.randn(64, 256, 384)),
+}
+
+
+def time_model(model: nn.Module, x: torch.Tensor, warmup: float, rep: float) -> list[float]:
+    """fwd+bwd milliseconds per repetition, cache flushed before each (benchmark/model.py:119-142)."""
+    cache = torch.empty(FLUSH_BYTES, dtype=torch.int8, device="cuda")
+
+    def f():
+        model(x).float().square().mean().backward()
+
+    for _ in range(10):
+        f()
+    t0 = time.time()
+    while time.time() - t0 < warmup:
+        f()
+        torch.cuda.synchronize()
+    timings, t0 = [], time.time()
+    while time.time() - t0 < rep or len(timings) < 5:
+        cache.zero_()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        f()
+        b.record()
+        torch.cuda.synchronize()
+        timings.append(a.elapsed_time(b))
+    return timings
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--model", nargs="+", choices=sorted(MODELS), default=sorted(MODELS))
+    ap.add_argument("--p", type=float, nargs="+", default=[0.0, 0.1, 0.3, 0.5, 0.7])
+    ap.add_argument("--block-size", type=int, default=64)
+    ap.add_argument("--rep", type=float, default=0.3, help="seconds of timed repetitions per point")
+    args = ap.parse_args()
+    torch.manual_seed(0)
+    for name in args.model:
+        cls, make_x = MODELS[name]
+        x = make_x().cuda().half()
+        print(f"=== {name}  input {tuple(x.shape)}  block_size {args.block_size}")
+        for variant, ps in (("none", [0.0]), ("vanilla", [0.5]), ("blockwise[hip]", args.p)):
+            for p in ps:
+                model = cls(variant, p, args.block_size).cuda().half().train()
+                ts = time_model(model, x, warmup=0.2, rep=args.rep)
+                sem = statistics.stdev(ts) / len(ts) ** 0.5 if len(ts) > 1 else 0.0
+                print(f"{variant:<16} p={p:<4} median {statistics.median(ts):8.4f} ms  "
+                      f"mean {statistics.mean(ts):8.4f} +- {1.96 * sem:.4f}  n={len(ts)}")
+
+
+if __name__ == "__main__":
+    main()

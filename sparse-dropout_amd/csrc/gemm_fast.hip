@@ -357,11 +357,15 @@ __global__ __launch_bounds__(THREADS) void sdd_kernel(GemmArgs g, int tiles_m, i
   if (tid == 0) *kept_p = 0;
   __syncthreads();
   if (wave < R && rb0 + wave < Mb) {
-    const int beg = g.row_ptr[rb0 + wave], end = g.row_ptr[rb0 + wave + 1];
     uint32_t bits = 0;
-    for (int i = beg + lane; i < end; i += 64) {
-      const int c = g.col_idx[i] - cb0;
-      if (c >= 0 && c < R) bits |= 1u << (wave * 4 + c);
+    if (g.row_ptr) {
+      const int beg = g.row_ptr[rb0 + wave], end = g.row_ptr[rb0 + wave + 1];
+      for (int i = beg + lane; i < end; i += 64) {
+        const int c = g.col_idx[i] - cb0;
+        if (c >= 0 && c < R) bits |= 1u << (wave * 4 + c);
+      }
+    } else if (lane < R && cb0 + lane < Cb) {  // no list: a dense product in this operand layout
+      bits = 1u << (wave * 4 + lane);
     }
     if (bits) atomicOr(kept_p, bits);
   }
@@ -542,7 +546,7 @@ int launch_sdd(const GemmArgs& g, hipStream_t stream) {
 }
 
 int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
-  if (g.bs != BS) return SD_ERR_UNSUPPORTED;
+  if (g.row_ptr && g.bs != BS) return SD_ERR_UNSUPPORTED;
   const bool layout_ok = g.a.sc == 1 && g.b.sr == 1 && g.b.sc != 1 && g.c_sc == 1;
   const bool shape_ok = g.M > 0 && g.M % BS == 0 && g.N > 0 && g.N % BS == 0 && g.K > 0 && g.K % BS == 0;
   const bool align_ok = aligned16(g.a.ptr) && aligned16(g.b.ptr) && aligned16(g.c) && g.a.sr % 8 == 0 &&
@@ -556,6 +560,9 @@ int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
 
 int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   if (mode == kSdd) return try_sdd(g, dtype, stream);
+  // a dense product of a row-major A with a reduction-strided B (dX = dY.W without dropout) is the SDD
+  // kernel with every tile kept
+  if (mode == kDense && g.a.sc == 1 && g.b.sr == 1 && g.b.sc != 1 && g.c_sc == 1) return try_sdd(g, dtype, stream);
   if (mode == kDsd && g.bs != BS) return SD_ERR_UNSUPPORTED;
   // everything tile-aligned and 16-byte aligned; the three matrices agree on which index is contiguous
   const bool nt = g.a.sc == 1 && g.b.sc == 1 && g.c_sc == 1;  // reduction-contiguous, C row-major

@@ -1,10 +1,13 @@
 // Block mask -> compacted kept-block lists (CSR over row blocks, CSC over column blocks).
 //
-// Integer/byte work, bound by launch latency and a few KB of HBM traffic: one wave owns one row
-// (or column) of the mask, 64 mask bytes per step; __ballot + popcount give each kept block its
-// slot, so the lists come out in ascending order — the order of nonzero(~mask)
+// Integer/byte work, bound by launch latency and a few KB of HBM traffic.  The lists come out in
+// ascending order — the order of nonzero(~mask)
 // (flash_dropout/functional/blockwise_dropout_matmul_triton.py:48) — without atomics and without
-// a device->host synchronisation.
+// a device->host synchronisation.  Masks of up to 2^18 entries are listed by one launch (a flat
+// stream compaction, see build_lists_flat); larger ones by count / scan / fill launches in which one
+// wave owns one row (or column) of the mask, 64 entries per step, __ballot + popcount giving each kept
+// block its slot.  The mask is either stored (bool bytes, any of the two majornesses) or drawn on the
+// fly from a counter-based generator, and may be listed at a finer granularity than it was drawn.
 #include "common.h"
 
 namespace sd {
@@ -128,33 +131,89 @@ __device__ inline void write_mask(const MaskSrc& src, int64_t mb, uint8_t* out, 
     out[e] = src.dropped_entry((int32_t)(e / src.kb), (int32_t)(e % src.kb)) ? 1 : 0;
 }
 
-// One thread block does count -> scan -> fill for one list.  Block 0 takes job0, block 1 job1, block 2
-// (launched only for a drawn mask) stores the mask.  All traffic of a job stays inside its block, so
-// __syncthreads() (which also orders the block's global writes for the block's own later reads) is
-// the only synchronisation needed.
-template <int THREADS>
-__global__ __launch_bounds__(THREADS) void build_lists_fused(ListJob job0, ListJob job1,
-                                                             uint8_t* mask_out, int64_t mask_rows) {
-  __shared__ int32_t lds[THREADS];
-  if (blockIdx.x == 2) {
-    write_mask(job0.src, mask_rows, mask_out, threadIdx.x, THREADS);
+// ---- single-launch builder for masks of up to 2^18 entries ------------------------------------------
+// A list is a stream compaction of the mask read in line-major order ("flat" index f = line * len + e):
+// idx gets e of every kept entry, ptr[line] the number of kept entries before the line.  A block owns
+// kFlatChunk consecutive flat entries.  Blocks do not talk to each other: each first counts the kept
+// entries in front of its chunk itself (one sweep over at most 2^18 mask bytes, or draws), which replaces
+// the grid-wide scan and keeps the whole build in one launch with every load independent of the others.
+constexpr int kFlatThreads = 1024;
+constexpr int kFlatPer = 4;  // consecutive entries per thread
+constexpr int kFlatChunk = kFlatThreads * kFlatPer;
+
+// Exclusive prefix of v over the block (thread order) and the block total; lds holds one int per wave.
+__device__ inline int block_exclusive_scan(int v, int32_t* lds, int& total) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  int incl = v;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const int up = __shfl_up(incl, off, kWave);
+    if (lane >= off) incl += up;
+  }
+  __syncthreads();  // lds may still be read from a previous call
+  if (lane == kWave - 1) lds[wave] = incl;
+  __syncthreads();
+  int before = 0, sum = 0;
+  for (int w = 0; w < kFlatThreads / kWave; ++w) {
+    const int t = lds[w];
+    if (w < wave) before += t;
+    sum += t;
+  }
+  total = sum;
+  return before + incl - v;
+}
+
+__global__ __launch_bounds__(kFlatThreads) void build_lists_flat(ListJob job0, ListJob job1, int blocks0,
+                                                                int blocks1, uint8_t* mask_out,
+                                                                int64_t mask_rows) {
+  __shared__ int32_t lds[kFlatThreads / kWave];
+  const int tid = threadIdx.x;
+  int b = blockIdx.x;
+  if (b >= blocks0 + blocks1) {  // launched only for a drawn mask: store it for the caller
+    const int nb = gridDim.x - blocks0 - blocks1;
+    write_mask(job0.src, mask_rows, mask_out, (int64_t)(b - blocks0 - blocks1) * kFlatThreads + tid,
+               (int64_t)nb * kFlatThreads);
     return;
   }
-  const ListJob job = (blockIdx.x == 0) ? job0 : job1;
-  if (job.ptr == nullptr) return;
-  const int lane = threadIdx.x % kWave;
-  const int wave = threadIdx.x / kWave;
-  constexpr int kWaves = THREADS / kWave;
-  for (int64_t line = wave; line < job.nlines; line += kWaves) {
-    int c = wave_count_kept(job, line, lane);
-    if (lane == 0) job.ptr[1 + line] = c;
+  const bool second = b >= blocks0;
+  const ListJob job = second ? job1 : job0;
+  if (second) b -= blocks0;
+  const int len = (int)job.len;
+  const int total_entries = (int)(job.nlines * job.len);
+  const int f0 = b * kFlatChunk;
+
+  // kept entries in front of this block's chunk
+  int cnt = 0;
+  for (int f = tid; f < f0; f += kFlatThreads) {
+    const int line = f / len;
+    cnt += job.kept(line, f - line * len) ? 1 : 0;
   }
-  __syncthreads();
-  block_scan_inplace<THREADS>(job.ptr, job.nlines, lds);
-  __syncthreads();
-  for (int64_t line = wave; line < job.nlines; line += kWaves) {
-    wave_fill_kept(job, line, lane, job.idx + job.ptr[line]);
+  int base;
+  block_exclusive_scan(cnt, lds, base);
+
+  // this thread's entries
+  const int mine = f0 + tid * kFlatPer;
+  int line = mine / len, e = mine - line * len;
+  uint32_t bits = 0;
+  {
+    int l = line, x = e;
+#pragma unroll
+    for (int v = 0; v < kFlatPer; ++v) {
+      if (mine + v < total_entries && job.kept(l, x)) bits |= 1u << v;
+      if (++x == len) { x = 0; ++l; }
+    }
   }
+  int chunk_total;
+  int pos = base + block_exclusive_scan(__popc(bits), lds, chunk_total);
+#pragma unroll
+  for (int v = 0; v < kFlatPer; ++v) {
+    if (mine + v < total_entries) {
+      if (e == 0) job.ptr[line] = pos;
+      if (bits & (1u << v)) job.idx[pos++] = e;
+    }
+    if (++e == len) { e = 0; ++line; }
+  }
+  if (tid == 0 && f0 + kFlatChunk >= total_entries) job.ptr[job.nlines] = base + chunk_total;
 }
 
 __global__ __launch_bounds__(256) void mask_store_kernel(MaskSrc src, int64_t mb, uint8_t* out) {
@@ -221,9 +280,12 @@ static int launch_lists(const MaskSrc& src, int64_t mb, int64_t kb, int32_t* row
   ListJob csr{src, 0, mb, kb, row_ptr, col_idx};
   ListJob csc{src, 1, kb, mb, col_ptr, row_idx};
   if (mb * kb <= (1 << 18)) {
-    hipLaunchKernelGGL(build_lists_fused<1024>, dim3(mask_out ? 3 : 2), dim3(1024), 0, stream, csr, csc,
-                       mask_out, mask_rows);
-    return check_launch("build_lists_fused");
+    const int per_list = (int)ceil_div(mb * kb, kFlatChunk);
+    const int blocks0 = row_ptr ? per_list : 0, blocks1 = col_ptr ? per_list : 0;
+    const int blocks_mask = mask_out ? (int)ceil_div(mask_rows * src.kb, kFlatChunk) : 0;
+    hipLaunchKernelGGL(build_lists_flat, dim3(blocks0 + blocks1 + blocks_mask), dim3(kFlatThreads), 0, stream,
+                       csr, csc, blocks0, blocks1, mask_out, mask_rows);
+    return check_launch("build_lists_flat");
   }
   if (mask_out) {
     const int64_t total = mask_rows * src.kb;

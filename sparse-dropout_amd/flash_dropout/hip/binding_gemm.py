@@ -11,6 +11,7 @@ libsparsedrop.so with raw pointers.  Tensors must live on the GPU; there is no C
 """
 from __future__ import annotations
 
+import contextlib
 from dataclasses import dataclass
 from functools import cache
 from math import ceil
@@ -50,6 +51,14 @@ class KeptLists:
         """Lists of mask.T: CSR and CSC swap roles."""
         return KeptLists(self.col_ptr, self.row_idx, self.row_ptr, self.col_idx,
                          (self.shape[1], self.shape[0]))
+
+
+_NO_GUARD = contextlib.nullcontext()
+
+
+def _guard(dev: torch.device):
+    """Makes ``dev`` the current device for a launch; free when it already is."""
+    return _NO_GUARD if dev.index == torch.cuda.current_device() else torch.cuda.device(dev)
 
 
 def _block_size(block_size) -> int:
@@ -151,7 +160,7 @@ class GEMM:
         if A.shape[0] == 0 or B.shape[0] == 0:
             return C
         ws, ws_ptr, ws_bytes = self._splitk_scratch(A, B, 0, 0)
-        with torch.cuda.device(A.device):
+        with _guard(A.device):
             self._call(self.lib.sd_gemm, *_mat(A), *_mat(B), *_mat(C), A.shape[0], B.shape[0],
                        A.shape[1], _DTYPES[A.dtype], ws_ptr, ws_bytes, self._stream(A))
         return C
@@ -181,7 +190,7 @@ class GEMM:
         if mask_cols == "K":
             ws_bytes += self.lib.sd_splitk_workspace_bytes(M, N, K, bs, 1)
         ws = torch.empty((ws_bytes + 3) // 4, dtype=torch.int32, device=A.device)
-        with torch.cuda.device(A.device):
+        with _guard(A.device):
             self._call(fn, *_mat(A), *_mat(B), *_mat(C), mask.data_ptr(), *_mask_strides(mask),
                        M, N, K, bs, float(scale), _DTYPES[A.dtype], ws.data_ptr(), ws_bytes,
                        self._stream(A))
@@ -229,7 +238,7 @@ class GEMM:
         if mask.stride(0) != 1 and mask.stride(1) != 1:
             mask = mask.contiguous()
         row_ptr, col_ptr, col_idx, row_idx = self._list_buffers(out_mb, out_kb, mask.device)
-        with torch.cuda.device(mask.device):
+        with _guard(mask.device):
             self._call(self.lib.sd_build_lists_split, mask.data_ptr(), mb, kb, *_mask_strides(mask),
                        split, out_mb, out_kb, row_ptr.data_ptr(), col_idx.data_ptr(), col_ptr.data_ptr(),
                        row_idx.data_ptr(), self._stream(mask))
@@ -246,10 +255,12 @@ class GEMM:
         if not 0.0 <= p < 1.0:
             raise ValueError(f"p must be in [0, 1), got {p}")
         split, out_mb, out_kb = self._list_grid(mb, kb, split, grid)
-        dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+        dev = torch.device("cuda") if device is None else torch.device(device)
+        if dev.index is None:
+            dev = torch.device("cuda", torch.cuda.current_device())
         mask = torch.empty((mb, kb), dtype=torch.bool, device=dev)
         row_ptr, col_ptr, col_idx, row_idx = self._list_buffers(out_mb, out_kb, dev)
-        with torch.cuda.device(dev):
+        with _guard(dev):
             self._call(self.lib.sd_random_lists, int(seed) & (2 ** 64 - 1), int(offset) & (2 ** 64 - 1),
                        float(p), mb, kb, mask.data_ptr(), split, out_mb, out_kb, row_ptr.data_ptr(),
                        col_idx.data_ptr(), col_ptr.data_ptr(), row_idx.data_ptr(), self._stream(mask))
@@ -288,7 +299,7 @@ class GEMM:
         table = torch.empty(lists.col_idx.numel(), dtype=torch.int64, device=dev)
         row_indices = torch.empty(mb, dtype=torch.int64, device=dev)
         row_widths = torch.empty(mb, dtype=torch.int64, device=dev)
-        with torch.cuda.device(dev):
+        with _guard(dev):
             self._call(self.lib.sd_increment_table, lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(),
                        mb, int(block_k), table.data_ptr(), row_indices.data_ptr(),
                        row_widths.data_ptr(), self._stream(table))
@@ -308,7 +319,7 @@ class GEMM:
         if mask_cols == "K":  # DSD may split a long reduction
             ws, ws_ptr, ws_bytes = self._splitk_scratch(A, B, bs, 1)
             extra = (ws_ptr, ws_bytes)
-        with torch.cuda.device(A.device):
+        with _guard(A.device):
             self._call(fn, *_mat(A), *_mat(B), *_mat(C), lists.row_ptr.data_ptr(),
                        lists.col_idx.data_ptr(), M, N, K, bs, float(scale), _DTYPES[A.dtype],
                        *extra, self._stream(A))
@@ -357,7 +368,7 @@ class GEMM:
             if tuple(lists.shape) != want:
                 raise ValueError(f"lists are for a {lists.shape} mask, patch matrix needs {want}")
             rp, ci = lists.row_ptr.data_ptr(), lists.col_idx.data_ptr()
-        with torch.cuda.device(x.device):
+        with _guard(x.device):
             self._call(self.lib.sd_im2col, x.data_ptr(), *x.stride(), cols.data_ptr(), cols.stride(0),
                        n, c, h, w, r, s, *padding, *stride, *dilation, rp, ci, bs, _DTYPES[x.dtype],
                        self._stream(x))
@@ -383,7 +394,7 @@ class GEMM:
             mask = _check_mask(mask, (ceil(n * p * q / bs), ceil(c * r * s / bs)), cols)
             mp = mask.data_ptr()
             msr, msc = _mask_strides(mask)
-        with torch.cuda.device(cols.device):
+        with _guard(cols.device):
             self._call(self.lib.sd_col2im, cols.data_ptr(), cols.stride(0), dx.data_ptr(), *dx.stride(),
                        n, c, h, w, r, s, *padding, *stride, *dilation, mp, msr, msc, bs,
                        _DTYPES[cols.dtype], self._stream(cols))
