@@ -166,7 +166,11 @@ int sd_increment_table(const int32_t* row_ptr, const int32_t* col_idx, int64_t m
 
 int64_t sd_splitk_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t block_size, int sparse) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
-  const int splits = generic_splits(M, N, K, sparse ? block_size : 0, sparse ? kDsd : kDense);
+  int splits = generic_splits(M, N, K, sparse ? block_size : 0, sparse ? kDsd : kDense);
+  if (!sparse || block_size == 64) {
+    const int fs = fast_splits(M, N, K);
+    if (fs > splits) splits = fs;
+  }
   return splits > 1 ? (int64_t)splits * M * N * 4 : 0;
 }
 

@@ -115,6 +115,10 @@ int launch_generic(const GemmArgs& g, int mode, int dtype, hipStream_t stream);
 // number of reduction splits the generic kernel would like for this problem (1 = none); it needs
 // splits * M * N * 4 bytes of workspace for that
 int generic_splits(int64_t M, int64_t N, int64_t K, int64_t bs, int mode);
+// reduction splits the fast DSD kernel would like (1 = none); same scratch rule
+int fast_splits(int64_t M, int64_t N, int64_t K);
+// C = scale * sum of `splits` fp32 partials [splits][M*N] laid out in C's element order
+int launch_splitk_reduce(const GemmArgs& g, int splits, bool trans_out, int dtype, hipStream_t stream);
 // returns SD_ERR_UNSUPPORTED (without setting an error message) when the fast path does not apply
 int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream);
 

@@ -98,7 +98,7 @@ __device__ inline u32x2 lds_read_tr(const char* p) {
 // In both cases "Mb" counts the row blocks of A (of X^T for dW) and "Kb" the reduction blocks.
 template <typename T, bool TRANS>
 __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, int tiles_n,
-                                                      int Mb, int Kb) {
+                                                      int Mb, int Kb_all) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   uint16_t* step_kb = reinterpret_cast<uint16_t*>(smem + SMEM_STEPS);
   uint8_t* step_fl = reinterpret_cast<uint8_t*>(smem + SMEM_FLAGS);
@@ -114,6 +114,11 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
   const int rh = wave / 4;  // row-block pair
   const int rb0 = tm * R;   // first row block
   const int64_t n0 = (int64_t)tn * BN;
+  const int nvalid = (int)((g.N - n0) < BN ? (g.N - n0) : BN);  // columns of this tile inside C (multiple of 64)
+  // split reduction: blockIdx.y takes the reduction blocks [kb_lo, kb_lo + Kb) and leaves an fp32 partial
+  const int nsplit = gridDim.y, split = blockIdx.y;
+  const int kb_lo = (int)((int64_t)Kb_all * split / nsplit);
+  const int Kb = (int)((int64_t)Kb_all * (split + 1) / nsplit) - kb_lo;
 
   // ---- union of the kept lists of the 4 row blocks: (K block, 4-bit keep flags) per step -------
   for (int i = tid; i < Kb; i += THREADS) scratch[i] = 0;
@@ -122,7 +127,10 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
     for (int r = 0; r < R; ++r) {
       if (rb0 + r >= Mb) break;
       const int beg = g.row_ptr[rb0 + r], end = g.row_ptr[rb0 + r + 1];
-      for (int i = beg + tid; i < end; i += THREADS) atomicOr(&scratch[g.col_idx[i]], 1u << r);
+      for (int i = beg + tid; i < end; i += THREADS) {
+        const int k = g.col_idx[i] - kb_lo;
+        if (k >= 0 && k < Kb) atomicOr(&scratch[k], 1u << r);
+      }
     }
   } else {
     const uint32_t all = (rb0 + R <= Mb) ? 0xfu : ((1u << (Mb - rb0)) - 1u);
@@ -138,7 +146,7 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
       const uint64_t bal = __ballot(f != 0);
       if (f) {
         const int pos = base + __popcll(bal & lt);
-        step_kb[pos] = (uint16_t)k;
+        step_kb[pos] = (uint16_t)(kb_lo + k);
         step_fl[pos] = (uint8_t)f;
       }
       base += __popcll(bal);
@@ -182,6 +190,7 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
   // global -> LDS: every wave-wide load fills 1 KB of LDS in lane order.  Per-lane byte offsets are
   // fixed for the whole kernel; per step only a wave-uniform base moves.
   uint32_t b_lane[4], a_lane;
+  bool b_valid[4];  // the lane's 16 bytes of the W tile lie inside the matrix (a tile may overhang N)
   const char* a_tile0;  // first X tile of the patch at reduction block 0
   const char* b_tile0;  // W tile at reduction block 0
   int64_t red_stride;   // bytes between consecutive reduction blocks
@@ -193,6 +202,7 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
     for (int jj = 0; jj < 4; ++jj) {
       const int row = (wave * 4 + jj) * 8 + ld_row;
       b_lane[jj] = (uint32_t)(row * g.b.sr + (ld_pch ^ ((row >> 1) & 7)) * 8) * 2u;
+      b_valid[jj] = row < nvalid;
     }
     const int row = wave * 8 + ld_row;
     a_lane = (uint32_t)(row * g.a.sr + (ld_pch ^ ((row >> 1) & 7)) * 8) * 2u;
@@ -205,7 +215,9 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
       const int row = (wave * 4 + jj) * 2 + lane / 32;
-      b_lane[jj] = (uint32_t)(row * g.b.sc + ((lane % 32) ^ ((row & 3) << 2)) * 8) * 2u;
+      const int col = ((lane % 32) ^ ((row & 3) << 2)) * 8;
+      b_lane[jj] = (uint32_t)(row * g.b.sc + col) * 2u;
+      b_valid[jj] = col < nvalid;
     }
     const int row = wave * 8 + lane / 8;
     a_lane = (uint32_t)(row * g.a.sc + ((lane % 8) ^ (((row >> 1) & 1) << 2)) * 8) * 2u;
@@ -223,7 +235,8 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
     const char* bp = b_tile0 + kb * b_red_stride;
     const char* ap = a_tile0 + kb * red_stride;
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) load16_to_lds(bp + b_lane[jj], st + (wave * 4 + jj) * 1024);
+    for (int jj = 0; jj < 4; ++jj)
+      if (b_valid[jj]) load16_to_lds(bp + b_lane[jj], st + (wave * 4 + jj) * 1024);
 #pragma unroll
     for (int r = 0; r < R; ++r)
       if (fl & (1u << r)) load16_to_lds(ap + r * a_rstride + a_lane, st + A_OFF + r * TILE + wave * 1024);
@@ -317,6 +330,8 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
   // ---- epilogue: scale, round once, store ---------------------------------------------------------
   // accumulator register v of lane l is element (8*(v/4) + 4*(l/32) + v%4, l%32) of the 32x32 product
   // (first MFMA operand's rows) x (second operand's rows); lanes run along C's contiguous index.
+  if (ns * 64 >= nvalid) return;  // this wave's column slice overhangs N: nothing of it is stored
+  float* part = nsplit > 1 ? g.ws + (int64_t)split * g.M * g.N : nullptr;
 #pragma unroll
   for (int rr = 0; rr < 2; ++rr) {
     const int rb = rb0 + 2 * rh + rr;
@@ -331,7 +346,10 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
           const int lane_i = lane % 32;
           const int64_t m = (int64_t)rb * BS + mt * 32 + (TRANS ? lane_i : reg_i);
           const int64_t n = n0 + ns * 64 + nt * 32 + (TRANS ? reg_i : lane_i);
-          g.c[m * g.c_sr + n * g.c_sc] = T::from_float(acc[rr][mt][nt][v] * g.scale);
+          if (part)  // unscaled fp32 partial in C's own element order; the reduce pass scales and rounds
+            part[TRANS ? n * g.M + m : m * g.N + n] = acc[rr][mt][nt][v];
+          else
+            g.c[m * g.c_sr + n * g.c_sc] = T::from_float(acc[rr][mt][nt][v] * g.scale);
         }
   }
 }
@@ -514,7 +532,7 @@ __global__ __launch_bounds__(THREADS) void sdd_kernel(GemmArgs g, int tiles_m, i
 bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
 
 template <typename T, bool TRANS>
-int launch_dsd(const GemmArgs& g, hipStream_t stream) {
+int launch_dsd(const GemmArgs& g, int splits, hipStream_t stream) {
   static bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dsd_kernel<T, TRANS>),
@@ -523,10 +541,12 @@ int launch_dsd(const GemmArgs& g, hipStream_t stream) {
     configured = true;
   }
   const int Mb = (int)(g.M / BS), Kb = (int)(g.K / BS);
-  const int tiles_m = (Mb + R - 1) / R, tiles_n = (int)(g.N / BN);
-  hipLaunchKernelGGL((dsd_kernel<T, TRANS>), dim3((unsigned)(tiles_m * tiles_n)), dim3(THREADS),
-                     SMEM_BYTES, stream, g, tiles_m, tiles_n, Mb, Kb);
-  return check_launch("dsd_kernel");
+  const int tiles_m = (Mb + R - 1) / R, tiles_n = (int)((g.N + BN - 1) / BN);
+  hipLaunchKernelGGL((dsd_kernel<T, TRANS>), dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits),
+                     dim3(THREADS), SMEM_BYTES, stream, g, tiles_m, tiles_n, Mb, Kb);
+  if (int rc = check_launch("dsd_kernel")) return rc;
+  if (splits > 1) return launch_splitk_reduce(g, splits, TRANS, T::id, stream);
+  return SD_OK;
 }
 
 template <typename T>
@@ -567,22 +587,42 @@ int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   // everything tile-aligned and 16-byte aligned; the three matrices agree on which index is contiguous
   const bool nt = g.a.sc == 1 && g.b.sc == 1 && g.c_sc == 1;  // reduction-contiguous, C row-major
   const bool tn = !nt && g.a.sr == 1 && g.b.sr == 1 && g.c_sr == 1;  // reduction-strided, C column-major
-  const bool shape_ok = g.M > 0 && g.M % BS == 0 && g.N > 0 && g.N % BN == 0 && g.K > 0 &&
-                        g.K % BS == 0 && g.K / BS <= MAX_STEPS;
+  const bool shape_ok = g.M > 0 && g.M % BS == 0 && g.N > 0 && g.N % BS == 0 && g.K > 0 && g.K % BS == 0 &&
+                        g.K / BS < 65536;
   const int64_t lda = nt ? g.a.sr : g.a.sc, ldb = nt ? g.b.sr : g.b.sc;
   const bool align_ok = aligned16(g.a.ptr) && aligned16(g.b.ptr) && lda % 8 == 0 && ldb % 8 == 0 &&
                         lda < (1 << 22) && ldb < (1 << 22);  // per-lane byte offsets are 32-bit
-  const int64_t tiles = ((g.M / BS + R - 1) / R) * (g.N / BN);
+  const int64_t tiles = ((g.M / BS + R - 1) / R) * ((g.N + BN - 1) / BN);
   if (!(nt || tn) || !shape_ok || !align_ok || tiles > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
-  // a long reduction over few output tiles (weight gradient of a tall matrix) is better served by the
-  // generic kernel's split-K when the caller gave it a workspace
-  if (tiles < 128 && g.ws != nullptr) {
-    const int splits = generic_splits(g.M, g.N, g.K, g.bs, mode);
-    if (splits > 1 && g.ws_bytes >= (int64_t)splits * g.M * g.N * 4) return SD_ERR_UNSUPPORTED;
+  // few output tiles and a long reduction (the weight gradient of a tall matrix): split the reduction
+  // over workgroups when the caller gave scratch for the fp32 partials
+  int splits = fast_splits(g.M, g.N, g.K);
+  const int64_t part_bytes = g.M * g.N * 4;
+  if (splits > 1 && (g.ws == nullptr || g.ws_bytes < part_bytes * splits))
+    splits = g.ws ? (int)(g.ws_bytes / part_bytes) : 1;
+  if (splits < 1) splits = 1;
+  if ((g.K / BS + splits - 1) / splits > MAX_STEPS) return SD_ERR_UNSUPPORTED;  // step table is per workgroup
+  if (splits == 1 && tiles < 128 && g.ws != nullptr) {
+    // scratch too small for this kernel's partials: the generic kernel's split may still fit
+    const int gs = generic_splits(g.M, g.N, g.K, g.bs, mode);
+    if (gs > 1 && g.ws_bytes >= (int64_t)gs * part_bytes) return SD_ERR_UNSUPPORTED;
   }
   if (nt)
-    return dtype == SD_BF16 ? launch_dsd<BF16, false>(g, stream) : launch_dsd<F16, false>(g, stream);
-  return dtype == SD_BF16 ? launch_dsd<BF16, true>(g, stream) : launch_dsd<F16, true>(g, stream);
+    return dtype == SD_BF16 ? launch_dsd<BF16, false>(g, splits, stream) : launch_dsd<F16, false>(g, splits, stream);
+  return dtype == SD_BF16 ? launch_dsd<BF16, true>(g, splits, stream) : launch_dsd<F16, true>(g, splits, stream);
+}
+
+// One round of workgroups (one per CU) when the output alone gives fewer than half of that, at least 4
+// reduction blocks per split.
+int fast_splits(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 1;
+  const int64_t tiles = ((M + BS * R - 1) / (BS * R)) * ((N + BN - 1) / BN);
+  const int64_t kb = K / BS;
+  if (tiles >= 128 || kb < 8) return 1;
+  int64_t want = 256 / tiles;
+  if (want > kb / 4) want = kb / 4;
+  while (want > 1 && want * M * N * 4 > (256LL << 20)) --want;
+  return want < 2 ? 1 : (int)want;
 }
 
 }  // namespace sd

@@ -285,9 +285,7 @@ int launch_t(const GemmArgs& g, hipStream_t stream) {
       hipLaunchKernelGGL((gemm_generic_kernel<T, MODE, false, true>), grid, block, 0, stream, g,
                          (int)tiles_n, a_kc, b_kc, a_vec, b_vec);
     if (int rc = check_launch("gemm_generic (split)")) return rc;
-    hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)ceil_div(g.M * g.N, 256)), dim3(256), 0,
-                       stream, g, splits, trans_out);
-    return check_launch("splitk_reduce");
+    return launch_splitk_reduce(g, splits, trans_out, T::id, stream);
   }
   dim3 grid((unsigned)(tiles_m * tiles_n));
   if (trans_out)
@@ -310,6 +308,15 @@ int launch_mode(const GemmArgs& g, int mode, hipStream_t stream) {
 }
 
 }  // namespace
+
+int launch_splitk_reduce(const GemmArgs& g, int splits, bool trans_out, int dtype, hipStream_t stream) {
+  const dim3 grid((unsigned)ceil_div(g.M * g.N, 256));
+  if (dtype == SD_BF16)
+    hipLaunchKernelGGL(splitk_reduce_kernel<BF16>, grid, dim3(256), 0, stream, g, splits, trans_out);
+  else
+    hipLaunchKernelGGL(splitk_reduce_kernel<F16>, grid, dim3(256), 0, stream, g, splits, trans_out);
+  return check_launch("splitk_reduce");
+}
 
 // Split the reduction when the output tiles alone cannot fill the 256 CUs and each tile has a long
 // reduction: aim for about two workgroups per CU, keep at least 8 K-steps (two 64-blocks) per split.

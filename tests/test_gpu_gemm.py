@@ -125,8 +125,11 @@ def test_all_majorness_combinations(a_rm, b_rm, m_rm, out_t):
     (16384, 384, 1536, 64),  # transformer MLP down-projection
     (512, 512, 512, 256),    # large block
     (300, 200, 500, 128),
+    (16384, 128, 576, 64),   # conv patch matrix (8 images): dW = 576 x 128 over a 16384-long reduction, split over workgroups
+    (73728, 64, 128, 64),    # dW reduction of 1152 blocks: more than one workgroup's step table, only reachable split
+    (4096, 320, 192, 64),    # N = 256 + 64: the second column tile overhangs
 ])
-@pytest.mark.parametrize("p", [0.5])
+@pytest.mark.parametrize("p", [0.0, 0.5])
 def test_tails_and_model_shapes(M, N, K, bs, p):
     gen = torch.Generator().manual_seed(3)
     A = make_operand(M, K, torch.float16, "cuda", gen=gen)
@@ -184,7 +187,9 @@ def test_lists_entry_points_match_mask_entry_points():
     assert torch.equal(ext.gemm_sdd_lists(dC, B.T, lists, bs, s), ext.gemm_sdd(dC, B.T, mask, bs, s))
     dW = ext.gemm_dsd_lists(A.T, dC.T, lists.transposed(), bs, s, transposed_out=True).T
     assert dW.is_contiguous()
-    assert torch.equal(dW, ext.gemm_dsd(A.T, dC.T, mask.T, bs, s).T)
+    # the row-major [K, N] result of the mask form comes from a different kernel (other summation order)
+    assert rel_fro(dW, ext.gemm_dsd(A.T, dC.T, mask.T, bs, s).T.float()) <= 1e-3
+    assert torch.equal(dW, ext.gemm_dsd(A.T, dC.T, mask.T, bs, s, transposed_out=True).T)
 
 
 def test_errors_through_the_shim():
