@@ -612,15 +612,15 @@ int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   return dtype == SD_BF16 ? launch_dsd<BF16, true>(g, splits, stream) : launch_dsd<F16, true>(g, splits, stream);
 }
 
-// One round of workgroups (one per CU) when the output alone gives fewer than half of that, at least 4
-// reduction blocks per split.
+// One round of workgroups (one per CU) when the output alone gives fewer than half of that and the
+// reduction is long enough to pay for the extra pass: at least 8 reduction blocks per split.
 int fast_splits(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0) return 1;
   const int64_t tiles = ((M + BS * R - 1) / (BS * R)) * ((N + BN - 1) / BN);
   const int64_t kb = K / BS;
-  if (tiles >= 128 || kb < 8) return 1;
+  if (tiles >= 128 || kb < 32) return 1;
   int64_t want = 256 / tiles;
-  if (want > kb / 4) want = kb / 4;
+  if (want > kb / 8) want = kb / 8;
   while (want > 1 && want * M * N * 4 > (256LL << 20)) --want;
   return want < 2 ? 1 : (int)want;
 }
