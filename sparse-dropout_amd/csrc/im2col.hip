@@ -254,6 +254,194 @@ __global__ __launch_bounds__(256) void col2im_kernel(const uint16_t* __restrict_
       T::from_float(acc);
 }
 
+// Tiled adjoint for aligned patch matrices.  A workgroup owns one image, a band of `hb` input rows and a
+// group of 8 channels.  Everything of the patch matrix that feeds those outputs — the 8*R*S columns of
+// the channel group, for every output row p that touches the band and every q — is copied to LDS first
+// with 16-byte loads (R*S consecutive lanes cover one contiguous row segment; dropped blocks are filled
+// with zeros instead of being read), then each thread sums the taps of its outputs out of LDS.  Global
+// reads are whole segments instead of one 2-byte element per lane and cache line.
+constexpr int C2I_CG = 8;
+constexpr int C2I_MAX_LDS = 64 * 1024;
+
+template <typename T>
+__global__ __launch_bounds__(256) void col2im_tile_kernel(const uint16_t* __restrict__ cols, int64_t ld,
+                                                          uint16_t* __restrict__ dx, ConvGeom g,
+                                                          const uint8_t* mask, int64_t msr, int64_t msc,
+                                                          int bs, int hb, int np_max, int bands) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t seg[];  // [p][q][8*R*S + 2]
+  const int t = threadIdx.x;
+  const int rs_n = g.r * g.s;
+  const int seg_h = C2I_CG * rs_n + 2;  // halfs per (p, q) segment; the 2 spare halfs spread the banks
+  int b = blockIdx.x;
+  const int band = b % bands;
+  b /= bands;
+  const int cgs = g.c / C2I_CG;
+  const int c0 = (b % cgs) * C2I_CG;
+  const int n_i = b / cgs;
+  const int h0 = band * hb;
+  const int h1 = (h0 + hb < g.h ? h0 + hb : g.h);  // band = input rows [h0, h1)
+  // output rows p with a tap inside the band: p*str_h - pad_h + r*dil_h in [h0, h1) for some r
+  int p_lo = h0 + g.pad_h - (g.r - 1) * g.dil_h;
+  p_lo = p_lo <= 0 ? 0 : (p_lo + g.str_h - 1) / g.str_h;
+  int p_hi = (h1 - 1 + g.pad_h) / g.str_h;
+  if (p_hi > g.p - 1) p_hi = g.p - 1;
+  const int np = p_hi - p_lo + 1;  // <= np_max (may be <= 0 for a band no output row reaches)
+
+  // ---- stage: R*S 16-byte chunks per (p, q) --------------------------------------------------------
+  const int chunks = (np > 0 ? np : 0) * g.q * rs_n;
+  const int64_t row0 = ((int64_t)n_i * g.p + p_lo) * g.q;
+  const int col0 = c0 * rs_n;
+  for (int ch = t; ch < chunks; ch += 256) {
+    const int row_l = ch / rs_n, k = ch - row_l * rs_n;
+    const int64_t row = row0 + row_l;
+    const int col = col0 + k * 8;
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (!mask || !mask[(row / bs) * msr + (col / bs) * msc])
+      v = *reinterpret_cast<const u32x4*>(cols + row * ld + col);
+    uint32_t* dst = reinterpret_cast<uint32_t*>(seg + row_l * seg_h + k * 8);
+    dst[0] = v.x;
+    dst[1] = v.y;
+    dst[2] = v.z;
+    dst[3] = v.w;
+  }
+  __syncthreads();
+
+  // ---- sum the taps ----------------------------------------------------------------------------------
+  const bool c_fast = g.xs_c == 1;  // channels-last image: lanes along c, else along w
+  const int outs = C2I_CG * (h1 - h0) * g.w;
+  uint16_t* dxn = dx + (int64_t)n_i * g.xs_n;
+  for (int o = t; o < outs; o += 256) {
+    int c_l, hi, wi;
+    if (c_fast) {
+      c_l = o % C2I_CG;
+      wi = (o / C2I_CG) % g.w;
+      hi = h0 + o / (C2I_CG * g.w);
+    } else {
+      wi = o % g.w;
+      hi = h0 + (o / g.w) % (h1 - h0);
+      c_l = o / (g.w * (h1 - h0));
+    }
+    float acc = 0.f;
+    for (int rr = 0; rr < g.r; ++rr) {
+      const int pu = hi + g.pad_h - rr * g.dil_h;
+      if (pu < 0) break;  // pu only decreases with rr
+      int pp = pu;
+      if (g.str_h != 1) {
+        pp = pu / g.str_h;
+        if (pp * g.str_h != pu) continue;
+      }
+      if (pp >= g.p) continue;
+      const uint16_t* prow = seg + (pp - p_lo) * g.q * seg_h + (c_l * g.r + rr) * g.s;
+      for (int ss = 0; ss < g.s; ++ss) {
+        const int qu = wi + g.pad_w - ss * g.dil_w;
+        if (qu < 0) break;
+        int qq = qu;
+        if (g.str_w != 1) {
+          qq = qu / g.str_w;
+          if (qq * g.str_w != qu) continue;
+        }
+        if (qq >= g.q) continue;
+        acc += T::to_float(prow[qq * seg_h + ss]);
+      }
+    }
+    dxn[(int64_t)(c0 + c_l) * g.xs_c + (int64_t)hi * g.xs_h + (int64_t)wi * g.xs_w] = T::from_float(acc);
+  }
+}
+
+// The same for unit stride and dilation (the usual 3x3 / 5x5 layer), where output (h, w) takes tap
+// (r, s) from patch row (h + pad_h - r, w + pad_w - s): the staged window gets a zero halo, rows and
+// columns outside the patch matrix included, so the tap loop has no bounds checks and walks LDS with
+// constant strides.  A thread owns one (channel, w) column of the band and runs down its rows.
+template <typename T>
+__global__ __launch_bounds__(256) void col2im_unit_kernel(const uint16_t* __restrict__ cols, int64_t ld,
+                                                          uint16_t* __restrict__ dx, ConvGeom g,
+                                                          const uint8_t* mask, int64_t msr, int64_t msc,
+                                                          int bs, int hb, int bands) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t seg[];  // [hb + R - 1][W + S - 1][8*R*S + 2]
+  const int t = threadIdx.x;
+  const int rs_n = g.r * g.s;
+  const int seg_h = C2I_CG * rs_n + 2;
+  int b = blockIdx.x;
+  const int band = b % bands;
+  b /= bands;
+  const int cgs = g.c / C2I_CG;
+  const int c0 = (b % cgs) * C2I_CG;
+  const int n_i = b / cgs;
+  const int h0 = band * hb;
+  const int h1 = (h0 + hb < g.h ? h0 + hb : g.h);
+  const int pe = (h1 - h0) + g.r - 1, qe = g.w + g.s - 1;     // staged window
+  const int p_first = h0 + g.pad_h - (g.r - 1), q_first = g.pad_w - (g.s - 1);  // its top-left (p, q)
+
+  // ---- stage: R*S 16-byte chunks per window position, zeros outside the matrix and for dropped blocks
+  const int chunks = pe * qe * rs_n;
+  const int col0 = c0 * rs_n;
+  for (int ch0 = t; ch0 < chunks; ch0 += 4 * 256) {
+    u32x4 v[4];
+    const uint16_t* src[4];  // null: zeros
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {  // four independent mask reads, then four independent loads, per lane
+      const int ch = ch0 + i * 256;
+      src[i] = nullptr;
+      uint8_t dropped = 0;
+      if (ch < chunks) {
+        const int pos = ch / rs_n, k = ch - pos * rs_n;
+        const int pp = p_first + pos / qe, qq = q_first + pos % qe;
+        if (pp >= 0 && pp < g.p && qq >= 0 && qq < g.q) {
+          const int64_t row = ((int64_t)n_i * g.p + pp) * g.q + qq;
+          const int col = col0 + k * 8;
+          src[i] = cols + row * ld + col;
+          if (mask) dropped = mask[(row / bs) * msr + (col / bs) * msc];
+        }
+      }
+      if (dropped) src[i] = nullptr;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[i] = u32x4{0u, 0u, 0u, 0u};
+      if (src[i]) v[i] = *reinterpret_cast<const u32x4*>(src[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int ch = ch0 + i * 256;
+      if (ch < chunks) {
+        const int pos = ch / rs_n, k = ch - pos * rs_n;
+        uint32_t* dst = reinterpret_cast<uint32_t*>(seg + pos * seg_h + k * 8);
+        dst[0] = v[i].x;
+        dst[1] = v[i].y;
+        dst[2] = v[i].z;
+        dst[3] = v[i].w;
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- sum the taps: window position of tap (r, s) of output (h, w) is (h - h0 + R-1-r, w + S-1-s) ---
+  const bool c_fast = g.xs_c == 1;
+  const int pairs = C2I_CG * g.w;
+  const int row_h = qe * seg_h;  // halfs per window row
+  uint16_t* dxn = dx + (int64_t)n_i * g.xs_n;
+  for (int pr = t; pr < pairs; pr += 256) {
+    const int c_l = c_fast ? pr % C2I_CG : pr / g.w;
+    const int wi = c_fast ? pr / C2I_CG : pr % g.w;
+    // tap (0, 0) of the band's first row
+    const uint16_t* base = seg + (g.r - 1) * row_h + (wi + g.s - 1) * seg_h + c_l * rs_n;
+    uint16_t* out = dxn + (int64_t)(c0 + c_l) * g.xs_c + (int64_t)h0 * g.xs_h + (int64_t)wi * g.xs_w;
+    for (int hl = 0; hl < h1 - h0; ++hl) {
+      float acc = 0.f;
+      const uint16_t* tap_r = base + hl * row_h;
+      for (int rr = 0; rr < g.r; ++rr) {
+        const uint16_t* tap = tap_r;
+        for (int ss = 0; ss < g.s; ++ss) {
+          acc += T::to_float(*tap);
+          tap -= seg_h - 1;  // one window column to the left, next s
+        }
+        tap_r -= row_h - g.s;  // one window row up, next r
+      }
+      out[(int64_t)hl * g.xs_h] = T::from_float(acc);
+    }
+  }
+}
+
 }  // namespace
 
 static int make_geom(ConvGeom& g, int64_t n, int64_t c, int64_t h, int64_t w, int64_t r, int64_t s,
@@ -321,6 +509,44 @@ int col2im(const void* cols, int64_t ld, void* dx, int64_t sn, int64_t sc, int64
   SD_REQUIRE(dx && cols, "col2im: null pointer");
   SD_REQUIRE(ld >= c * r * s, "col2im: cols_ld %lld < C*R*S %lld", (long long)ld, (long long)(c * r * s));
   if (mask) SD_REQUIRE(bs > 0, "col2im: block_size must be positive with a mask");
+  // tiled kernel: 16-byte loads of 8-channel column groups need aligned rows and whole groups
+  if (c % C2I_CG == 0 && ld % 8 == 0 && reinterpret_cast<uintptr_t>(cols) % 16 == 0 &&
+      (!mask || bs % 8 == 0)) {
+    const int seg_bytes = (C2I_CG * g.r * g.s + 2) * 2;
+    const bool unit = g.str_h == 1 && g.str_w == 1 && g.dil_h == 1 && g.dil_w == 1;
+    for (int band_rows = 8; band_rows >= 1; band_rows /= 2) {  // the tallest band whose staging fits
+      const int hb = band_rows < g.h ? band_rows : g.h;
+      if (unit) {
+        const int64_t lds = (int64_t)(hb + g.r - 1) * (g.w + g.s - 1) * seg_bytes;
+        const int64_t bands = ceil_div(g.h, hb);
+        const int64_t wgs = n * (c / C2I_CG) * bands;
+        if (lds > C2I_MAX_LDS || wgs > 0x7fffffffLL) continue;
+        if (dtype == SD_BF16)
+          hipLaunchKernelGGL(col2im_unit_kernel<BF16>, dim3((unsigned)wgs), dim3(256), (size_t)lds, stream,
+                             (const uint16_t*)cols, ld, (uint16_t*)dx, g, mask, msr, msc, mask ? (int)bs : 1,
+                             hb, (int)bands);
+        else
+          hipLaunchKernelGGL(col2im_unit_kernel<F16>, dim3((unsigned)wgs), dim3(256), (size_t)lds, stream,
+                             (const uint16_t*)cols, ld, (uint16_t*)dx, g, mask, msr, msc, mask ? (int)bs : 1,
+                             hb, (int)bands);
+        return check_launch("col2im_unit");
+      }
+      const int np_max = (hb - 1 + (g.r - 1) * g.dil_h) / g.str_h + 1;
+      const int64_t lds = (int64_t)np_max * g.q * seg_bytes;
+      const int64_t bands = ceil_div(g.h, hb);
+      const int64_t wgs = n * (c / C2I_CG) * bands;
+      if (lds > C2I_MAX_LDS || wgs > 0x7fffffffLL) continue;
+      if (dtype == SD_BF16)
+        hipLaunchKernelGGL(col2im_tile_kernel<BF16>, dim3((unsigned)wgs), dim3(256), (size_t)lds, stream,
+                           (const uint16_t*)cols, ld, (uint16_t*)dx, g, mask, msr, msc, mask ? (int)bs : 1, hb,
+                           np_max, (int)bands);
+      else
+        hipLaunchKernelGGL(col2im_tile_kernel<F16>, dim3((unsigned)wgs), dim3(256), (size_t)lds, stream,
+                           (const uint16_t*)cols, ld, (uint16_t*)dx, g, mask, msr, msc, mask ? (int)bs : 1, hb,
+                           np_max, (int)bands);
+      return check_launch("col2im_tile");
+    }
+  }
   const int64_t total = n * c * h * w;
   const int64_t blocks = ceil_div(total, 256);
   SD_REQUIRE(blocks <= 0x7fffffffLL, "col2im: image too large");
