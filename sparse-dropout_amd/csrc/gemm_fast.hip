@@ -22,8 +22,11 @@
 // order [reduction][64 or 256 contiguous columns] and the MFMA fragments (8 consecutive reduction
 // elements of one column per lane) are formed by ds_read_b64_tr_b16, two per fragment.  That read
 // takes, per 16-lane group, 4 reduction rows x 32 bytes; the chunk swizzles below put those on
-// distinct banks.  The MFMA operands are swapped so that lanes run along K, the contiguous index of
-// the row-major dW the kernel writes.
+// distinct banks.
+//
+// Either instance writes C in either majorness: for a column-major C (the row-major dW[N,K] seen as
+// the [K,N] product's transpose) the two MFMA operands are swapped, so that lanes run along C's rows,
+// its contiguous index.
 //
 // ---- SDD (the input gradient dX = s*(dY.W) (.) keep) ----------------------------------------------
 // A workgroup owns a 4x4 patch of 64x64 output tiles and computes only the kept ones; the reduction
@@ -96,7 +99,8 @@ __device__ inline u32x2 lds_read_tr(const char* p) {
 // TRANS = false: A[row][red], B[col][red] with the reduction index contiguous (forward / dense)
 // TRANS = true : A and B are given as transposed views, the reduction index is the strided one (dW)
 // In both cases "Mb" counts the row blocks of A (of X^T for dW) and "Kb" the reduction blocks.
-template <typename T, bool TRANS>
+// CM = C is column-major: the MFMA operands are swapped so that lanes run along C's rows
+template <typename T, bool TRANS, bool CM>
 __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, int tiles_n,
                                                       int Mb, int Kb_all) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -305,8 +309,8 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt)
-          acc[rr][mt][nt] = TRANS ? T::mfma32(bf[nt][ks], af[u & 1][mt], acc[rr][mt][nt])
-                                  : T::mfma32(af[u & 1][mt], bf[nt][ks], acc[rr][mt][nt]);
+          acc[rr][mt][nt] = CM ? T::mfma32(bf[nt][ks], af[u & 1][mt], acc[rr][mt][nt])
+                               : T::mfma32(af[u & 1][mt], bf[nt][ks], acc[rr][mt][nt]);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -344,10 +348,10 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
         for (int v = 0; v < 16; ++v) {
           const int reg_i = 8 * (v / 4) + 4 * (lane / 32) + (v % 4);
           const int lane_i = lane % 32;
-          const int64_t m = (int64_t)rb * BS + mt * 32 + (TRANS ? lane_i : reg_i);
-          const int64_t n = n0 + ns * 64 + nt * 32 + (TRANS ? reg_i : lane_i);
+          const int64_t m = (int64_t)rb * BS + mt * 32 + (CM ? lane_i : reg_i);
+          const int64_t n = n0 + ns * 64 + nt * 32 + (CM ? reg_i : lane_i);
           if (part)  // unscaled fp32 partial in C's own element order; the reduce pass scales and rounds
-            part[TRANS ? n * g.M + m : m * g.N + n] = acc[rr][mt][nt][v];
+            part[CM ? n * g.M + m : m * g.N + n] = acc[rr][mt][nt][v];
           else
             g.c[m * g.c_sr + n * g.c_sc] = T::from_float(acc[rr][mt][nt][v] * g.scale);
         }
@@ -531,21 +535,21 @@ __global__ __launch_bounds__(THREADS) void sdd_kernel(GemmArgs g, int tiles_m, i
 
 bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
 
-template <typename T, bool TRANS>
+template <typename T, bool TRANS, bool CM>
 int launch_dsd(const GemmArgs& g, int splits, hipStream_t stream) {
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dsd_kernel<T, TRANS>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dsd_kernel<T, TRANS, CM>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
     if (e != hipSuccess) return fail(SD_ERR_RUNTIME, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     configured = true;
   }
   const int Mb = (int)(g.M / BS), Kb = (int)(g.K / BS);
   const int tiles_m = (Mb + R - 1) / R, tiles_n = (int)((g.N + BN - 1) / BN);
-  hipLaunchKernelGGL((dsd_kernel<T, TRANS>), dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits),
+  hipLaunchKernelGGL((dsd_kernel<T, TRANS, CM>), dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits),
                      dim3(THREADS), SMEM_BYTES, stream, g, tiles_m, tiles_n, Mb, Kb);
   if (int rc = check_launch("dsd_kernel")) return rc;
-  if (splits > 1) return launch_splitk_reduce(g, splits, TRANS, T::id, stream);
+  if (splits > 1) return launch_splitk_reduce(g, splits, CM, T::id, stream);
   return SD_OK;
 }
 
@@ -584,9 +588,10 @@ int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   // kernel with every tile kept
   if (mode == kDense && g.a.sc == 1 && g.b.sr == 1 && g.b.sc != 1 && g.c_sc == 1) return try_sdd(g, dtype, stream);
   if (mode == kDsd && g.bs != BS) return SD_ERR_UNSUPPORTED;
-  // everything tile-aligned and 16-byte aligned; the three matrices agree on which index is contiguous
-  const bool nt = g.a.sc == 1 && g.b.sc == 1 && g.c_sc == 1;  // reduction-contiguous, C row-major
-  const bool tn = !nt && g.a.sr == 1 && g.b.sr == 1 && g.c_sr == 1;  // reduction-strided, C column-major
+  // everything tile-aligned and 16-byte aligned; A and B agree on whether the reduction index is contiguous
+  const bool nt = g.a.sc == 1 && g.b.sc == 1;         // reduction-contiguous operands
+  const bool tn = !nt && g.a.sr == 1 && g.b.sr == 1;  // reduction-strided operands
+  const bool cm = g.c_sc != 1;                        // column-major C
   const bool shape_ok = g.M > 0 && g.M % BS == 0 && g.N > 0 && g.N % BS == 0 && g.K > 0 && g.K % BS == 0 &&
                         g.K / BS < 65536;
   const int64_t lda = nt ? g.a.sr : g.a.sc, ldb = nt ? g.b.sr : g.b.sc;
@@ -607,9 +612,12 @@ int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
     const int gs = generic_splits(g.M, g.N, g.K, g.bs, mode);
     if (gs > 1 && g.ws_bytes >= (int64_t)gs * part_bytes) return SD_ERR_UNSUPPORTED;
   }
-  if (nt)
-    return dtype == SD_BF16 ? launch_dsd<BF16, false>(g, splits, stream) : launch_dsd<F16, false>(g, splits, stream);
-  return dtype == SD_BF16 ? launch_dsd<BF16, true>(g, splits, stream) : launch_dsd<F16, true>(g, splits, stream);
+  if (dtype == SD_BF16) {
+    if (nt) return cm ? launch_dsd<BF16, false, true>(g, splits, stream) : launch_dsd<BF16, false, false>(g, splits, stream);
+    return cm ? launch_dsd<BF16, true, true>(g, splits, stream) : launch_dsd<BF16, true, false>(g, splits, stream);
+  }
+  if (nt) return cm ? launch_dsd<F16, false, true>(g, splits, stream) : launch_dsd<F16, false, false>(g, splits, stream);
+  return cm ? launch_dsd<F16, true, true>(g, splits, stream) : launch_dsd<F16, true, false>(g, splits, stream);
 }
 
 // One round of workgroups (one per CU) when the output alone gives fewer than half of that and the
