@@ -51,10 +51,15 @@ constexpr int TILE = BS * BS * 2;              // bytes of one 64 x 64 tile (row
 constexpr int STAGE = (BN / BS) * TILE + R * TILE;  // W tile (32 KB) + up to 4 X tiles (32 KB)
 constexpr int A_OFF = (BN / BS) * TILE;
 constexpr int MAX_STEPS = 1024;
-constexpr int SMEM_STEPS = 2 * STAGE;                  // uint16 kb[MAX_STEPS]
-constexpr int SMEM_FLAGS = SMEM_STEPS + 2 * MAX_STEPS;  // uint8 flags[MAX_STEPS]
-constexpr int SMEM_SCRATCH = SMEM_FLAGS + MAX_STEPS;    // uint32 per K block while merging
+// step table: one uint32 per step of the union walk, reduction block | keep flags << 16, followed by
+// STEP_PAD zero entries so that look-ahead reads past the end are harmless
+constexpr int STEP_PAD = 4;
+constexpr int SMEM_STEPS = 2 * STAGE;
+constexpr int SMEM_SCRATCH = SMEM_STEPS + 4 * (MAX_STEPS + STEP_PAD);  // uint32 per K block while merging
 constexpr int SMEM_BYTES = SMEM_SCRATCH + 4 * MAX_STEPS + 16;
+__device__ inline int step_block(uint32_t e) { return (int)(e & 0xffffu); }
+__device__ inline uint32_t step_flags(uint32_t e) { return e >> 16; }
+__device__ inline uint32_t uniform(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane(v); }
 
 typedef __attribute__((address_space(3))) void lds_void;
 
@@ -104,8 +109,7 @@ template <typename T, bool TRANS, bool CM>
 __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, int tiles_n,
                                                       int Mb, int Kb_all) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  uint16_t* step_kb = reinterpret_cast<uint16_t*>(smem + SMEM_STEPS);
-  uint8_t* step_fl = reinterpret_cast<uint8_t*>(smem + SMEM_FLAGS);
+  uint32_t* step_e = reinterpret_cast<uint32_t*>(smem + SMEM_STEPS);
   uint32_t* scratch = reinterpret_cast<uint32_t*>(smem + SMEM_SCRATCH);
   int* nsteps_p = reinterpret_cast<int*>(smem + SMEM_SCRATCH + 4 * MAX_STEPS);
 
@@ -150,11 +154,11 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
       const uint64_t bal = __ballot(f != 0);
       if (f) {
         const int pos = base + __popcll(bal & lt);
-        step_kb[pos] = (uint16_t)(kb_lo + k);
-        step_fl[pos] = (uint8_t)f;
+        step_e[pos] = (uint32_t)(kb_lo + k) | (f << 16);
       }
       base += __popcll(bal);
     }
+    if (lane < STEP_PAD) step_e[base + lane] = 0u;
     if (lane == 0) *nsteps_p = base;
   }
   __syncthreads();
@@ -232,9 +236,9 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
   }
   const int64_t b_red_stride = TRANS ? (int64_t)BS * g.b.sc * 2 : (int64_t)BS * 2;
 
-  auto issue_loads = [&](int step, int stage) {
-    const int kb = __builtin_amdgcn_readfirstlane((int)step_kb[step]);
-    const uint32_t fl = __builtin_amdgcn_readfirstlane((uint32_t)step_fl[step]);
+  auto issue_loads = [&](uint32_t entry, int stage) {  // entry: wave-uniform step table word
+    const int kb = step_block(entry);
+    const uint32_t fl = step_flags(entry);
     char* st = smem + stage * STAGE;
     const char* bp = b_tile0 + kb * b_red_stride;
     const char* ap = a_tile0 + kb * red_stride;
@@ -315,20 +319,26 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
     }
   };
 
-  if (nsteps > 0) issue_loads(0, 0);
+  // Table words are read two steps ahead into a VGPR and made uniform a step later, when the read has
+  // long returned: a read-and-wait at the top of a step would put an LDS round trip in front of its MFMAs.
+  uint32_t e_cur = uniform(step_e[0]), e_next = uniform(step_e[1]);
+  if (nsteps > 0) issue_loads(e_cur, 0);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
   for (int step = 0; step < nsteps; ++step) {
     const int stage = step & 1;
-    if (step + 1 < nsteps) issue_loads(step + 1, stage ^ 1);
-    const uint32_t mine = (__builtin_amdgcn_readfirstlane((uint32_t)step_fl[step]) >> (2 * rh)) & 3u;
+    const uint32_t e_after = step_e[step + 2];
+    if (step + 1 < nsteps) issue_loads(e_next, stage ^ 1);
+    const uint32_t mine = (step_flags(e_cur) >> (2 * rh)) & 3u;
     const char* st = smem + stage * STAGE;
     if (mine == 3u) compute(std::integral_constant<int, 3>{}, st);
     else if (mine == 1u) compute(std::integral_constant<int, 1>{}, st);
     else if (mine == 2u) compute(std::integral_constant<int, 2>{}, st);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    e_cur = e_next;
+    e_next = uniform(e_after);
   }
 
   // ---- epilogue: scale, round once, store ---------------------------------------------------------
