@@ -489,15 +489,17 @@ __global__ __launch_bounds__(THREADS) void sdd_kernel(GemmArgs g, int tiles_m, i
     if (step + 1 < nsteps) issue_loads(step + 1, stage ^ 1);
     if (mine) {
       const char* st = smem + stage * STAGE;
-      // this wave's 32-row slice of the dY tiles of its two row blocks, all four 16-wide sub-steps
+      // this wave's 32-row slice of the dY tiles of its two row blocks, all four 16-wide sub-steps.
+      // Every fragment read of the step is unconditional (tiles that were not loaded give unused
+      // garbage): a read under a branch would make the compiler's LDS wait counts imprecise and every
+      // MFMA below would wait for all reads in flight instead of just its own operands.
       u32x4 af[2][4];
 #pragma unroll
-      for (int rr = 0; rr < 2; ++rr)
-        if ((mine >> (4 * rr)) & 0xfu) {
+      for (int rr = 0; rr < 2; ++rr) {
 #pragma unroll
-          for (int ks = 0; ks < 4; ++ks)
-            af[rr][ks] = *reinterpret_cast<const u32x4*>(st + (2 * rh + rr) * TILE + a_off[ks]);
-        }
+        for (int ks = 0; ks < 4; ++ks)
+          af[rr][ks] = *reinterpret_cast<const u32x4*>(st + (2 * rh + rr) * TILE + a_off[ks]);
+      }
       // W fragments of column block c+1 are read before the MFMAs of column block c
       u32x4 bf[2][4];
       auto read_b = [&](int c) {
@@ -508,19 +510,17 @@ __global__ __launch_bounds__(THREADS) void sdd_kernel(GemmArgs g, int tiles_m, i
           bf[c & 1][ks] = u32x4{lo.x, lo.y, hi.x, hi.y};
         }
       };
-      if (mycols & 1u) read_b(0);
+      read_b(0);
 #pragma unroll
       for (int c = 0; c < R; ++c) {
-        if (c + 1 < R && (mycols & (1u << (c + 1)))) read_b(c + 1);
+        if (c + 1 < R) read_b(c + 1);
         __builtin_amdgcn_sched_barrier(0);
-        if (mycols & (1u << c)) {
 #pragma unroll
-          for (int rr = 0; rr < 2; ++rr)
-            if (mine & (1u << (4 * rr + c))) {
+        for (int rr = 0; rr < 2; ++rr)
+          if (mine & (1u << (4 * rr + c))) {
 #pragma unroll
-              for (int ks = 0; ks < 4; ++ks) acc[rr][c] = T::mfma32(af[rr][ks], bf[c & 1][ks], acc[rr][c]);
-            }
-        }
+            for (int ks = 0; ks < 4; ++ks) acc[rr][c] = T::mfma32(af[rr][ks], bf[c & 1][ks], acc[rr][c]);
+          }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
