@@ -36,6 +36,7 @@
 // Waves are (32x32 quadrant of every tile = wave%4) x (row-block pair = wave/4), so the two waves of a
 // SIMD together issue 4 MFMAs per kept tile per step: MFMA work follows the kept count and stays
 // balanced over the SIMDs.  Dropped tiles of the patch are written as zeros by the same workgroup.
+#include <cstdlib>
 #include <type_traits>
 
 #include "common.h"
@@ -543,6 +544,264 @@ __global__ __launch_bounds__(THREADS) void sdd_kernel(GemmArgs g, int tiles_m, i
     }
 }
 
+// ---- SDD with column groups ---------------------------------------------------------------------------
+// With half of the tiles dropped a 4x4 patch still needs nearly all of its 4 + 4 operand tiles per
+// reduction step for about 8 kept tiles.  Here a workgroup owns 4 row blocks x a GROUP of consecutive
+// column blocks, chosen greedily along the row so that it has at most GW column blocks with anything
+// kept and at most 16 kept tiles: 4 + 6 operand tiles per step for about 12 kept tiles at p = 0.5, the
+// same 4 + 4 for 16 as the patch kernel at p = 0.  Column blocks with nothing kept in these 4 rows
+// cost nothing (zeros are stored for them).  Group boundaries depend on the mask, so every workgroup of
+// a row quad repeats the same scan over the quad's per-column keep flags and takes the group whose index
+// it was launched with (the grid has the worst case ceil(Cb/4) groups per quad; surplus workgroups exit).
+// A wave owns up to two WHOLE kept tiles (tile t of the group goes to wave t%8, so the two waves of a
+// SIMD always carry equal work +-1): 2x2 MFMAs per 16-wide step from 2 + 2 fragments, accumulators
+// statically indexed by the wave's slot, operand tiles addressed dynamically.
+constexpr int GW = 6;                      // column blocks with kept tiles per group
+constexpr int G_BOFF = R * TILE;           // dY tiles first, then W tiles
+constexpr int G_STAGE = (R + GW) * TILE;   // 80 KB
+constexpr int G_SMEM = 2 * G_STAGE;        // all of the 160 KB; everything else lives in registers
+constexpr int G_MAX_CB = 32768;            // per-column flags share the first stage before the loads start
+
+template <typename T>
+__global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tiles_m, int gmax, int Mb,
+                                                            int Cb) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  uint32_t* flags = reinterpret_cast<uint32_t*>(smem);  // bit r: tile (row block rb0 + r, column block c) kept
+  int* rec = reinterpret_cast<int*>(smem + 4 * ((Cb + 3) & ~3));  // c_lo, c_hi, ncols, kept bits, cols[GW]
+
+  int tm, gi;
+  tile_of_block(blockIdx.x, tiles_m, gmax, tm, gi);
+  const int tid = threadIdx.x;
+  const int lane = tid % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  const int rb0 = tm * R;
+
+  // ---- per-column keep flags of this row quad -------------------------------------------------------
+  {
+    const uint32_t all = (rb0 + R <= Mb) ? 0xfu : ((1u << (Mb - rb0)) - 1u);
+    const uint32_t init = g.row_ptr ? 0u : all;
+    for (int i = tid; i < Cb; i += THREADS) flags[i] = init;
+    if (tid < 16) rec[tid] = 0;
+  }
+  __syncthreads();
+  if (g.row_ptr) {
+    for (int r = 0; r < R; ++r) {
+      if (rb0 + r >= Mb) break;
+      const int beg = g.row_ptr[rb0 + r], end = g.row_ptr[rb0 + r + 1];
+      for (int i = beg + tid; i < end; i += THREADS) atomicOr(&flags[g.col_idx[i]], 1u << r);
+    }
+    __syncthreads();
+  }
+
+  // ---- the group this workgroup was launched for ---------------------------------------------------------
+  if (wave == 0) {
+    int grp = 0, start = 0, width = 0, cnt = 0, lo = -1, hi = -1;
+    for (int base = 0; base < Cb && hi < 0; base += 64) {
+      const uint32_t fv = (base + lane < Cb) ? flags[base + lane] : 0u;
+      const int lim = Cb - base < 64 ? Cb - base : 64;
+      for (int i = 0; i < lim; ++i) {
+        const uint32_t f = (uint32_t)__builtin_amdgcn_readlane((int)fv, i);
+        if (f == 0) continue;
+        const int a = __builtin_popcount(f);
+        if (width == GW || cnt + a > 16) {  // the group ends in front of this column block
+          if (grp == gi) {
+            lo = start;
+            hi = base + i;
+            break;
+          }
+          ++grp;
+          start = base + i;
+          width = 0;
+          cnt = 0;
+        }
+        ++width;
+        cnt += a;
+      }
+    }
+    if (hi < 0 && grp == gi) {  // the last group runs to the end of the row
+      lo = start;
+      hi = Cb;
+    }
+    int n = 0;
+    uint32_t kept = 0;  // bit 4*j + r
+    for (int c = lo; c < hi; ++c) {
+      const uint32_t f = (uint32_t)__builtin_amdgcn_readfirstlane((int)flags[c]);
+      if (f) {
+        if (lane == 0) rec[4 + n] = c;
+        kept |= f << (4 * n);
+        ++n;
+      }
+    }
+    if (lane == 0) {
+      rec[0] = lo;
+      rec[1] = hi;
+      rec[2] = n;
+      rec[3] = (int)kept;
+    }
+  }
+  __syncthreads();
+  const int c_lo = __builtin_amdgcn_readfirstlane(rec[0]);
+  const int c_hi = __builtin_amdgcn_readfirstlane(rec[1]);
+  if (c_lo < 0) return;  // fewer groups in this row quad than the grid provides for
+  const int ncols = __builtin_amdgcn_readfirstlane(rec[2]);
+  const uint32_t kept = (uint32_t)__builtin_amdgcn_readfirstlane(rec[3]);
+  int cols[GW];
+#pragma unroll
+  for (int j = 0; j < GW; ++j) cols[j] = __builtin_amdgcn_readfirstlane(rec[4 + j]);
+  const int ntiles = __builtin_popcount(kept);
+
+  // this wave's tiles: tile t of the group (set bits of `kept` in order) belongs to wave t % 8
+  int my_r[2], my_j[2], my_c[2];
+  bool act[2];
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const int t = wave + 8 * k;
+    act[k] = t < ntiles;
+    uint32_t m = kept;
+    for (int i = 0; i < t; ++i) m &= m - 1u;
+    const int b = (act[k] && m) ? __builtin_ctz(m) : 0;
+    my_j[k] = b / 4;
+    my_r[k] = b % 4;
+    my_c[k] = __builtin_amdgcn_readfirstlane(rec[4 + my_j[k]]);
+  }
+  uint32_t rowmask = 0;
+#pragma unroll
+  for (int j = 0; j < GW; ++j) rowmask |= (kept >> (4 * j)) & 0xfu;
+
+  // ---- zeros for the dropped tiles of the group's column range ----------------------------------------
+  {
+    const int row = tid / 8, ch = tid % 8;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    for (int c = c_lo; c < c_hi; ++c) {
+      const uint32_t f = (uint32_t)__builtin_amdgcn_readfirstlane((int)flags[c]);
+      for (int r = 0; r < R; ++r) {
+        if (rb0 + r >= Mb) break;
+        if (!((f >> r) & 1u))
+          *reinterpret_cast<u32x4*>(g.c + ((int64_t)(rb0 + r) * BS + row) * g.c_sr + (int64_t)c * BS + ch * 8) = z;
+      }
+    }
+  }
+  if (kept == 0) return;
+  __syncthreads();  // flags and rec are dead: the stages may be written
+
+  // ---- per-lane constants -----------------------------------------------------------------------------
+  int a_off[4], b_off[4];
+  {
+    const int fr_sw = (lane >> 1) & 7;
+    const int b4 = lane / 16, e = (lane % 16) / 4, j = lane % 4;
+    const int row = 8 * (b4 / 2) + e;
+    const int b_ch = (2 * (b4 % 2) + j / 2) ^ (((e >> 1) & 1) << 2);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      a_off[ks] = (lane % 32) * 128 + ((2 * ks + lane / 32) ^ fr_sw) * 16;  // + 32*128 for the second 32 rows
+      b_off[ks] = (16 * ks + row) * 128 + b_ch * 16 + (j % 2) * 8;           // ^ 64 for the second 32 columns
+    }
+  }
+  const int nsteps = (int)(g.K / BS);
+  const char* a_ptr0;
+  const char* b_ptr0;
+  {
+    const int row = wave * 8 + lane / 8;
+    const int pch = lane % 8;
+    a_ptr0 = reinterpret_cast<const char*>(g.a.ptr + ((int64_t)rb0 * BS + row) * g.a.sr +
+                                           (pch ^ ((row >> 1) & 7)) * 8);
+    b_ptr0 = reinterpret_cast<const char*>(g.b.ptr + (int64_t)row * g.b.sc +
+                                           (pch ^ (((row >> 1) & 1) << 2)) * 8);
+  }
+  const uint32_t a_tile_stride = (uint32_t)(BS * g.a.sr) * 2u;
+  const int64_t b_step_stride = (int64_t)BS * g.b.sc * 2;
+  auto issue_loads = [&](int step, int stage) {
+    char* st = smem + stage * G_STAGE + wave * 1024;
+    const char* ap = a_ptr0 + step * (BS * 2);
+    const char* bp = b_ptr0 + step * b_step_stride;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (rowmask & (1u << r)) load16_to_lds(ap + r * a_tile_stride, st + r * TILE);
+#pragma unroll
+    for (int j = 0; j < GW; ++j)
+      if (j < ncols) load16_to_lds(bp + (int64_t)cols[j] * (BS * 2), st + G_BOFF + j * TILE);
+  };
+
+  f32x16 acc[2][2][2];  // [slot][32-row half][32-column half]
+#pragma unroll
+  for (int k = 0; k < 2; ++k)
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[k][a][b][v] = 0.f;
+
+  issue_loads(0, 0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  for (int step = 0; step < nsteps; ++step) {
+    const int stage = step & 1;
+    if (step + 1 < nsteps) issue_loads(step + 1, stage ^ 1);
+    if (act[0]) {
+      const char* st = smem + stage * G_STAGE;
+      // units u = 4*slot + ks; the fragments of unit u+1 are read before the MFMAs of unit u.  Slot 1's
+      // first fragments are read whether it is active or not (its tile indices are valid either way).
+      u32x4 af[2][2], bf[2][2];
+      auto read_unit = [&](int u) {
+        const int k = u / 4, ks = u % 4;
+        const char* at = st + my_r[k] * TILE;
+        const char* bt = st + G_BOFF + my_j[k] * TILE;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          af[u & 1][h] = *reinterpret_cast<const u32x4*>(at + a_off[ks] + h * 32 * 128);
+          const char* p = bt + (b_off[ks] ^ (h * 64));
+          const u32x2 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * 128);
+          bf[u & 1][h] = u32x4{lo.x, lo.y, hi.x, hi.y};
+        }
+      };
+      auto mfma_unit = [&](auto k_c, int u) {
+        constexpr int k = decltype(k_c)::value;
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+          for (int nt = 0; nt < 2; ++nt) acc[k][mt][nt] = T::mfma32(af[u & 1][mt], bf[u & 1][nt], acc[k][mt][nt]);
+      };
+      read_unit(0);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        read_unit(u + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_unit(std::integral_constant<int, 0>{}, u);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (act[1]) {
+#pragma unroll
+        for (int u = 4; u < 8; ++u) {
+          if (u + 1 < 8) read_unit(u + 1);
+          __builtin_amdgcn_sched_barrier(0);
+          mfma_unit(std::integral_constant<int, 1>{}, u);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+
+  // ---- epilogue ---------------------------------------------------------------------------------------
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    if (!act[k]) continue;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int64_t m = (int64_t)(rb0 + my_r[k]) * BS + mt * 32 + 8 * (v / 4) + 4 * (lane / 32) + (v % 4);
+          const int64_t n = (int64_t)my_c[k] * BS + nt * 32 + (lane % 32);
+          g.c[m * g.c_sr + n] = T::from_float(acc[k][mt][nt][v] * g.scale);
+        }
+  }
+}
+
 bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
 
 template <typename T, bool TRANS, bool CM>
@@ -579,6 +838,22 @@ int launch_sdd(const GemmArgs& g, hipStream_t stream) {
   return check_launch("sdd_kernel");
 }
 
+template <typename T>
+int launch_sdd_group(const GemmArgs& g, hipStream_t stream) {
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sdd_group_kernel<T>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, G_SMEM);
+    if (e != hipSuccess) return fail(SD_ERR_RUNTIME, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  const int Mb = (int)(g.M / BS), Cb = (int)(g.N / BS);
+  const int tiles_m = (Mb + R - 1) / R, gmax = (Cb + R - 1) / R;
+  hipLaunchKernelGGL(sdd_group_kernel<T>, dim3((unsigned)(tiles_m * gmax)), dim3(THREADS), G_SMEM, stream, g,
+                     tiles_m, gmax, Mb, Cb);
+  return check_launch("sdd_group_kernel");
+}
+
 int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
   if (g.row_ptr && g.bs != BS) return SD_ERR_UNSUPPORTED;
   const bool layout_ok = g.a.sc == 1 && g.b.sr == 1 && g.b.sc != 1 && g.c_sc == 1;
@@ -587,6 +862,12 @@ int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
                         g.b.sc % 8 == 0 && g.c_sr % 8 == 0;
   const int64_t tiles = ((g.M / BS + R - 1) / R) * ((g.N / BS + R - 1) / R);
   if (!layout_ok || !shape_ok || !align_ok || tiles > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
+  static const bool no_groups = [] {
+    const char* e = std::getenv("SPARSEDROP_SDD_PATCH");
+    return e && e[0] == '1';
+  }();
+  if (g.row_ptr && !no_groups && g.N / BS <= G_MAX_CB)
+    return dtype == SD_BF16 ? launch_sdd_group<BF16>(g, stream) : launch_sdd_group<F16>(g, stream);
   return dtype == SD_BF16 ? launch_sdd<BF16>(g, stream) : launch_sdd<F16>(g, stream);
 }
 
