@@ -29,14 +29,9 @@
 // its contiguous index.
 //
 // ---- SDD (the input gradient dX = s*(dY.W) (.) keep) ----------------------------------------------
-// A workgroup owns a 4x4 patch of 64x64 output tiles and computes only the kept ones; the reduction
-// (over N) is dense.  Per 64-wide reduction step it loads the dY tiles of the row blocks that have
-// anything kept in the patch (reduction-contiguous, swizzled as in the forward) and the W tiles of the
-// column blocks that have anything kept (reduction-strided, read with ds_read_b64_tr_b16 as in dW).
-// Waves are (32x32 quadrant of every tile = wave%4) x (row-block pair = wave/4), so the two waves of a
-// SIMD together issue 4 MFMAs per kept tile per step: MFMA work follows the kept count and stays
-// balanced over the SIMDs.  Dropped tiles of the patch are written as zeros by the same workgroup.
-#include <cstdlib>
+// Only kept output tiles are computed; the reduction (over N) is dense.  dY tiles are reduction-contiguous
+// (swizzled as in the forward), W tiles reduction-strided (read with ds_read_b64_tr_b16 as in dW).  See
+// sdd_group_kernel for how tiles are grouped into workgroups; dropped tiles are written as zeros.
 #include <type_traits>
 
 #include "common.h"
@@ -369,184 +364,12 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
   }
 }
 
-// A = dY [M, red] reduction-contiguous; B = W^T [cols, red] given with the reduction index strided
-// (b.sr == 1); C row-major.  Mb x Cb is the block grid of the output (and of the mask).
-template <typename T>
-__global__ __launch_bounds__(THREADS) void sdd_kernel(GemmArgs g, int tiles_m, int tiles_n, int Mb,
-                                                      int Cb) {
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  uint32_t* kept_p = reinterpret_cast<uint32_t*>(smem + 2 * STAGE);
-
-  int tm, tn;
-  tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn);
-  const int tid = threadIdx.x;
-  const int lane = tid % 64;
-  const int wave = tid / 64;
-  const int quad = wave % 4, mq = quad / 2, nq = quad % 2;
-  const int rh = wave / 4;
-  const int rb0 = tm * R, cb0 = tn * R;
-
-  // ---- which of the 16 tiles are kept: bit r*4 + c ------------------------------------------------
-  if (tid == 0) *kept_p = 0;
-  __syncthreads();
-  if (wave < R && rb0 + wave < Mb) {
-    uint32_t bits = 0;
-    if (g.row_ptr) {
-      const int beg = g.row_ptr[rb0 + wave], end = g.row_ptr[rb0 + wave + 1];
-      for (int i = beg + lane; i < end; i += 64) {
-        const int c = g.col_idx[i] - cb0;
-        if (c >= 0 && c < R) bits |= 1u << (wave * 4 + c);
-      }
-    } else if (lane < R && cb0 + lane < Cb) {  // no list: a dense product in this operand layout
-      bits = 1u << (wave * 4 + lane);
-    }
-    if (bits) atomicOr(kept_p, bits);
-  }
-  __syncthreads();
-  const uint32_t kept = *kept_p;
-  uint32_t rowmask = 0, colmask = 0;  // row / column blocks with anything kept
-#pragma unroll
-  for (int r = 0; r < R; ++r)
-    if ((kept >> (4 * r)) & 0xfu) rowmask |= 1u << r;
-#pragma unroll
-  for (int c = 0; c < R; ++c)
-    if (kept & (0x1111u << c)) colmask |= 1u << c;
-
-  // ---- zeros for the dropped tiles of the patch ---------------------------------------------------
-  {
-    const int row = tid / 8, ch = tid % 8;
-    const u32x4 z = {0u, 0u, 0u, 0u};
-    for (int r = 0; r < R; ++r) {
-      if (rb0 + r >= Mb) break;
-      for (int c = 0; c < R; ++c) {
-        if (cb0 + c >= Cb) break;
-        if (!((kept >> (4 * r + c)) & 1u))
-          *reinterpret_cast<u32x4*>(g.c + ((int64_t)(rb0 + r) * BS + row) * g.c_sr +
-                                    (int64_t)(cb0 + c) * BS + ch * 8) = z;
-      }
-    }
-  }
-  if (kept == 0) return;
-
-  // ---- per-lane constants ---------------------------------------------------------------------
-  int a_off[4], b_off[4];
-  {
-    const int fr_sw = (lane >> 1) & 7;
-    const int b4 = lane / 16, e = (lane % 16) / 4, j = lane % 4;
-    const int row = 8 * (b4 / 2) + e;
-    const int b_ch = (nq * 4 + 2 * (b4 % 2) + j / 2) ^ (((e >> 1) & 1) << 2);
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      a_off[ks] = (mq * 32 + lane % 32) * 128 + ((2 * ks + lane / 32) ^ fr_sw) * 16;
-      b_off[ks] = (16 * ks + row) * 128 + b_ch * 16 + (j % 2) * 8;
-    }
-  }
-
-  const int nsteps = (int)(g.K / BS);
-  // per-lane source pointers of the wave's 1 KiB of a tile at reduction step 0
-  const char* a_ptr0;
-  const char* b_ptr0;
-  {
-    const int row = wave * 8 + lane / 8;
-    const int pch = lane % 8;
-    // dY tiles: [64 rows][64 red], chunk swizzle (row>>1)&7
-    a_ptr0 = reinterpret_cast<const char*>(g.a.ptr + ((int64_t)rb0 * BS + row) * g.a.sr +
-                                           (pch ^ ((row >> 1) & 7)) * 8);
-    // W tiles: [64 red][64 cols], chunk swizzle ((red>>1)&1)<<2
-    b_ptr0 = reinterpret_cast<const char*>(g.b.ptr + (int64_t)cb0 * BS + (int64_t)row * g.b.sc +
-                                           (pch ^ (((row >> 1) & 1) << 2)) * 8);
-  }
-  const uint32_t a_tile_stride = (uint32_t)(BS * g.a.sr) * 2u;
-  const int64_t b_step_stride = (int64_t)BS * g.b.sc * 2;
-  auto issue_loads = [&](int step, int stage) {
-    char* st = smem + stage * STAGE + wave * 1024;
-    const char* ap = a_ptr0 + step * (BS * 2);
-    const char* bp = b_ptr0 + step * b_step_stride;
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-      if (rowmask & (1u << r)) load16_to_lds(ap + r * a_tile_stride, st + r * TILE);
-#pragma unroll
-    for (int c = 0; c < R; ++c)
-      if (colmask & (1u << c)) load16_to_lds(bp + c * (BS * 2), st + A_OFF + c * TILE);
-  };
-
-  f32x16 acc[2][R];
-#pragma unroll
-  for (int a = 0; a < 2; ++a)
-#pragma unroll
-    for (int c = 0; c < R; ++c)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[a][c][v] = 0.f;
-
-  const uint32_t mine = (kept >> (8 * rh)) & 0xffu;  // bit rr*4 + c
-  const uint32_t mycols = (mine | (mine >> 4)) & 0xfu;
-
-  issue_loads(0, 0);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-
-  for (int step = 0; step < nsteps; ++step) {
-    const int stage = step & 1;
-    if (step + 1 < nsteps) issue_loads(step + 1, stage ^ 1);
-    if (mine) {
-      const char* st = smem + stage * STAGE;
-      // this wave's 32-row slice of the dY tiles of its two row blocks, all four 16-wide sub-steps.
-      // Every fragment read of the step is unconditional (tiles that were not loaded give unused
-      // garbage): a read under a branch would make the compiler's LDS wait counts imprecise and every
-      // MFMA below would wait for all reads in flight instead of just its own operands.
-      u32x4 af[2][4];
-#pragma unroll
-      for (int rr = 0; rr < 2; ++rr) {
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
-          af[rr][ks] = *reinterpret_cast<const u32x4*>(st + (2 * rh + rr) * TILE + a_off[ks]);
-      }
-      // W fragments of column block c+1 are read before the MFMAs of column block c
-      u32x4 bf[2][4];
-      auto read_b = [&](int c) {
-        const char* bt = st + A_OFF + c * TILE;
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-          const u32x2 lo = lds_read_tr(bt + b_off[ks]), hi = lds_read_tr(bt + b_off[ks] + 4 * 128);
-          bf[c & 1][ks] = u32x4{lo.x, lo.y, hi.x, hi.y};
-        }
-      };
-      read_b(0);
-#pragma unroll
-      for (int c = 0; c < R; ++c) {
-        if (c + 1 < R) read_b(c + 1);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int rr = 0; rr < 2; ++rr)
-          if (mine & (1u << (4 * rr + c))) {
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) acc[rr][c] = T::mfma32(af[rr][ks], bf[c & 1][ks], acc[rr][c]);
-          }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-  }
-
-  // ---- epilogue -----------------------------------------------------------------------------------
-#pragma unroll
-  for (int rr = 0; rr < 2; ++rr)
-#pragma unroll
-    for (int c = 0; c < R; ++c) {
-      if (!(mine & (1u << (4 * rr + c)))) continue;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int64_t m = (int64_t)(rb0 + 2 * rh + rr) * BS + mq * 32 + 8 * (v / 4) + 4 * (lane / 32) + (v % 4);
-        const int64_t n = (int64_t)(cb0 + c) * BS + nq * 32 + (lane % 32);
-        g.c[m * g.c_sr + n] = T::from_float(acc[rr][c][v] * g.scale);
-      }
-    }
-}
-
 // ---- SDD with column groups ---------------------------------------------------------------------------
-// With half of the tiles dropped a 4x4 patch still needs nearly all of its 4 + 4 operand tiles per
-// reduction step for about 8 kept tiles.  Here a workgroup owns 4 row blocks x a GROUP of consecutive
+// A = dY [M, red] reduction-contiguous; B = W^T [cols, red] given with the reduction index strided
+// (b.sr == 1); C row-major.  Mb x Cb is the block grid of the output (and of the mask); without a list
+// every tile is kept (the dense product in this operand layout).
+// With half of the tiles dropped a fixed 4x4 patch of tiles would still need nearly all of its 4 + 4 operand
+// tiles per reduction step for about 8 kept tiles.  Here a workgroup owns 4 row blocks x a GROUP of consecutive
 // column blocks, chosen greedily along the row so that it has at most GW column blocks with anything
 // kept and at most 16 kept tiles: 4 + 6 operand tiles per step for about 12 kept tiles at p = 0.5, the
 // same 4 + 4 for 16 as the patch kernel at p = 0.  Column blocks with nothing kept in these 4 rows
@@ -823,22 +646,6 @@ int launch_dsd(const GemmArgs& g, int splits, hipStream_t stream) {
 }
 
 template <typename T>
-int launch_sdd(const GemmArgs& g, hipStream_t stream) {
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sdd_kernel<T>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
-    if (e != hipSuccess) return fail(SD_ERR_RUNTIME, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
-  const int Mb = (int)(g.M / BS), Cb = (int)(g.N / BS);
-  const int tiles_m = (Mb + R - 1) / R, tiles_n = (Cb + R - 1) / R;
-  hipLaunchKernelGGL(sdd_kernel<T>, dim3((unsigned)(tiles_m * tiles_n)), dim3(THREADS), SMEM_BYTES,
-                     stream, g, tiles_m, tiles_n, Mb, Cb);
-  return check_launch("sdd_kernel");
-}
-
-template <typename T>
 int launch_sdd_group(const GemmArgs& g, hipStream_t stream) {
   static bool configured = false;
   if (!configured) {
@@ -862,13 +669,8 @@ int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
                         g.b.sc % 8 == 0 && g.c_sr % 8 == 0;
   const int64_t tiles = ((g.M / BS + R - 1) / R) * ((g.N / BS + R - 1) / R);
   if (!layout_ok || !shape_ok || !align_ok || tiles > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
-  static const bool no_groups = [] {
-    const char* e = std::getenv("SPARSEDROP_SDD_PATCH");
-    return e && e[0] == '1';
-  }();
-  if (g.row_ptr && !no_groups && g.N / BS <= G_MAX_CB)
-    return dtype == SD_BF16 ? launch_sdd_group<BF16>(g, stream) : launch_sdd_group<F16>(g, stream);
-  return dtype == SD_BF16 ? launch_sdd<BF16>(g, stream) : launch_sdd<F16>(g, stream);
+  if (g.N / BS > G_MAX_CB) return SD_ERR_UNSUPPORTED;
+  return dtype == SD_BF16 ? launch_sdd_group<BF16>(g, stream) : launch_sdd_group<F16>(g, stream);
 }
 
 }  // namespace
