@@ -266,3 +266,51 @@ def test_full_size_8192_sampled_against_oracle(p):
         ext = GEMM()
         assert rel_fro(C, ext.gemm(A, B).float()) <= 1e-3
         assert rel_fro(dA, ext.gemm(dC, B.T).float()) <= 1e-3
+
+
+def _structured_masks(mb, cb, gen):
+    """Masks that steer the grouped SDD kernel through its branches: groups cut by the 6-active-column
+    limit, by the 16-kept-tile limit, long runs of all-dropped columns, single tiles, ragged row quads."""
+    masks = {}
+    for p in (0.05, 0.3, 0.9, 0.97):
+        masks[f"bernoulli_{p}"] = cpu_mask((mb, cb), p, gen)
+    m = torch.ones(mb, cb, dtype=torch.bool)
+    m[:, ::2] = False
+    masks["every_other_column_kept"] = m            # 4 kept per active column: cut at 16 tiles
+    m = torch.ones(mb, cb, dtype=torch.bool)
+    m[::4, :] = False
+    masks["one_row_of_each_quad_kept"] = m          # 1 kept per column: cut at 6 active columns
+    m = torch.ones(mb, cb, dtype=torch.bool)
+    m[0, 0] = False
+    masks["single_first_tile"] = m
+    m = torch.ones(mb, cb, dtype=torch.bool)
+    m[mb - 1, cb - 1] = False
+    masks["single_last_tile"] = m
+    m = torch.ones(mb, cb, dtype=torch.bool)
+    m[:, cb - 1] = False
+    masks["last_column_only"] = m
+    m = torch.zeros(mb, cb, dtype=torch.bool)
+    m[:, 3: cb - 2] = True
+    masks["gap_in_the_middle"] = m
+    masks["all_dropped"] = torch.ones(mb, cb, dtype=torch.bool)
+    masks["none_dropped"] = torch.zeros(mb, cb, dtype=torch.bool)
+    return masks
+
+
+@pytest.mark.parametrize("M,N,K", [(576, 256, 1216), (256, 128, 4480)])
+def test_sdd_column_groups(M, N, K):
+    """dX = (dY . W) (.) keep on shapes whose block grid is not a multiple of the 4-row quads (9 row blocks)
+    or of any group width (19 / 70 column blocks), under structured masks."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(11)
+    dC = make_operand(M, N, torch.float16, "cuda", gen=gen)
+    B = make_operand(N, K, torch.float16, "cuda", scale=N ** -0.5, gen=gen)
+    dc, b = to_np(dC), to_np(B)
+    for name, mk in _structured_masks(M // 64, K // 64, gen).items():
+        got = ext.gemm_sdd(dC, B.T, mk.cuda(), 64, 2.0)
+        ref = O.gemm_sdd(dc, b.T, mk.numpy(), 64, 2.0, np.float32)
+        assert rel_fro(got, ref) <= REL_FRO_TOL, name
+        keep = O.expand_keep(mk.numpy(), 64, M, K)
+        assert (got.cpu().numpy()[~keep] == 0).all(), name
