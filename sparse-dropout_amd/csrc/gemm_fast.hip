@@ -69,6 +69,16 @@ __device__ inline void load16_to_lds(const void* g, char* lds_dst) {
   const uint32_t a = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_void*)lds_dst);
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(a) : "memory");
 }
+// The same with the address split into a wave-uniform 64-bit base (SGPRs) and a 32-bit per-lane byte
+// offset: half the VGPR reads per load and no 64-bit VALU add to form the lane addresses.
+__device__ inline void load16_to_lds(const char* base, uint32_t lane_off, char* lds_dst) {
+  const uint64_t b = (uint64_t)(uintptr_t)base;
+  const uint64_t sb = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32)) << 32) |
+                      (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+  const uint32_t a = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_void*)lds_dst);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(sb), "s"(a)
+               : "memory");
+}
 
 // Maps the launch index to an output tile so that the workgroups resident on one XCD (the hardware
 // deals consecutive workgroup ids round-robin over the 8 XCDs, each with its own L2) cover a compact
@@ -244,10 +254,10 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
     const char* ap = a_tile0 + kb * red_stride;
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj)
-      if (b_valid[jj]) load16_to_lds(bp + b_lane[jj], st + (wave * 4 + jj) * 1024);
+      if (b_valid[jj]) load16_to_lds(bp, b_lane[jj], st + (wave * 4 + jj) * 1024);
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      if (fl & (1u << r)) load16_to_lds(ap + r * a_rstride + a_lane, st + A_OFF + r * TILE + wave * 1024);
+      if (fl & (1u << r)) load16_to_lds(ap + r * a_rstride, a_lane, st + A_OFF + r * TILE + wave * 1024);
   };
 
   f32x16 acc[2][2][2];  // [row block of the pair][m tile][n tile]
@@ -291,7 +301,7 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
   // (MINE = 1, 2 or 3).  The work is a chain of units (row block, ks); the LDS reads of unit u+1 are
   // issued before the MFMAs of unit u so that their latency hides behind 4 MFMAs (128 cycles).  The W
   // fragments are read during the first row block's units and stay in registers for the second.
-  auto compute = [&](auto mine_c, const char* st) {
+  auto compute = [&](auto mine_c, const char* st, bool mid_loads, uint32_t mid_entry, int mid_stage) {
     constexpr int MINE = decltype(mine_c)::value;
     constexpr int NR = (MINE == 3) ? 2 : 1;
     constexpr int R0 = (MINE == 2) ? 1 : 0;
@@ -316,11 +326,13 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
           acc[rr][mt][nt] = CM ? T::mfma32(bf[nt][ks], af[u & 1][mt], acc[rr][mt][nt])
                                : T::mfma32(af[u & 1][mt], bf[nt][ks], acc[rr][mt][nt]);
       __builtin_amdgcn_sched_barrier(0);
+      if (u == NR * 2 - 1 && mid_loads) issue_loads(mid_entry, mid_stage);
     }
   };
 
   // Table words are read two steps ahead into a VGPR and made uniform a step later, when the read has
   // long returned: a read-and-wait at the top of a step would put an LDS round trip in front of its MFMAs.
+  const bool late = __builtin_amdgcn_readfirstlane(rh) != 0;
   uint32_t e_cur = uniform(step_e[0]), e_next = uniform(step_e[1]);
   if (nsteps > 0) issue_loads(e_cur, 0);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -329,12 +341,14 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
   for (int step = 0; step < nsteps; ++step) {
     const int stage = step & 1;
     const uint32_t e_after = step_e[step + 2];
-    if (step + 1 < nsteps) issue_loads(e_next, stage ^ 1);
+    const bool more = step + 1 < nsteps;
     const uint32_t mine = (step_flags(e_cur) >> (2 * rh)) & 3u;
+    const bool mid = late && more && mine != 0u;
+    if (more && !mid) issue_loads(e_next, stage ^ 1);
     const char* st = smem + stage * STAGE;
-    if (mine == 3u) compute(std::integral_constant<int, 3>{}, st);
-    else if (mine == 1u) compute(std::integral_constant<int, 1>{}, st);
-    else if (mine == 2u) compute(std::integral_constant<int, 2>{}, st);
+    if (mine == 3u) compute(std::integral_constant<int, 3>{}, st, mid, e_next, stage ^ 1);
+    else if (mine == 1u) compute(std::integral_constant<int, 1>{}, st, mid, e_next, stage ^ 1);
+    else if (mine == 2u) compute(std::integral_constant<int, 2>{}, st, mid, e_next, stage ^ 1);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     e_cur = e_next;
@@ -525,29 +539,31 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
     }
   }
   const int nsteps = (int)(g.K / BS);
-  const char* a_ptr0;
-  const char* b_ptr0;
+  // loads: wave-uniform tile bases plus this lane's 16 bytes of the wave's 8 tile rows
+  const char* a_base = reinterpret_cast<const char*>(g.a.ptr + (int64_t)rb0 * BS * g.a.sr);
+  const char* b_base = reinterpret_cast<const char*>(g.b.ptr);
+  uint32_t a_lane, b_lane;
   {
     const int row = wave * 8 + lane / 8;
     const int pch = lane % 8;
-    a_ptr0 = reinterpret_cast<const char*>(g.a.ptr + ((int64_t)rb0 * BS + row) * g.a.sr +
-                                           (pch ^ ((row >> 1) & 7)) * 8);
-    b_ptr0 = reinterpret_cast<const char*>(g.b.ptr + (int64_t)row * g.b.sc +
-                                           (pch ^ (((row >> 1) & 1) << 2)) * 8);
+    a_lane = (uint32_t)(row * g.a.sr + (pch ^ ((row >> 1) & 7)) * 8) * 2u;
+    b_lane = (uint32_t)(row * g.b.sc + (pch ^ (((row >> 1) & 1) << 2)) * 8) * 2u;
   }
-  const uint32_t a_tile_stride = (uint32_t)(BS * g.a.sr) * 2u;
+  const int64_t a_tile_stride = (int64_t)BS * g.a.sr * 2;
   const int64_t b_step_stride = (int64_t)BS * g.b.sc * 2;
   auto issue_loads = [&](int step, int stage) {
     char* st = smem + stage * G_STAGE + wave * 1024;
-    const char* ap = a_ptr0 + step * (BS * 2);
-    const char* bp = b_ptr0 + step * b_step_stride;
+    const char* ap = a_base + step * (BS * 2);
+    const char* bp = b_base + step * b_step_stride;
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      if (rowmask & (1u << r)) load16_to_lds(ap + r * a_tile_stride, st + r * TILE);
+      if (rowmask & (1u << r)) load16_to_lds(ap + r * a_tile_stride, a_lane, st + r * TILE);
 #pragma unroll
     for (int j = 0; j < GW; ++j)
-      if (j < ncols) load16_to_lds(bp + (int64_t)cols[j] * (BS * 2), st + G_BOFF + j * TILE);
+      if (j < ncols) load16_to_lds(bp + (int64_t)cols[j] * (BS * 2), b_lane, st + G_BOFF + j * TILE);
   };
+  // the two waves of a SIMD (w and w + 4) issue their loads half a step apart
+  const bool late = wave >= 4;
 
   f32x16 acc[2][2][2];  // [slot][32-row half][32-column half]
 #pragma unroll
@@ -565,7 +581,9 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
 
   for (int step = 0; step < nsteps; ++step) {
     const int stage = step & 1;
-    if (step + 1 < nsteps) issue_loads(step + 1, stage ^ 1);
+    const bool more = step + 1 < nsteps;
+    const bool mid = late && more && act[0];
+    if (more && !mid) issue_loads(step + 1, stage ^ 1);
     if (act[0]) {
       const char* st = smem + stage * G_STAGE;
       // units u = 4*slot + ks; the fragments of unit u+1 are read before the MFMAs of unit u.  Slot 1's
@@ -597,6 +615,7 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
         __builtin_amdgcn_sched_barrier(0);
         mfma_unit(std::integral_constant<int, 0>{}, u);
         __builtin_amdgcn_sched_barrier(0);
+        if (u == 1 && mid) issue_loads(step + 1, stage ^ 1);
       }
       if (act[1]) {
 #pragma unroll
@@ -670,7 +689,8 @@ int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
   const bool layout_ok = g.a.sc == 1 && g.b.sr == 1 && g.b.sc != 1 && g.c_sc == 1;
   const bool shape_ok = g.M > 0 && g.M % BS == 0 && g.N > 0 && g.N % BS == 0 && g.K > 0 && g.K % BS == 0;
   const bool align_ok = aligned16(g.a.ptr) && aligned16(g.b.ptr) && aligned16(g.c) && g.a.sr % 8 == 0 &&
-                        g.b.sc % 8 == 0 && g.c_sr % 8 == 0;
+                        g.b.sc % 8 == 0 && g.c_sr % 8 == 0 && g.a.sr < (1 << 22) &&
+                        g.b.sc < (1 << 22);  // per-lane byte offsets are 32-bit
   const int64_t tiles = ((g.M / BS + R - 1) / R) * ((g.N / BS + R - 1) / R);
   if (!layout_ok || !shape_ok || !align_ok || tiles > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
   if (g.N / BS > G_MAX_CB) return SD_ERR_UNSUPPORTED;
