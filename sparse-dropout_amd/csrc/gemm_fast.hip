@@ -650,15 +650,26 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
 
 bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
 
+// Raises a kernel's dynamic LDS limit once per device (the attribute belongs to the device's copy of the
+// kernel); `done` is the caller's per-kernel record.
+constexpr int kMaxDevices = 64;
+int allow_big_lds(const void* kernel, int bytes, bool (&done)[kMaxDevices]) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return fail(SD_ERR_RUNTIME, "hipGetDevice failed or device index out of range");
+  if (!done[dev]) {
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return fail(SD_ERR_RUNTIME, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    done[dev] = true;
+  }
+  return SD_OK;
+}
+
 template <typename T, bool TRANS, bool CM>
 int launch_dsd(const GemmArgs& g, int splits, hipStream_t stream) {
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dsd_kernel<T, TRANS, CM>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
-    if (e != hipSuccess) return fail(SD_ERR_RUNTIME, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static bool configured[kMaxDevices] = {};
+  if (int rc = allow_big_lds(reinterpret_cast<const void*>(&dsd_kernel<T, TRANS, CM>), SMEM_BYTES, configured))
+    return rc;
   const int Mb = (int)(g.M / BS), Kb = (int)(g.K / BS);
   const int tiles_m = (Mb + R - 1) / R, tiles_n = (int)((g.N + BN - 1) / BN);
   hipLaunchKernelGGL((dsd_kernel<T, TRANS, CM>), dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits),
@@ -670,13 +681,8 @@ int launch_dsd(const GemmArgs& g, int splits, hipStream_t stream) {
 
 template <typename T>
 int launch_sdd_group(const GemmArgs& g, hipStream_t stream) {
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sdd_group_kernel<T>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, G_SMEM);
-    if (e != hipSuccess) return fail(SD_ERR_RUNTIME, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static bool configured[kMaxDevices] = {};
+  if (int rc = allow_big_lds(reinterpret_cast<const void*>(&sdd_group_kernel<T>), G_SMEM, configured)) return rc;
   const int Mb = (int)(g.M / BS), Cb = (int)(g.N / BS);
   const int tiles_m = (Mb + R - 1) / R, gmax = (Cb + R - 1) / R;
   hipLaunchKernelGGL(sdd_group_kernel<T>, dim3((unsigned)(tiles_m * gmax)), dim3(THREADS), G_SMEM, stream, g,

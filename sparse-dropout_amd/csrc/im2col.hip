@@ -261,7 +261,7 @@ __global__ __launch_bounds__(256) void col2im_kernel(const uint16_t* __restrict_
 // with zeros instead of being read), then each thread sums the taps of its outputs out of LDS.  Global
 // reads are whole segments instead of one 2-byte element per lane and cache line.
 constexpr int C2I_CG = 8;
-constexpr int C2I_MAX_LDS = 64 * 1024;
+constexpr int C2I_MAX_LDS = 60 * 1024;  // below the 64 KB a kernel gets without asking
 
 template <typename T>
 __global__ __launch_bounds__(256) void col2im_tile_kernel(const uint16_t* __restrict__ cols, int64_t ld,
