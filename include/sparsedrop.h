@@ -98,6 +98,16 @@ int sd_random_lists(uint64_t seed, uint64_t offset, float p, int64_t mb, int64_t
                     int64_t split, int64_t out_mb, int64_t out_kb, int32_t* row_ptr, int32_t* col_idx,
                     int32_t* col_ptr, int32_t* row_idx, void* stream);
 
+/* The same draw keyed by device memory: state is a device pointer to {seed, offset} (two uint64); the
+ * kernels read both from there and a trailing one-thread kernel adds 1 to the offset, all on `stream`.
+ * Nothing about the draw is baked into the launch arguments, so a captured HIP graph that contains this
+ * call draws a new mask at every replay (with sd_random_lists the seed is a launch argument and a replay
+ * would repeat the mask).  The reference has no counterpart: its mask comes from torch.rand on torch's
+ * generator (flash_dropout/functional/utils.py:15), which torch itself makes graph-safe the same way. */
+int sd_random_lists_state(uint64_t* state, float p, int64_t mb, int64_t kb, uint8_t* mask_out, int64_t split,
+                          int64_t out_mb, int64_t out_kb, int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr,
+                          int32_t* row_idx, void* stream);
+
 /* Pointer-increment table of flash_dropout/functional/utils.py:19-69 from a CSR list:
  * table[i] = col_idx[i]*block_k for the first kept block of a row, else (col_idx[i]-col_idx[i-1])*block_k;
  * row_indices[r] = row_ptr[r]; row_widths[r] = row_ptr[r+1]-row_ptr[r].

@@ -53,12 +53,30 @@ MODELS = {
 }
 
 
-def time_model(model: nn.Module, x: torch.Tensor, warmup: float, rep: float) -> list[float]:
-    """fwd+bwd milliseconds per repetition, cache flushed before each (benchmark/model.py:119-142)."""
+def time_model(model: nn.Module, x: torch.Tensor, warmup: float, rep: float, graph: bool = False) -> list[float]:
+    """fwd+bwd milliseconds per repetition, cache flushed before each (benchmark/model.py:119-142).
+    With ``graph`` the step is captured once in a HIP graph and replayed: no Python or launch path in the
+    timed region (block-dropout masks still change from replay to replay, they are drawn from device state)."""
     cache = torch.empty(FLUSH_BYTES, dtype=torch.int8, device="cuda")
 
-    def f():
+    def step():
         model(x).float().square().mean().backward()
+
+    f = step
+    if graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        for prm in model.parameters():
+            prm.grad = None
+        captured = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(captured):
+            step()
+        f = captured.replay
 
     for _ in range(10):
         f()
@@ -84,16 +102,17 @@ def main() -> None:
     ap.add_argument("--p", type=float, nargs="+", default=[0.0, 0.1, 0.3, 0.5, 0.7])
     ap.add_argument("--block-size", type=int, default=64)
     ap.add_argument("--rep", type=float, default=0.3, help="seconds of timed repetitions per point")
+    ap.add_argument("--graph", action="store_true", help="capture the step in a HIP graph and time replays")
     args = ap.parse_args()
     torch.manual_seed(0)
     for name in args.model:
         cls, make_x = MODELS[name]
         x = make_x().cuda().half()
-        print(f"=== {name}  input {tuple(x.shape)}  block_size {args.block_size}")
+        print(f"=== {name}  input {tuple(x.shape)}  block_size {args.block_size}{'  (graph replay)' if args.graph else ''}")
         for variant, ps in (("none", [0.0]), ("vanilla", [0.5]), ("blockwise[hip]", args.p)):
             for p in ps:
                 model = cls(variant, p, args.block_size).cuda().half().train()
-                ts = time_model(model, x, warmup=0.2, rep=args.rep)
+                ts = time_model(model, x, warmup=0.2, rep=args.rep, graph=args.graph)
                 sem = statistics.stdev(ts) / len(ts) ** 0.5 if len(ts) > 1 else 0.0
                 print(f"{variant:<16} p={p:<4} median {statistics.median(ts):8.4f} ms  "
                       f"mean {statistics.mean(ts):8.4f} +- {1.96 * sem:.4f}  n={len(ts)}")

@@ -14,7 +14,7 @@ char* last_error_buf() {
 int build_lists(const uint8_t* mask, int64_t msr, int64_t msc, int64_t stored_kb, int64_t split,
                 int64_t mb, int64_t kb, int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr,
                 int32_t* row_idx, hipStream_t stream);
-int random_lists(uint64_t seed, uint64_t offset, float p, int64_t stored_mb, int64_t stored_kb,
+int random_lists(uint64_t seed, uint64_t offset, uint64_t* state, float p, int64_t stored_mb, int64_t stored_kb,
                  uint8_t* mask_out, int64_t split, int64_t mb, int64_t kb, int32_t* row_ptr,
                  int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx, hipStream_t stream);
 int increment_table(const int32_t* row_ptr, const int32_t* col_idx, int64_t mb, int64_t block_k,
@@ -153,8 +153,19 @@ int sd_random_lists(uint64_t seed, uint64_t offset, float p, int64_t mb, int64_t
   SD_REQUIRE(p >= 0.f && p < 1.f, "random_lists: p must be in [0, 1) (got %g)", (double)p);
   SD_REQUIRE(mask_out != nullptr, "random_lists: null mask_out");
   if (int rc = check_list_grid(mb, kb, split, out_mb, out_kb, row_ptr, col_idx, col_ptr, row_idx)) return rc;
-  return random_lists(seed, offset, p, mb, kb, mask_out, split, out_mb, out_kb, row_ptr, col_idx, col_ptr,
+  return random_lists(seed, offset, nullptr, p, mb, kb, mask_out, split, out_mb, out_kb, row_ptr, col_idx, col_ptr,
                       row_idx, (hipStream_t)stream);
+}
+
+int sd_random_lists_state(uint64_t* state, float p, int64_t mb, int64_t kb, uint8_t* mask_out, int64_t split,
+                          int64_t out_mb, int64_t out_kb, int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr,
+                          int32_t* row_idx, void* stream) {
+  SD_REQUIRE(state != nullptr && reinterpret_cast<uintptr_t>(state) % 8 == 0, "random_lists: state must be an aligned device pointer");
+  SD_REQUIRE(p >= 0.f && p < 1.f, "random_lists: p must be in [0, 1) (got %g)", (double)p);
+  SD_REQUIRE(mask_out != nullptr, "random_lists: null mask_out");
+  if (int rc = check_list_grid(mb, kb, split, out_mb, out_kb, row_ptr, col_idx, col_ptr, row_idx)) return rc;
+  return random_lists(0, 0, state, p, mb, kb, mask_out, split, out_mb, out_kb, row_ptr, col_idx, col_ptr, row_idx,
+                      (hipStream_t)stream);
 }
 
 int sd_increment_table(const int32_t* row_ptr, const int32_t* col_idx, int64_t mb, int64_t block_k,

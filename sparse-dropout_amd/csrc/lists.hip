@@ -51,6 +51,18 @@ struct MaskSrc {
   int32_t kb;  // entries per row of the stored / drawn mask
   uint32_t seed_lo, seed_hi, off_lo, off_hi;
   float p;
+  const uint64_t* state;  // device-resident {seed, offset} that overrides the four words above, or null
+  // Kernels call this once on their copy: a draw keyed by device memory lets a captured graph draw a
+  // fresh mask at every replay (the host bumps nothing; a one-thread kernel advances the offset).
+  __device__ inline void resolve() {
+    if (state) {
+      const uint64_t sd = state[0], off = state[1];
+      seed_lo = (uint32_t)sd;
+      seed_hi = (uint32_t)(sd >> 32);
+      off_lo = (uint32_t)off;
+      off_hi = (uint32_t)(off >> 32);
+    }
+  }
   __device__ inline bool dropped_entry(int32_t si, int32_t sj) const {
     if (mask) return mask[si * st_row + sj * st_col] != 0;
     const uint64_t e = (uint64_t)si * (uint32_t)kb + (uint32_t)sj;
@@ -171,12 +183,14 @@ __global__ __launch_bounds__(kFlatThreads) void build_lists_flat(ListJob job0, L
   int b = blockIdx.x;
   if (b >= blocks0 + blocks1) {  // launched only for a drawn mask: store it for the caller
     const int nb = gridDim.x - blocks0 - blocks1;
+    job0.src.resolve();
     write_mask(job0.src, mask_rows, mask_out, (int64_t)(b - blocks0 - blocks1) * kFlatThreads + tid,
                (int64_t)nb * kFlatThreads);
     return;
   }
   const bool second = b >= blocks0;
-  const ListJob job = second ? job1 : job0;
+  ListJob job = second ? job1 : job0;
+  job.src.resolve();
   if (second) b -= blocks0;
   const int len = (int)job.len;
   const int total_entries = (int)(job.nlines * job.len);
@@ -216,7 +230,11 @@ __global__ __launch_bounds__(kFlatThreads) void build_lists_flat(ListJob job0, L
   if (tid == 0 && f0 + kFlatChunk >= total_entries) job.ptr[job.nlines] = base + chunk_total;
 }
 
+// After every kernel of a draw has read the state: the next draw gets the next offset.
+__global__ void advance_state_kernel(uint64_t* state) { state[1] += 1; }
+
 __global__ __launch_bounds__(256) void mask_store_kernel(MaskSrc src, int64_t mb, uint8_t* out) {
+  src.resolve();
   write_mask(src, mb, out, (int64_t)blockIdx.x * 256 + threadIdx.x, (int64_t)gridDim.x * 256);
 }
 
@@ -225,9 +243,10 @@ __global__ __launch_bounds__(256) void lists_count(ListJob job0, ListJob job1) {
   const int lane = threadIdx.x % kWave;
   const int64_t w = (int64_t)blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
   const int64_t n0 = job0.ptr ? job0.nlines : 0;
-  const ListJob job = (w < n0) ? job0 : job1;
+  ListJob job = (w < n0) ? job0 : job1;
   const int64_t line = (w < n0) ? w : w - n0;
   if (job.ptr == nullptr || line >= job.nlines) return;
+  job.src.resolve();
   int c = wave_count_kept(job, line, lane);
   if (lane == 0) job.ptr[1 + line] = c;
 }
@@ -243,9 +262,10 @@ __global__ __launch_bounds__(256) void lists_fill(ListJob job0, ListJob job1) {
   const int lane = threadIdx.x % kWave;
   const int64_t w = (int64_t)blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
   const int64_t n0 = job0.ptr ? job0.nlines : 0;
-  const ListJob job = (w < n0) ? job0 : job1;
+  ListJob job = (w < n0) ? job0 : job1;
   const int64_t line = (w < n0) ? w : w - n0;
   if (job.ptr == nullptr || line >= job.nlines) return;
+  job.src.resolve();
   wave_fill_kept(job, line, lane, job.idx + job.ptr[line]);
 }
 
@@ -304,17 +324,22 @@ static int launch_lists(const MaskSrc& src, int64_t mb, int64_t kb, int32_t* row
 int build_lists(const uint8_t* mask, int64_t msr, int64_t msc, int64_t stored_kb, int64_t split,
                 int64_t mb, int64_t kb, int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr,
                 int32_t* row_idx, hipStream_t stream) {
-  MaskSrc src{mask, msr, msc, (int32_t)split, (int32_t)stored_kb, 0, 0, 0, 0, 0.f};
+  MaskSrc src{mask, msr, msc, (int32_t)split, (int32_t)stored_kb, 0, 0, 0, 0, 0.f, nullptr};
   return launch_lists(src, mb, kb, row_ptr, col_idx, col_ptr, row_idx, nullptr, 0, stream);
 }
 
 // Same with the mask drawn on the device; it is also stored to mask_out ([stored_mb, stored_kb] bytes).
-int random_lists(uint64_t seed, uint64_t offset, float p, int64_t stored_mb, int64_t stored_kb,
+int random_lists(uint64_t seed, uint64_t offset, uint64_t* state, float p, int64_t stored_mb, int64_t stored_kb,
                  uint8_t* mask_out, int64_t split, int64_t mb, int64_t kb, int32_t* row_ptr,
                  int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx, hipStream_t stream) {
   MaskSrc src{nullptr, 0, 0, (int32_t)split, (int32_t)stored_kb, (uint32_t)seed, (uint32_t)(seed >> 32),
-              (uint32_t)offset, (uint32_t)(offset >> 32), p};
-  return launch_lists(src, mb, kb, row_ptr, col_idx, col_ptr, row_idx, mask_out, stored_mb, stream);
+              (uint32_t)offset, (uint32_t)(offset >> 32), p, state};
+  if (int rc = launch_lists(src, mb, kb, row_ptr, col_idx, col_ptr, row_idx, mask_out, stored_mb, stream)) return rc;
+  if (state) {
+    hipLaunchKernelGGL(advance_state_kernel, dim3(1), dim3(1), 0, stream, state);
+    return check_launch("advance_state");
+  }
+  return SD_OK;
 }
 
 int increment_table(const int32_t* row_ptr, const int32_t* col_idx, int64_t mb, int64_t block_k,

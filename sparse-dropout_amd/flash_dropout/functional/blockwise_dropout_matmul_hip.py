@@ -92,8 +92,10 @@ def blockwise_dropout_matmul(input: torch.Tensor, weight: torch.Tensor, block_si
     """``(keep ⊙ input)/(1-p) @ weight.T`` with a fresh block mask (reference: …_cuda.py:56-59).
 
     The mask is drawn on the device inside the list-building launch; ``seed`` pins it (the same mask
-    comes back from ``GEMM().random_lists(mask_shape, p, seed)``), otherwise a seed is taken from
-    torch's default generator."""
+    comes back from ``GEMM().random_lists(mask_shape, p, seed)``), otherwise it comes from the
+    device-resident generator state, which starts at ``torch.initial_seed()`` and advances by one per
+    call on the stream: nothing about the draw is a launch argument, so a captured graph draws a new
+    mask at every replay."""
     if not 0 <= p < 1:
         raise ValueError("Dropout probability must be in [0, 1)")
     bs = _block_size(block_size)

@@ -25,6 +25,8 @@ SIGNATURES = {
                                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sd_random_lists": (c_int, [c_uint64, c_uint64, c_float, c_int64, c_int64, c_void_p, c_int64, c_int64,
                                 c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sd_random_lists_state": (c_int, [c_void_p, c_float, c_int64, c_int64, c_void_p, c_int64, c_int64,
+                                      c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sd_increment_table": (c_int, [c_void_p, c_void_p, c_int64, c_int64,
                                    c_void_p, c_void_p, c_void_p, c_void_p]),
     "sd_splitk_workspace_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int64, c_int]),

@@ -56,6 +56,13 @@ class KeptLists:
 _NO_GUARD = contextlib.nullcontext()
 
 
+def _device(device) -> torch.device:
+    dev = torch.device("cuda") if device is None else torch.device(device)
+    if dev.index is None:
+        dev = torch.device("cuda", torch.cuda.current_device())
+    return dev
+
+
 def _guard(dev: torch.device):
     """Makes ``dev`` the current device for a launch; free when it already is."""
     return _NO_GUARD if dev.index == torch.cuda.current_device() else torch.cuda.device(dev)
@@ -117,6 +124,7 @@ class GEMM:
 
     def __init__(self) -> None:
         self.lib = _loader.load()
+        self._rng: dict[int, tuple[int, torch.Tensor]] = {}  # device index -> (torch seed it follows, state)
 
     # ------------------------------------------------------------------ plumbing
     def _call(self, fn, *args) -> None:
@@ -244,34 +252,60 @@ class GEMM:
                        row_idx.data_ptr(), self._stream(mask))
         return KeptLists(row_ptr, col_idx, col_ptr, row_idx, (out_mb, out_kb))
 
-    def random_lists(self, shape, p: float, seed: int, offset: int = 0, device=None, split: int = 1,
-                     grid=None):
+    def manual_seed(self, seed: int, device=None) -> None:
+        """(Re)starts the device-resident mask generator of ``device`` at (seed, offset 0).  Without this
+        call the generator starts from ``torch.initial_seed()`` at first use and restarts whenever that
+        value changes (``torch.manual_seed`` with a new seed)."""
+        dev = _device(device)
+        seed = int(seed) & (2 ** 64 - 1)
+        as_i64 = seed if seed < 2 ** 63 else seed - 2 ** 64
+        state = torch.tensor([as_i64, 0], dtype=torch.int64, device=dev)
+        self._rng[dev.index] = (torch.initial_seed(), state)
+
+    def rng_state(self, device=None) -> torch.Tensor:
+        """int64[2] device tensor {seed, offset} behind the draws that are given no explicit seed; every
+        such draw advances the offset by one on the stream it runs on.  Create it (one draw, or
+        :meth:`manual_seed`) before capturing a graph: the first use copies the seed from the host."""
+        dev = _device(device)
+        entry = self._rng.get(dev.index)
+        if entry is None or entry[0] != torch.initial_seed():
+            self.manual_seed(torch.initial_seed(), dev)
+            entry = self._rng[dev.index]
+        return entry[1]
+
+    def random_lists(self, shape, p: float, seed: int | None = None, offset: int = 0, device=None,
+                     split: int = 1, grid=None):
         """Draws a Bernoulli(p) block mask of ``shape`` on the device (True = dropped) and lists it in
         the same launch: (mask, lists).  The mask is a pure function of (seed, offset, shape[1]) —
-        Philox4x32-10, one 32-bit word per entry — not torch's generator stream."""
+        Philox4x32-10, one 32-bit word per entry — not torch's generator stream.  With ``seed=None``
+        seed and offset come from the device-resident state (:meth:`rng_state`), which the call
+        advances: the form that survives graph capture."""
         mb, kb = int(shape[0]), int(shape[1])
         if mb <= 0 or kb <= 0:
             raise ValueError("mask must be non-empty")
         if not 0.0 <= p < 1.0:
             raise ValueError(f"p must be in [0, 1), got {p}")
         split, out_mb, out_kb = self._list_grid(mb, kb, split, grid)
-        dev = torch.device("cuda") if device is None else torch.device(device)
-        if dev.index is None:
-            dev = torch.device("cuda", torch.cuda.current_device())
+        dev = _device(device)
+        state = self.rng_state(dev) if seed is None else None
         mask = torch.empty((mb, kb), dtype=torch.bool, device=dev)
         row_ptr, col_ptr, col_idx, row_idx = self._list_buffers(out_mb, out_kb, dev)
+        tail = (mb, kb, mask.data_ptr(), split, out_mb, out_kb, row_ptr.data_ptr(), col_idx.data_ptr(),
+                col_ptr.data_ptr(), row_idx.data_ptr(), self._stream(mask))
         with _guard(dev):
-            self._call(self.lib.sd_random_lists, int(seed) & (2 ** 64 - 1), int(offset) & (2 ** 64 - 1),
-                       float(p), mb, kb, mask.data_ptr(), split, out_mb, out_kb, row_ptr.data_ptr(),
-                       col_idx.data_ptr(), col_ptr.data_ptr(), row_idx.data_ptr(), self._stream(mask))
+            if state is None:
+                self._call(self.lib.sd_random_lists, int(seed) & (2 ** 64 - 1), int(offset) & (2 ** 64 - 1),
+                           float(p), *tail)
+            else:
+                self._call(self.lib.sd_random_lists_state, state.data_ptr(), float(p), *tail)
         return mask, KeptLists(row_ptr, col_idx, col_ptr, row_idx, (out_mb, out_kb))
 
     def kept_lists(self, rows: int, cols: int, block_size, mask: torch.Tensor | None = None,
                    p: float = 0.0, seed: int | None = None, device=None):
         """Lists for a [rows, cols] matrix masked in block_size tiles -> (mask, lists, kernel block size).
 
-        The mask is the given one, or drawn on the device (Bernoulli(p), ``seed`` or a fresh seed from
-        torch's default CPU generator, so ``torch.manual_seed`` makes runs repeatable).  A block size
+        The mask is the given one, or drawn on the device (Bernoulli(p); ``seed`` pins it, otherwise the
+        device-resident generator state is used and advanced, which follows ``torch.manual_seed``).  A block size
         that is a larger multiple of 64 is listed at 64 granularity, which is what the fast kernels
         take: pass the returned block size, not the logical one, to the ``*_lists`` calls."""
         bs = _block_size(block_size)
@@ -280,8 +314,6 @@ class GEMM:
         if bs > 64 and bs % 64 == 0:
             split, grid, kernel_bs = bs // 64, (ceil(rows / 64), ceil(cols / 64)), 64
         if mask is None:
-            if seed is None:
-                seed = int(torch.empty((), dtype=torch.int64).random_().item())
             mask, lists = self.random_lists(shape, p, seed, 0, device, split, grid)
         else:
             if tuple(mask.shape) != shape:

@@ -128,18 +128,83 @@ def test_functional_draws_its_mask_on_the_device(bs, p):
 
 def test_functional_mask_follows_torch_seed():
     import flash_dropout.functional as F
+    from flash_dropout.hip import GEMM
 
     x = torch.ones(256, 256, dtype=torch.float16, device="cuda")
     w = torch.eye(256, dtype=torch.float16, device="cuda")
     torch.manual_seed(3)
     a = F.hip_blockwise_dropout_matmul(x, w, 64, 0.5)
     b = F.hip_blockwise_dropout_matmul(x, w, 64, 0.5)
+    assert not torch.equal(a, b)        # consecutive calls draw different masks
+    torch.manual_seed(4)                # a new torch seed restarts the device generator from it
+    c = F.hip_blockwise_dropout_matmul(x, w, 64, 0.5)
+    assert not torch.equal(a, c)
     torch.manual_seed(3)
     a2 = F.hip_blockwise_dropout_matmul(x, w, 64, 0.5)
-    assert torch.equal(a, a2)           # same seed, same mask
-    assert not torch.equal(a, b)        # consecutive calls draw different masks
-    kept = (a != 0).float().mean().item()
-    assert 0.2 < kept < 0.8
+    assert torch.equal(a, a2)           # same seed, same first mask
+    keep = torch.from_numpy(O.expand_keep(O.random_mask((4, 4), 0.5, 3, offset=0), 64, 256, 256)).cuda()
+    assert torch.equal(a != 0, keep)    # and it is draw 0 of seed 3
+    ext = GEMM()
+    ext.manual_seed(77)                 # explicit restart, independent of torch's seed
+    m0, _ = ext.random_lists((5, 7), 0.4)
+    m1, _ = ext.random_lists((5, 7), 0.4)
+    assert ext.rng_state().tolist() == [77, 2]
+    assert np.array_equal(m0.cpu().numpy(), O.random_mask((5, 7), 0.4, 77, offset=0))
+    assert np.array_equal(m1.cpu().numpy(), O.random_mask((5, 7), 0.4, 77, offset=1))
+    # large mask: the multi-launch builder reads the same state in all of its kernels
+    m2, l2 = ext.random_lists((600, 600), 0.5)
+    want = O.random_mask((600, 600), 0.5, 77, offset=2)
+    assert np.array_equal(m2.cpu().numpy(), want)
+    _assert_lists(l2, want)
+    assert ext.rng_state().tolist() == [77, 3]
+
+
+def test_graph_replays_draw_fresh_masks():
+    """A captured forward + backward step replays correctly and every replay draws a new mask: nothing
+    about the draw is a launch argument.  Replays are separated by eager work and synchronisation, and
+    each is checked against the oracle under the mask it must have drawn."""
+    import flash_dropout.functional as F
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    m, n, k, p = 512, 256, 384, 0.5
+    gen = torch.Generator().manual_seed(21)
+    x = make_operand((m, k), torch.float16, gen)
+    w = make_operand((n, k), torch.float16, gen, scale=k ** -0.5)
+    dy = make_operand((m, n), torch.float16, gen)
+    xg, wg, dyg = x.cuda().requires_grad_(), w.cuda().requires_grad_(), dy.cuda()
+    ext.manual_seed(5)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):       # warm-up on the capture stream: kernels configured, state created
+        for _ in range(2):
+            F.hip_blockwise_dropout_matmul(xg, wg, 64, p).backward(dyg)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    xg.grad = wg.grad = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = F.hip_blockwise_dropout_matmul(xg, wg, 64, p)
+        y.backward(dyg)
+    torch.cuda.synchronize()
+    first = int(ext.rng_state()[1].item())   # capture itself does not run the kernels
+    assert first == 2
+    xf, wf, dyf = x.float().numpy(), w.float().numpy(), dy.float().numpy()
+    seen = []
+    for r in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        mask = O.random_mask(O.mask_shape(m, k, 64), p, 5, offset=first + r)
+        assert rel_fro(y, O.dsd_forward(xf, wf, mask, 64, p)) <= REL_FRO_TOL, r
+        assert rel_fro(xg.grad, O.sdd_dx(dyf, wf, mask, 64, p)) <= REL_FRO_TOL, r
+        assert rel_fro(wg.grad, O.dsd_dw(dyf, xf, mask, 64, p)) <= REL_FRO_TOL, r
+        seen.append(mask)
+        # eager work between replays
+        eager = F.hip_blockwise_dropout_matmul_mask(xg.detach(), torch.from_numpy(mask).cuda(), 64, p, wg.detach())
+        assert rel_fro(eager, y) <= 1e-3
+        torch.cuda.synchronize()
+    assert not np.array_equal(seen[0], seen[1]) and not np.array_equal(seen[1], seen[2])
+    assert int(ext.rng_state()[1].item()) == first + 3
 
 
 def test_conv_with_larger_blocks_and_device_mask():
