@@ -59,6 +59,15 @@ class BlockwiseDropoutMatmulHIP(torch.autograd.Function):
         return grad_input, grad_weight, None, None, None, None
 
 
+def _apply_outside_autocast(function, *args):
+    """``function.apply(*args)`` with autocast off inside, as ``custom_fwd(cast_inputs=...)`` arranges in the
+    reference (…_cuda.py:9); the context is only entered when autocast is on (it costs microseconds per call)."""
+    if torch.is_autocast_enabled("cuda"):
+        with torch.autocast("cuda", enabled=False):
+            return function.apply(*args)
+    return function.apply(*args)
+
+
 def _prepare(input: torch.Tensor, weight: torch.Tensor):
     """Autocast contract of the reference (``custom_fwd(cast_inputs=torch.float16)``, …_cuda.py:9):
     under autocast the operands are cast to the autocast dtype; outside it they must already be
@@ -83,8 +92,7 @@ def blockwise_dropout_matmul_mask(input: torch.Tensor, mask: torch.Tensor, block
         raise ValueError("Dropout probability must be in [0, 1)")
     bs = _block_size(block_size)
     input, weight = _prepare(input, weight)
-    with torch.autocast("cuda", enabled=False):
-        return BlockwiseDropoutMatmulHIP.apply(input, weight, mask, bs, float(p))
+    return _apply_outside_autocast(BlockwiseDropoutMatmulHIP, input, weight, mask, bs, float(p))
 
 
 def blockwise_dropout_matmul(input: torch.Tensor, weight: torch.Tensor, block_size, p: float,
@@ -100,5 +108,4 @@ def blockwise_dropout_matmul(input: torch.Tensor, weight: torch.Tensor, block_si
         raise ValueError("Dropout probability must be in [0, 1)")
     bs = _block_size(block_size)
     input, weight = _prepare(input, weight)
-    with torch.autocast("cuda", enabled=False):
-        return BlockwiseDropoutMatmulHIP.apply(input, weight, None, bs, float(p), seed)
+    return _apply_outside_autocast(BlockwiseDropoutMatmulHIP, input, weight, None, bs, float(p), seed)

@@ -85,6 +85,15 @@ class _Im2colConv2d(torch.autograd.Function):
         return dx, dk, None, None, None, None, None, None, None
 
 
+def _apply_outside_autocast(function, *args):
+    """``function.apply(*args)`` with autocast off inside, as ``custom_fwd(cast_inputs=...)`` arranges in the
+    reference (…_cuda.py:9); the context is only entered when autocast is on (it costs microseconds per call)."""
+    if torch.is_autocast_enabled("cuda"):
+        with torch.autocast("cuda", enabled=False):
+            return function.apply(*args)
+    return function.apply(*args)
+
+
 def _prepare(input: torch.Tensor, kernel: torch.Tensor):
     if input.dim() != 4 or kernel.dim() != 4:
         raise ValueError("input must be (N, C, H, W) and kernel (K, C, R, S)")
@@ -100,8 +109,7 @@ def im2col_conv2d(input: torch.Tensor, kernel: torch.Tensor, padding=(0, 0), str
                   dilation=(1, 1)) -> torch.Tensor:
     """Dense convolution through the patch matrix (reference: im2col_conv2d.py:5-27)."""
     input, kernel = _prepare(input, kernel)
-    with torch.autocast("cuda", enabled=False):
-        return _Im2colConv2d.apply(input, kernel, None, 0, 0.0, _pair(padding), _pair(stride), _pair(dilation))
+    return _apply_outside_autocast(_Im2colConv2d, input, kernel, None, 0, 0.0, _pair(padding), _pair(stride), _pair(dilation))
 
 
 def conv_patch_matrix_shape(input_shape, kernel_shape, padding=(0, 0), stride=(1, 1), dilation=(1, 1)):
@@ -120,8 +128,7 @@ def blockwise_dropout_conv2d_mask(input, mask, block_size, p: float, kernel, pad
         raise ValueError("Dropout probability must be in [0, 1)")
     bs = _block_size(block_size)
     input, kernel = _prepare(input, kernel)
-    with torch.autocast("cuda", enabled=False):
-        return _Im2colConv2d.apply(input, kernel, mask, bs, float(p), _pair(padding), _pair(stride), _pair(dilation))
+    return _apply_outside_autocast(_Im2colConv2d, input, kernel, mask, bs, float(p), _pair(padding), _pair(stride), _pair(dilation))
 
 
 def blockwise_dropout_conv2d(input, kernel, block_size, p: float, padding=(0, 0), stride=(1, 1),
@@ -132,8 +139,7 @@ def blockwise_dropout_conv2d(input, kernel, block_size, p: float, padding=(0, 0)
         raise ValueError("Dropout probability must be in [0, 1)")
     bs = _block_size(block_size)
     input, kernel = _prepare(input, kernel)
-    with torch.autocast("cuda", enabled=False):
-        return _Im2colConv2d.apply(input, kernel, None, bs, float(p), _pair(padding), _pair(stride),
+    return _apply_outside_autocast(_Im2colConv2d, input, kernel, None, bs, float(p), _pair(padding), _pair(stride),
                                    _pair(dilation), seed)
 
 

@@ -55,6 +55,11 @@ class KeptLists:
 
 _NO_GUARD = contextlib.nullcontext()
 
+# torch keeps a fast accessor for the raw current-stream handle (an order of magnitude cheaper than building
+# a Stream object per launch); fall back to the public API where it is missing
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None) or (
+    lambda index: torch.cuda.current_stream(index).cuda_stream)
+
 
 def _device(device) -> torch.device:
     dev = torch.device("cuda") if device is None else torch.device(device)
@@ -136,7 +141,8 @@ class GEMM:
 
     @staticmethod
     def _stream(t: torch.Tensor) -> int:
-        return torch.cuda.current_stream(t.device).cuda_stream
+        """Raw handle of torch's current stream on the tensor's device (what the launches go to)."""
+        return _raw_stream(t.device.index)
 
     def _check_pair(self, A, B):
         _check_operand("A", A)
@@ -180,6 +186,7 @@ class GEMM:
             return None, None, 0
         ws = torch.empty(nbytes // 4, dtype=torch.float32, device=A.device)
         return ws, ws.data_ptr(), nbytes
+
 
     def _masked(self, fn, mask_cols, A, B, mask, block_size, scale, out, transposed_out):
         self._check_pair(A, B)
