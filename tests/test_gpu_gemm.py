@@ -71,8 +71,6 @@ def test_reference_grid(mnk, block_size, p):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_block64_square(mnk, p, dtype):
     M, N, K = mnk
-    if dtype == torch.bfloat16 and M > 1024:
-        pytest.skip("bf16 covered at the smaller sizes")
     bs = 64
     gen = torch.Generator().manual_seed(1)
     A = make_operand(M, K, dtype, "cuda", gen=gen)
