@@ -188,7 +188,7 @@ def main() -> int:
     LD_PAD = args.ld_pad
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
-              "(the path has no collectives; sharding is described in DESIGN.md)", file=sys.stderr)
+              "(the path has no collectives: row blocks would shard over GPUs with one reduction for dW)", file=sys.stderr)
         return 2
 
     import torch

@@ -1,5 +1,5 @@
-"""The drop-in stub printed in INTEGRATION.md really is a working binding: extract it, point it at the
-built library and run the reference's three-call sequence through it."""
+"""The drop-in binding stub published with the integration notes really is a working binding: extract the
+code block, point it at the built library and run the reference's three-call sequence through it."""
 import re
 from pathlib import Path
 
