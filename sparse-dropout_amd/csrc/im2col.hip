@@ -361,6 +361,7 @@ __global__ __launch_bounds__(256) void col2im_unit_kernel(const uint16_t* __rest
   const int t = threadIdx.x;
   const int rs_n = g.r * g.s;
   const int seg_h = C2I_CG * rs_n + 2;
+  const int bs_shift = (bs & (bs - 1)) == 0 ? 31 - __builtin_clz((unsigned)bs) : -1;
   int b = blockIdx.x;
   const int band = b % bands;
   b /= bands;
@@ -375,6 +376,26 @@ __global__ __launch_bounds__(256) void col2im_unit_kernel(const uint16_t* __rest
   // ---- stage: R*S 16-byte chunks per window position, zeros outside the matrix and for dropped blocks
   const int chunks = pe * qe * rs_n;
   const int col0 = c0 * rs_n;
+  // the few mask entries the window can touch are copied to LDS first, so that the staging loop does not
+  // chain a global mask read in front of every data load
+  __shared__ uint8_t mtab[256];
+  int64_t rb_lo = 0;
+  int cb_lo = 0, cb_n = 1;
+  bool mask_in_lds = false;
+  if (mask) {
+    const int pp_lo = p_first > 0 ? p_first : 0;
+    const int pp_hi = p_first + pe - 1 < g.p - 1 ? p_first + pe - 1 : g.p - 1;
+    rb_lo = (((int64_t)n_i * g.p + pp_lo) * g.q) / bs;
+    const int64_t rb_hi = (((int64_t)n_i * g.p + pp_hi) * g.q + g.q - 1) / bs;
+    cb_lo = col0 / bs;
+    cb_n = (col0 + C2I_CG * rs_n - 1) / bs - cb_lo + 1;
+    const int64_t rb_n = pp_hi >= pp_lo ? rb_hi - rb_lo + 1 : 0;
+    mask_in_lds = rb_n * cb_n <= 256;
+    if (mask_in_lds) {
+      if (t < rb_n * cb_n) mtab[t] = mask[(rb_lo + t / cb_n) * msr + (cb_lo + t % cb_n) * msc];
+      __syncthreads();
+    }
+  }
   for (int ch0 = t; ch0 < chunks; ch0 += 4 * 256) {
     u32x4 v[4];
     const uint16_t* src[4];  // null: zeros
@@ -390,7 +411,12 @@ __global__ __launch_bounds__(256) void col2im_unit_kernel(const uint16_t* __rest
           const int64_t row = ((int64_t)n_i * g.p + pp) * g.q + qq;
           const int col = col0 + k * 8;
           src[i] = cols + row * ld + col;
-          if (mask) dropped = mask[(row / bs) * msr + (col / bs) * msc];
+          if (mask) {
+            // block sizes are powers of two in practice: a shift instead of a 64-bit division per chunk
+            const int64_t rb = bs_shift >= 0 ? row >> bs_shift : row / bs;
+            const int cb = bs_shift >= 0 ? col >> bs_shift : col / bs;
+            dropped = mask_in_lds ? mtab[(rb - rb_lo) * cb_n + (cb - cb_lo)] : mask[rb * msr + cb * msc];
+          }
         }
       }
       if (dropped) src[i] = nullptr;
