@@ -59,6 +59,12 @@ int sd_version(void);
  * exceptions of gemm_binding.cu:18-22,87-89. */
 const char* sd_last_error(void);
 
+/* Which GEMM kernel family the calling thread's last sd_gemm* call ran on: "specialised" (the tiled
+ * kernels for 64-blocks and aligned operands) or "generic" (any shape and layout, several times slower
+ * per FLOP); "" before the first call.  For tests and for callers who want to know whether a shape is on
+ * the fast path.  No counterpart in the reference. */
+const char* sd_last_kernel(void);
+
 /* ---------------------------------------------------------------------------------------------
  * (a) block-mask -> compacted kept-block lists
  *

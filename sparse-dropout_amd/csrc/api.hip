@@ -61,6 +61,8 @@ int check_sparse(int64_t bs, float scale) {
   return SD_OK;
 }
 
+thread_local const char* last_kernel = "";
+
 int run(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   static const bool force_generic = [] {
     const char* e = std::getenv("SPARSEDROP_FORCE_GENERIC");
@@ -68,8 +70,12 @@ int run(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   }();
   if (!force_generic) {
     const int rc = launch_fast(g, mode, dtype, stream);
-    if (rc != SD_ERR_UNSUPPORTED) return rc;
+    if (rc != SD_ERR_UNSUPPORTED) {
+      last_kernel = "specialised";
+      return rc;
+    }
   }
+  last_kernel = "generic";
   return launch_generic(g, mode, dtype, stream);
 }
 
@@ -107,6 +113,8 @@ extern "C" {
 int sd_version(void) { return 100; }
 
 const char* sd_last_error(void) { return last_error_buf(); }
+
+const char* sd_last_kernel(void) { return last_kernel; }
 
 int64_t sd_workspace_bytes(int64_t mb, int64_t kb) {
   if (mb < 0 || kb < 0) return 0;

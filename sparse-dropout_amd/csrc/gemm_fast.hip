@@ -209,6 +209,15 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
   // fixed for the whole kernel; per step only a wave-uniform base moves.
   uint32_t b_lane[4], a_lane;
   bool b_valid[4];  // the lane's 16 bytes of the W tile lie inside the matrix (a tile may overhang N)
+  // Ragged edges.  Reduction-contiguous operands: M need not be a multiple of 64; the rows of the last row
+  // block that lie past M are fetched from its last valid row instead (rows are independent, theirs are
+  // never stored).  Reduction-strided operands: the reduction length need not be a multiple of 64; the
+  // rows of the last reduction block past the end are fetched from its last valid row and the fragments
+  // are zeroed from that index on before they reach an MFMA.
+  uint32_t b_lane_t[4], a_lane_t;  // lane offsets for the ragged block
+  const int r_tail = (!TRANS && g.M % BS) ? Mb - 1 - rb0 : -1;       // patch row block that is ragged
+  const int kb_tail = (TRANS && g.K % BS) ? Kb_all - 1 : -1;         // reduction block that is ragged
+  const int tail_valid = TRANS ? (int)(g.K % BS) : (int)(g.M % BS);  // rows of it inside the matrix
   const char* a_tile0;  // first X tile of the patch at reduction block 0
   const char* b_tile0;  // W tile at reduction block 0
   int64_t red_stride;   // bytes between consecutive reduction blocks
@@ -224,6 +233,12 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
     }
     const int row = wave * 8 + ld_row;
     a_lane = (uint32_t)(row * g.a.sr + (ld_pch ^ ((row >> 1) & 7)) * 8) * 2u;
+    {
+      const int rc = (r_tail >= 0 && row >= tail_valid) ? tail_valid - 1 : row;  // swizzle stays that of `row`
+      a_lane_t = (uint32_t)(rc * g.a.sr + (ld_pch ^ ((row >> 1) & 7)) * 8) * 2u;
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) b_lane_t[jj] = b_lane[jj];
+    }
     a_tile0 = reinterpret_cast<const char*>(g.a.ptr + (int64_t)rb0 * BS * g.a.sr);
     b_tile0 = reinterpret_cast<const char*>(g.b.ptr + n0 * g.b.sr);
     red_stride = BS * 2;
@@ -236,9 +251,15 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
       const int col = ((lane % 32) ^ ((row & 3) << 2)) * 8;
       b_lane[jj] = (uint32_t)(row * g.b.sc + col) * 2u;
       b_valid[jj] = col < nvalid;
+      const int rc = (kb_tail >= 0 && row >= tail_valid) ? tail_valid - 1 : row;
+      b_lane_t[jj] = (uint32_t)(rc * g.b.sc + col) * 2u;
     }
     const int row = wave * 8 + lane / 8;
     a_lane = (uint32_t)(row * g.a.sc + ((lane % 8) ^ (((row >> 1) & 1) << 2)) * 8) * 2u;
+    {
+      const int rc = (kb_tail >= 0 && row >= tail_valid) ? tail_valid - 1 : row;
+      a_lane_t = (uint32_t)(rc * g.a.sc + ((lane % 8) ^ (((row >> 1) & 1) << 2)) * 8) * 2u;
+    }
     a_tile0 = reinterpret_cast<const char*>(g.a.ptr + (int64_t)rb0 * BS);
     b_tile0 = reinterpret_cast<const char*>(g.b.ptr + n0);
     red_stride = (int64_t)BS * g.a.sc * 2;  // == BS * g.b.sc * 2 only if the leading dimensions agree
@@ -252,12 +273,24 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
     char* st = smem + stage * STAGE;
     const char* bp = b_tile0 + kb * b_red_stride;
     const char* ap = a_tile0 + kb * red_stride;
+    const bool red_tail = kb == kb_tail;  // wave-uniform
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj)
-      if (b_valid[jj]) load16_to_lds(bp, b_lane[jj], st + (wave * 4 + jj) * 1024);
+      if (b_valid[jj]) load16_to_lds(bp, red_tail ? b_lane_t[jj] : b_lane[jj], st + (wave * 4 + jj) * 1024);
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      if (fl & (1u << r)) load16_to_lds(ap + r * a_rstride, a_lane, st + A_OFF + r * TILE + wave * 1024);
+      if (fl & (1u << r))
+        load16_to_lds(ap + r * a_rstride, (red_tail || r == r_tail) ? a_lane_t : a_lane,
+                      st + A_OFF + r * TILE + wave * 1024);
+  };
+  // zeroes the elements of a fragment whose reduction index (16*ks + 8*(lane/32) + 0..7 inside the
+  // block) is not below tail_valid
+  auto mask_fragment = [&](u32x4& f, int ks) {
+    const int n = tail_valid - (16 * ks + 8 * (lane / 32));  // valid elements among the lane's 8
+    f.x &= n >= 2 ? ~0u : (n == 1 ? 0xffffu : 0u);
+    f.y &= n >= 4 ? ~0u : (n == 3 ? 0xffffu : 0u);
+    f.z &= n >= 6 ? ~0u : (n == 5 ? 0xffffu : 0u);
+    f.w &= n >= 8 ? ~0u : (n == 7 ? 0xffffu : 0u);
   };
 
   f32x16 acc[2][2][2];  // [row block of the pair][m tile][n tile]
@@ -301,7 +334,8 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
   // (MINE = 1, 2 or 3).  The work is a chain of units (row block, ks); the LDS reads of unit u+1 are
   // issued before the MFMAs of unit u so that their latency hides behind 4 MFMAs (128 cycles).  The W
   // fragments are read during the first row block's units and stay in registers for the second.
-  auto compute = [&](auto mine_c, const char* st, bool mid_loads, uint32_t mid_entry, int mid_stage) {
+  auto compute = [&](auto mine_c, const char* st, bool mid_loads, uint32_t mid_entry, int mid_stage,
+                     bool red_tail) {
     constexpr int MINE = decltype(mine_c)::value;
     constexpr int NR = (MINE == 3) ? 2 : 1;
     constexpr int R0 = (MINE == 2) ? 1 : 0;
@@ -319,6 +353,14 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
         read_a(at0 + ((u + 1) / 4) * TILE, ks1, af[(u + 1) & 1]);
       }
       __builtin_amdgcn_sched_barrier(0);
+      if (TRANS && red_tail) {  // ragged reduction block: nothing past the end may reach the MFMAs
+        mask_fragment(af[u & 1][0], ks);
+        mask_fragment(af[u & 1][1], ks);
+        if (u < 4) {
+          mask_fragment(bf[0][ks], ks);
+          mask_fragment(bf[1][ks], ks);
+        }
+      }
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -346,9 +388,10 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
     const bool mid = late && more && mine != 0u;
     if (more && !mid) issue_loads(e_next, stage ^ 1);
     const char* st = smem + stage * STAGE;
-    if (mine == 3u) compute(std::integral_constant<int, 3>{}, st, mid, e_next, stage ^ 1);
-    else if (mine == 1u) compute(std::integral_constant<int, 1>{}, st, mid, e_next, stage ^ 1);
-    else if (mine == 2u) compute(std::integral_constant<int, 2>{}, st, mid, e_next, stage ^ 1);
+    const bool red_tail = step_block(e_cur) == kb_tail;
+    if (mine == 3u) compute(std::integral_constant<int, 3>{}, st, mid, e_next, stage ^ 1, red_tail);
+    else if (mine == 1u) compute(std::integral_constant<int, 1>{}, st, mid, e_next, stage ^ 1, red_tail);
+    else if (mine == 2u) compute(std::integral_constant<int, 2>{}, st, mid, e_next, stage ^ 1, red_tail);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     e_cur = e_next;
@@ -374,6 +417,7 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
           const int lane_i = lane % 32;
           const int64_t m = (int64_t)rb * BS + mt * 32 + (CM ? lane_i : reg_i);
           const int64_t n = n0 + ns * 64 + nt * 32 + (CM ? reg_i : lane_i);
+          if (m >= g.M) continue;  // ragged last row block
           if (part)  // unscaled fp32 partial in C's own element order; the reduce pass scales and rounds
             part[CM ? n * g.M + m : m * g.N + n] = acc[rr][mt][nt][v];
           else
@@ -517,7 +561,7 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
       const uint32_t f = (uint32_t)__builtin_amdgcn_readfirstlane((int)flags[c]);
       for (int r = 0; r < R; ++r) {
         if (rb0 + r >= Mb) break;
-        if (!((f >> r) & 1u))
+        if (!((f >> r) & 1u) && (int64_t)(rb0 + r) * BS + row < g.M)
           *reinterpret_cast<u32x4*>(g.c + ((int64_t)(rb0 + r) * BS + row) * g.c_sr + (int64_t)c * BS + ch * 8) = z;
       }
     }
@@ -542,11 +586,17 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
   // loads: wave-uniform tile bases plus this lane's 16 bytes of the wave's 8 tile rows
   const char* a_base = reinterpret_cast<const char*>(g.a.ptr + (int64_t)rb0 * BS * g.a.sr);
   const char* b_base = reinterpret_cast<const char*>(g.b.ptr);
-  uint32_t a_lane, b_lane;
+  // M need not be a multiple of 64: rows of the last row block past M are fetched from its last valid row
+  // (rows are independent, theirs are never stored)
+  uint32_t a_lane, a_lane_t, b_lane;
+  const int r_tail = (g.M % BS) ? Mb - 1 - rb0 : -1;
   {
     const int row = wave * 8 + lane / 8;
     const int pch = lane % 8;
     a_lane = (uint32_t)(row * g.a.sr + (pch ^ ((row >> 1) & 7)) * 8) * 2u;
+    const int valid = (int)(g.M % BS);
+    const int rc = (r_tail >= 0 && row >= valid) ? valid - 1 : row;
+    a_lane_t = (uint32_t)(rc * g.a.sr + (pch ^ ((row >> 1) & 7)) * 8) * 2u;
     b_lane = (uint32_t)(row * g.b.sc + (pch ^ (((row >> 1) & 1) << 2)) * 8) * 2u;
   }
   const int64_t a_tile_stride = (int64_t)BS * g.a.sr * 2;
@@ -557,7 +607,7 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
     const char* bp = b_base + step * b_step_stride;
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      if (rowmask & (1u << r)) load16_to_lds(ap + r * a_tile_stride, a_lane, st + r * TILE);
+      if (rowmask & (1u << r)) load16_to_lds(ap + r * a_tile_stride, r == r_tail ? a_lane_t : a_lane, st + r * TILE);
 #pragma unroll
     for (int j = 0; j < GW; ++j)
       if (j < ncols) load16_to_lds(bp + (int64_t)cols[j] * (BS * 2), b_lane, st + G_BOFF + j * TILE);
@@ -643,7 +693,7 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
         for (int v = 0; v < 16; ++v) {
           const int64_t m = (int64_t)(rb0 + my_r[k]) * BS + mt * 32 + 8 * (v / 4) + 4 * (lane / 32) + (v % 4);
           const int64_t n = (int64_t)my_c[k] * BS + nt * 32 + (lane % 32);
-          g.c[m * g.c_sr + n] = T::from_float(acc[k][mt][nt][v] * g.scale);
+          if (m < g.M) g.c[m * g.c_sr + n] = T::from_float(acc[k][mt][nt][v] * g.scale);
         }
   }
 }
@@ -670,7 +720,7 @@ int launch_dsd(const GemmArgs& g, int splits, hipStream_t stream) {
   static bool configured[kMaxDevices] = {};
   if (int rc = allow_big_lds(reinterpret_cast<const void*>(&dsd_kernel<T, TRANS, CM>), SMEM_BYTES, configured))
     return rc;
-  const int Mb = (int)(g.M / BS), Kb = (int)(g.K / BS);
+  const int Mb = (int)((g.M + BS - 1) / BS), Kb = (int)((g.K + BS - 1) / BS);
   const int tiles_m = (Mb + R - 1) / R, tiles_n = (int)((g.N + BN - 1) / BN);
   hipLaunchKernelGGL((dsd_kernel<T, TRANS, CM>), dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits),
                      dim3(THREADS), SMEM_BYTES, stream, g, tiles_m, tiles_n, Mb, Kb);
@@ -683,7 +733,7 @@ template <typename T>
 int launch_sdd_group(const GemmArgs& g, hipStream_t stream) {
   static bool configured[kMaxDevices] = {};
   if (int rc = allow_big_lds(reinterpret_cast<const void*>(&sdd_group_kernel<T>), G_SMEM, configured)) return rc;
-  const int Mb = (int)(g.M / BS), Cb = (int)(g.N / BS);
+  const int Mb = (int)((g.M + BS - 1) / BS), Cb = (int)(g.N / BS);
   const int tiles_m = (Mb + R - 1) / R, gmax = (Cb + R - 1) / R;
   hipLaunchKernelGGL(sdd_group_kernel<T>, dim3((unsigned)(tiles_m * gmax)), dim3(THREADS), G_SMEM, stream, g,
                      tiles_m, gmax, Mb, Cb);
@@ -693,11 +743,11 @@ int launch_sdd_group(const GemmArgs& g, hipStream_t stream) {
 int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
   if (g.row_ptr && g.bs != BS) return SD_ERR_UNSUPPORTED;
   const bool layout_ok = g.a.sc == 1 && g.b.sr == 1 && g.b.sc != 1 && g.c_sc == 1;
-  const bool shape_ok = g.M > 0 && g.M % BS == 0 && g.N > 0 && g.N % BS == 0 && g.K > 0 && g.K % BS == 0;
+  const bool shape_ok = g.M > 0 && g.N > 0 && g.N % BS == 0 && g.K > 0 && g.K % BS == 0;  // any M
   const bool align_ok = aligned16(g.a.ptr) && aligned16(g.b.ptr) && aligned16(g.c) && g.a.sr % 8 == 0 &&
                         g.b.sc % 8 == 0 && g.c_sr % 8 == 0 && g.a.sr < (1 << 22) &&
                         g.b.sc < (1 << 22);  // per-lane byte offsets are 32-bit
-  const int64_t tiles = ((g.M / BS + R - 1) / R) * ((g.N / BS + R - 1) / R);
+  const int64_t tiles = (((g.M + BS - 1) / BS + R - 1) / R) * ((g.N / BS + R - 1) / R);
   if (!layout_ok || !shape_ok || !align_ok || tiles > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
   if (g.N / BS > G_MAX_CB) return SD_ERR_UNSUPPORTED;
   return dtype == SD_BF16 ? launch_sdd_group<BF16>(g, stream) : launch_sdd_group<F16>(g, stream);
@@ -715,12 +765,13 @@ int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   const bool nt = g.a.sc == 1 && g.b.sc == 1;         // reduction-contiguous operands
   const bool tn = !nt && g.a.sr == 1 && g.b.sr == 1;  // reduction-strided operands
   const bool cm = g.c_sc != 1;                        // column-major C
-  const bool shape_ok = g.M > 0 && g.M % BS == 0 && g.N > 0 && g.N % BS == 0 && g.K > 0 && g.K % BS == 0 &&
-                        g.K / BS < 65536;
+  // ragged edges: the rows of a reduction-contiguous A (M), the reduction length of reduction-strided operands (K)
+  const bool shape_ok = g.M > 0 && (nt || g.M % BS == 0) && g.N > 0 && g.N % BS == 0 && g.K > 0 &&
+                        (tn || g.K % BS == 0) && (g.K + BS - 1) / BS < 65536;
   const int64_t lda = nt ? g.a.sr : g.a.sc, ldb = nt ? g.b.sr : g.b.sc;
   const bool align_ok = aligned16(g.a.ptr) && aligned16(g.b.ptr) && lda % 8 == 0 && ldb % 8 == 0 &&
                         lda < (1 << 22) && ldb < (1 << 22);  // per-lane byte offsets are 32-bit
-  const int64_t tiles = ((g.M / BS + R - 1) / R) * ((g.N + BN - 1) / BN);
+  const int64_t tiles = (((g.M + BS - 1) / BS + R - 1) / R) * ((g.N + BN - 1) / BN);
   if (!(nt || tn) || !shape_ok || !align_ok || tiles > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
   // few output tiles and a long reduction (the weight gradient of a tall matrix): split the reduction
   // over workgroups when the caller gave scratch for the fp32 partials
@@ -729,7 +780,7 @@ int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   if (splits > 1 && (g.ws == nullptr || g.ws_bytes < part_bytes * splits))
     splits = g.ws ? (int)(g.ws_bytes / part_bytes) : 1;
   if (splits < 1) splits = 1;
-  if ((g.K / BS + splits - 1) / splits > MAX_STEPS) return SD_ERR_UNSUPPORTED;  // step table is per workgroup
+  if (((g.K + BS - 1) / BS + splits - 1) / splits > MAX_STEPS) return SD_ERR_UNSUPPORTED;  // step table is per workgroup
   if (splits == 1 && tiles < 128 && g.ws != nullptr) {
     // scratch too small for this kernel's partials: the generic kernel's split may still fit
     const int gs = generic_splits(g.M, g.N, g.K, g.bs, mode);

@@ -131,6 +131,10 @@ class GEMM:
         self.lib = _loader.load()
         self._rng: dict[int, tuple[int, torch.Tensor]] = {}  # device index -> (torch seed it follows, state)
 
+    def last_kernel(self) -> str:
+        """"specialised" or "generic": the kernel family this thread's last GEMM call ran on."""
+        return self.lib.sd_last_kernel().decode()
+
     # ------------------------------------------------------------------ plumbing
     def _call(self, fn, *args) -> None:
         rc = fn(*args)

@@ -312,3 +312,66 @@ def test_sdd_column_groups(M, N, K):
         assert rel_fro(got, ref) <= REL_FRO_TOL, name
         keep = O.expand_keep(mk.numpy(), 64, M, K)
         assert (got.cpu().numpy()[~keep] == 0).all(), name
+
+
+@pytest.mark.parametrize("M,N,K", [(1000, 256, 512), (19700 // 4, 384, 768), (70, 128, 192), (4097, 512, 256),
+                                   (8200, 128, 576)])
+@pytest.mark.parametrize("p", [0.0, 0.5])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_ragged_row_count_stays_on_the_specialised_kernels(M, N, K, p, dtype):
+    """M (batch x sequence) is rarely a multiple of 64: forward, dX and the row-major dW all run on the
+    specialised kernels with a ragged last row block, and match the oracle."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(M + N)
+    A = make_operand(M, K, dtype, "cuda", gen=gen)
+    B = make_operand(N, K, dtype, "cuda", scale=K ** -0.5, gen=gen)
+    dC = make_operand(M, N, dtype, "cuda", gen=gen)
+    mk = cpu_mask(O.mask_shape(M, K, 64), p, gen)
+    lists = ext.build_lists(mk.cuda())
+    s = 1 / (1 - p)
+    C = ext.gemm_dsd_lists(A, B, lists, 64, s)
+    assert ext.last_kernel() == "specialised"
+    dA = ext.gemm_sdd_lists(dC, B.T, lists, 64, s)
+    assert ext.last_kernel() == "specialised"
+    dB = ext.gemm_dsd_lists(A.T, dC.T, lists.transposed(), 64, s, transposed_out=True).T
+    assert ext.last_kernel() == "specialised"
+    rC, rdA, rdB = _oracle_products(A, B, dC, mk, 64, p)
+    for got, ref, what in ((C, rC, "C"), (dA, rdA, "dA"), (dB, rdB, "dB")):
+        assert rel_fro(got, ref) <= REL_FRO_TOL, what
+    keep = O.expand_keep(mk.numpy(), 64, M, K)
+    assert (to_np(dA)[~keep] == 0).all()
+    # the dense products on the same ragged shape
+    assert rel_fro(ext.gemm(A, B), to_np(A) @ to_np(B).T) <= REL_FRO_TOL
+    assert ext.last_kernel() == "specialised"
+    assert rel_fro(ext.gemm(A.T, dC.T, transposed_out=True), to_np(A).T @ to_np(dC)) <= REL_FRO_TOL
+    assert ext.last_kernel() == "specialised"
+
+
+@pytest.mark.parametrize("M,N,K", [(8192, 8192, 8192), (16384, 1536, 384), (16384, 384, 1536), (131072, 128, 576)])
+def test_baseline_shapes_run_on_the_specialised_kernels(M, N, K):
+    """The benchmark configurations must not fall back to the generic kernel (shapes only: tiny launches
+    on uninitialised operands)."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    A = torch.empty(M, K, dtype=torch.float16, device="cuda").zero_()
+    B = torch.empty(N, K, dtype=torch.float16, device="cuda").zero_()
+    dC = torch.empty(M, N, dtype=torch.float16, device="cuda").zero_()
+    mask = torch.rand(M // 64, K // 64, device="cuda") < 0.5
+    lists = ext.build_lists(mask)
+    ext.gemm_dsd_lists(A, B, lists, 64, 2.0)
+    assert ext.last_kernel() == "specialised"
+    ext.gemm_sdd_lists(dC, B.T, lists, 64, 2.0)
+    assert ext.last_kernel() == "specialised"
+    ext.gemm_dsd_lists(A.T, dC.T, lists.transposed(), 64, 2.0, transposed_out=True)
+    assert ext.last_kernel() == "specialised"
+    # and the reference-style calls with a block size of 128
+    mask128 = torch.rand(-(-M // 128), -(-K // 128), device="cuda") < 0.5
+    ext.gemm_dsd(A, B, mask128, 128, 2.0)
+    assert ext.last_kernel() == "specialised"
+    ext.gemm_sdd(dC, B.T, mask128, 128, 2.0)
+    assert ext.last_kernel() == "specialised"
+    ext.gemm_dsd(A.T, dC.T, mask128.T, 128, 2.0)
+    assert ext.last_kernel() == "specialised"
