@@ -115,7 +115,9 @@ __device__ inline u32x2 lds_read_tr(const char* p) {
 // TRANS = true : A and B are given as transposed views, the reduction index is the strided one (dW)
 // In both cases "Mb" counts the row blocks of A (of X^T for dW) and "Kb" the reduction blocks.
 // CM = C is column-major: the MFMA operands are swapped so that lanes run along C's rows
-template <typename T, bool TRANS, bool CM>
+// RAGGED = M (reduction-contiguous operands) or the reduction length (reduction-strided operands) is not a
+// multiple of 64; a separate instance so that the aligned case carries none of the edge handling
+template <typename T, bool TRANS, bool CM, bool RAGGED>
 __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, int tiles_n,
                                                       int Mb, int Kb_all) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -215,8 +217,8 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
   // rows of the last reduction block past the end are fetched from its last valid row and the fragments
   // are zeroed from that index on before they reach an MFMA.
   uint32_t b_lane_t[4], a_lane_t;  // lane offsets for the ragged block
-  const int r_tail = (!TRANS && g.M % BS) ? Mb - 1 - rb0 : -1;       // patch row block that is ragged
-  const int kb_tail = (TRANS && g.K % BS) ? Kb_all - 1 : -1;         // reduction block that is ragged
+  const int r_tail = (RAGGED && !TRANS && g.M % BS) ? Mb - 1 - rb0 : -1;  // patch row block that is ragged
+  const int kb_tail = (RAGGED && TRANS && g.K % BS) ? Kb_all - 1 : -1;    // reduction block that is ragged
   const int tail_valid = TRANS ? (int)(g.K % BS) : (int)(g.M % BS);  // rows of it inside the matrix
   const char* a_tile0;  // first X tile of the patch at reduction block 0
   const char* b_tile0;  // W tile at reduction block 0
@@ -273,14 +275,15 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
     char* st = smem + stage * STAGE;
     const char* bp = b_tile0 + kb * b_red_stride;
     const char* ap = a_tile0 + kb * red_stride;
-    const bool red_tail = kb == kb_tail;  // wave-uniform
+    const bool red_tail = RAGGED && kb == kb_tail;  // wave-uniform
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj)
-      if (b_valid[jj]) load16_to_lds(bp, red_tail ? b_lane_t[jj] : b_lane[jj], st + (wave * 4 + jj) * 1024);
+      if (b_valid[jj])
+        load16_to_lds(bp, (RAGGED && red_tail) ? b_lane_t[jj] : b_lane[jj], st + (wave * 4 + jj) * 1024);
 #pragma unroll
     for (int r = 0; r < R; ++r)
       if (fl & (1u << r))
-        load16_to_lds(ap + r * a_rstride, (red_tail || r == r_tail) ? a_lane_t : a_lane,
+        load16_to_lds(ap + r * a_rstride, (RAGGED && (red_tail || r == r_tail)) ? a_lane_t : a_lane,
                       st + A_OFF + r * TILE + wave * 1024);
   };
   // zeroes the elements of a fragment whose reduction index (16*ks + 8*(lane/32) + 0..7 inside the
@@ -353,7 +356,7 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
         read_a(at0 + ((u + 1) / 4) * TILE, ks1, af[(u + 1) & 1]);
       }
       __builtin_amdgcn_sched_barrier(0);
-      if (TRANS && red_tail) {  // ragged reduction block: nothing past the end may reach the MFMAs
+      if (RAGGED && TRANS && red_tail) {  // ragged reduction block: nothing past the end may reach the MFMAs
         mask_fragment(af[u & 1][0], ks);
         mask_fragment(af[u & 1][1], ks);
         if (u < 4) {
@@ -388,7 +391,7 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
     const bool mid = late && more && mine != 0u;
     if (more && !mid) issue_loads(e_next, stage ^ 1);
     const char* st = smem + stage * STAGE;
-    const bool red_tail = step_block(e_cur) == kb_tail;
+    const bool red_tail = RAGGED && step_block(e_cur) == kb_tail;
     if (mine == 3u) compute(std::integral_constant<int, 3>{}, st, mid, e_next, stage ^ 1, red_tail);
     else if (mine == 1u) compute(std::integral_constant<int, 1>{}, st, mid, e_next, stage ^ 1, red_tail);
     else if (mine == 2u) compute(std::integral_constant<int, 2>{}, st, mid, e_next, stage ^ 1, red_tail);
@@ -417,7 +420,7 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
           const int lane_i = lane % 32;
           const int64_t m = (int64_t)rb * BS + mt * 32 + (CM ? lane_i : reg_i);
           const int64_t n = n0 + ns * 64 + nt * 32 + (CM ? reg_i : lane_i);
-          if (m >= g.M) continue;  // ragged last row block
+          if (RAGGED && m >= g.M) continue;  // ragged last row block
           if (part)  // unscaled fp32 partial in C's own element order; the reduce pass scales and rounds
             part[CM ? n * g.M + m : m * g.N + n] = acc[rr][mt][nt][v];
           else
@@ -715,18 +718,26 @@ int allow_big_lds(const void* kernel, int bytes, bool (&done)[kMaxDevices]) {
   return SD_OK;
 }
 
-template <typename T, bool TRANS, bool CM>
-int launch_dsd(const GemmArgs& g, int splits, hipStream_t stream) {
+template <typename T, bool TRANS, bool CM, bool RAGGED>
+int launch_dsd_r(const GemmArgs& g, int splits, hipStream_t stream) {
   static bool configured[kMaxDevices] = {};
-  if (int rc = allow_big_lds(reinterpret_cast<const void*>(&dsd_kernel<T, TRANS, CM>), SMEM_BYTES, configured))
+  if (int rc = allow_big_lds(reinterpret_cast<const void*>(&dsd_kernel<T, TRANS, CM, RAGGED>), SMEM_BYTES,
+                             configured))
     return rc;
   const int Mb = (int)((g.M + BS - 1) / BS), Kb = (int)((g.K + BS - 1) / BS);
   const int tiles_m = (Mb + R - 1) / R, tiles_n = (int)((g.N + BN - 1) / BN);
-  hipLaunchKernelGGL((dsd_kernel<T, TRANS, CM>), dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits),
+  hipLaunchKernelGGL((dsd_kernel<T, TRANS, CM, RAGGED>), dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits),
                      dim3(THREADS), SMEM_BYTES, stream, g, tiles_m, tiles_n, Mb, Kb);
   if (int rc = check_launch("dsd_kernel")) return rc;
   if (splits > 1) return launch_splitk_reduce(g, splits, CM, T::id, stream);
   return SD_OK;
+}
+
+template <typename T, bool TRANS, bool CM>
+int launch_dsd(const GemmArgs& g, int splits, hipStream_t stream) {
+  const bool ragged = TRANS ? (g.K % BS != 0) : (g.M % BS != 0);
+  return ragged ? launch_dsd_r<T, TRANS, CM, true>(g, splits, stream)
+                : launch_dsd_r<T, TRANS, CM, false>(g, splits, stream);
 }
 
 template <typename T>
