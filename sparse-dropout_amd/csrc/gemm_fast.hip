@@ -115,8 +115,8 @@ __device__ inline u32x2 lds_read_tr(const char* p) {
 // TRANS = true : A and B are given as transposed views, the reduction index is the strided one (dW)
 // In both cases "Mb" counts the row blocks of A (of X^T for dW) and "Kb" the reduction blocks.
 // CM = C is column-major: the MFMA operands are swapped so that lanes run along C's rows
-// RAGGED = M (reduction-contiguous operands) or the reduction length (reduction-strided operands) is not a
-// multiple of 64; a separate instance so that the aligned case carries none of the edge handling
+// RAGGED = some of M, N, K is not a multiple of 64; a separate instance so that the aligned case carries
+// none of the edge handling
 template <typename T, bool TRANS, bool CM, bool RAGGED>
 __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, int tiles_n,
                                                       int Mb, int Kb_all) {
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
   const int rh = wave / 4;  // row-block pair
   const int rb0 = tm * R;   // first row block
   const int64_t n0 = (int64_t)tn * BN;
-  const int nvalid = (int)((g.N - n0) < BN ? (g.N - n0) : BN);  // columns of this tile inside C (multiple of 64)
+  const int nvalid = (int)((g.N - n0) < BN ? (g.N - n0) : BN);  // columns of this tile inside C
   // split reduction: blockIdx.y takes the reduction blocks [kb_lo, kb_lo + Kb) and leaves an fp32 partial
   const int nsplit = gridDim.y, split = blockIdx.y;
   const int kb_lo = (int)((int64_t)Kb_all * split / nsplit);
@@ -211,15 +211,19 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
   // fixed for the whole kernel; per step only a wave-uniform base moves.
   uint32_t b_lane[4], a_lane;
   bool b_valid[4];  // the lane's 16 bytes of the W tile lie inside the matrix (a tile may overhang N)
-  // Ragged edges.  Reduction-contiguous operands: M need not be a multiple of 64; the rows of the last row
-  // block that lie past M are fetched from its last valid row instead (rows are independent, theirs are
-  // never stored).  Reduction-strided operands: the reduction length need not be a multiple of 64; the
-  // rows of the last reduction block past the end are fetched from its last valid row and the fragments
-  // are zeroed from that index on before they reach an MFMA.
-  uint32_t b_lane_t[4], a_lane_t;  // lane offsets for the ragged block
-  const int r_tail = (RAGGED && !TRANS && g.M % BS) ? Mb - 1 - rb0 : -1;  // patch row block that is ragged
-  const int kb_tail = (RAGGED && TRANS && g.K % BS) ? Kb_all - 1 : -1;    // reduction block that is ragged
-  const int tail_valid = TRANS ? (int)(g.K % BS) : (int)(g.M % BS);  // rows of it inside the matrix
+  // Ragged edges (all in units of 8 elements, the 16 bytes of one lane's load).  A 64-block that overhangs
+  // the matrix along the strided index of its operand is fetched with the overhanging rows redirected to
+  // its last valid row; one that overhangs along the contiguous index with the overhanging 16-byte chunks
+  // redirected to its first chunk.  Either way every load stays inside the matrix and lands in the LDS slot
+  // of the element it stands in for.  What stands in along M (or N) only ever reaches accumulator rows
+  // (columns) that are not stored; what stands in along the reduction is zeroed in the fragments before
+  // it reaches an MFMA.
+  const int m_valid = (int)(g.M % BS), k_valid = (int)(g.K % BS);
+  const int r_tail = (RAGGED && m_valid) ? Mb - 1 - rb0 : -1;   // patch row block that is ragged
+  const int kb_tail = (RAGGED && k_valid) ? Kb_all - 1 : -1;    // reduction block that is ragged
+  // what to add (mod 2^32) to a lane's offset for a block ragged along M / along the reduction: the row and
+  // the chunk term of an offset are redirected independently, so the two corrections add up
+  uint32_t a_delta_m, a_delta_k, b_delta_k[4];
   const char* a_tile0;  // first X tile of the patch at reduction block 0
   const char* b_tile0;  // W tile at reduction block 0
   int64_t red_stride;   // bytes between consecutive reduction blocks
@@ -227,20 +231,24 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
   if (!TRANS) {
     // 8 tile rows per load; lane -> (row lane/8, physical chunk lane%8)
     const int ld_row = lane / 8, ld_pch = lane % 8;
+    // element offset of the lane's chunk; the swizzle (the LDS slot) stays that of `row`
+    auto chunk_at = [&](int row, int64_t ld, int rows_valid, bool clamp_row, bool clamp_k) {
+      const int rc = (clamp_row && row >= rows_valid) ? rows_valid - 1 : row;
+      int c = ld_pch ^ ((row >> 1) & 7);
+      if (clamp_k && c * 8 >= k_valid) c = 0;
+      return (uint32_t)(rc * ld + c * 8) * 2u;
+    };
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
       const int row = (wave * 4 + jj) * 8 + ld_row;
-      b_lane[jj] = (uint32_t)(row * g.b.sr + (ld_pch ^ ((row >> 1) & 7)) * 8) * 2u;
+      b_lane[jj] = chunk_at(row, g.b.sr, 0, false, false);
+      b_delta_k[jj] = chunk_at(row, g.b.sr, 0, false, kb_tail >= 0) - b_lane[jj];
       b_valid[jj] = row < nvalid;
     }
     const int row = wave * 8 + ld_row;
-    a_lane = (uint32_t)(row * g.a.sr + (ld_pch ^ ((row >> 1) & 7)) * 8) * 2u;
-    {
-      const int rc = (r_tail >= 0 && row >= tail_valid) ? tail_valid - 1 : row;  // swizzle stays that of `row`
-      a_lane_t = (uint32_t)(rc * g.a.sr + (ld_pch ^ ((row >> 1) & 7)) * 8) * 2u;
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) b_lane_t[jj] = b_lane[jj];
-    }
+    a_lane = chunk_at(row, g.a.sr, 0, false, false);
+    a_delta_m = chunk_at(row, g.a.sr, m_valid, r_tail >= 0, false) - a_lane;
+    a_delta_k = chunk_at(row, g.a.sr, 0, false, kb_tail >= 0) - a_lane;
     a_tile0 = reinterpret_cast<const char*>(g.a.ptr + (int64_t)rb0 * BS * g.a.sr);
     b_tile0 = reinterpret_cast<const char*>(g.b.ptr + n0 * g.b.sr);
     red_stride = BS * 2;
@@ -253,15 +261,19 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
       const int col = ((lane % 32) ^ ((row & 3) << 2)) * 8;
       b_lane[jj] = (uint32_t)(row * g.b.sc + col) * 2u;
       b_valid[jj] = col < nvalid;
-      const int rc = (kb_tail >= 0 && row >= tail_valid) ? tail_valid - 1 : row;
-      b_lane_t[jj] = (uint32_t)(rc * g.b.sc + col) * 2u;
+      const int rc = (kb_tail >= 0 && row >= k_valid) ? k_valid - 1 : row;
+      b_delta_k[jj] = (uint32_t)(rc * g.b.sc + col) * 2u - b_lane[jj];
     }
     const int row = wave * 8 + lane / 8;
-    a_lane = (uint32_t)(row * g.a.sc + ((lane % 8) ^ (((row >> 1) & 1) << 2)) * 8) * 2u;
-    {
-      const int rc = (kb_tail >= 0 && row >= tail_valid) ? tail_valid - 1 : row;
-      a_lane_t = (uint32_t)(rc * g.a.sc + ((lane % 8) ^ (((row >> 1) & 1) << 2)) * 8) * 2u;
-    }
+    auto chunk_at = [&](bool clamp_m, bool clamp_k) {
+      const int rc = (clamp_k && row >= k_valid) ? k_valid - 1 : row;
+      int c = (lane % 8) ^ (((row >> 1) & 1) << 2);
+      if (clamp_m && c * 8 >= m_valid) c = 0;
+      return (uint32_t)(rc * g.a.sc + c * 8) * 2u;
+    };
+    a_lane = chunk_at(false, false);
+    a_delta_m = chunk_at(r_tail >= 0, false) - a_lane;
+    a_delta_k = chunk_at(false, kb_tail >= 0) - a_lane;
     a_tile0 = reinterpret_cast<const char*>(g.a.ptr + (int64_t)rb0 * BS);
     b_tile0 = reinterpret_cast<const char*>(g.b.ptr + n0);
     red_stride = (int64_t)BS * g.a.sc * 2;  // == BS * g.b.sc * 2 only if the leading dimensions agree
@@ -279,17 +291,23 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj)
       if (b_valid[jj])
-        load16_to_lds(bp, (RAGGED && red_tail) ? b_lane_t[jj] : b_lane[jj], st + (wave * 4 + jj) * 1024);
+        {
+        uint32_t off = b_lane[jj];
+        if (RAGGED) off += red_tail ? b_delta_k[jj] : 0u;
+        load16_to_lds(bp, off, st + (wave * 4 + jj) * 1024);
+      }
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      if (fl & (1u << r))
-        load16_to_lds(ap + r * a_rstride, (RAGGED && (red_tail || r == r_tail)) ? a_lane_t : a_lane,
-                      st + A_OFF + r * TILE + wave * 1024);
+      if (fl & (1u << r)) {
+        uint32_t off = a_lane;
+        if (RAGGED) off += (r == r_tail ? a_delta_m : 0u) + (red_tail ? a_delta_k : 0u);
+        load16_to_lds(ap + r * a_rstride, off, st + A_OFF + r * TILE + wave * 1024);
+      }
   };
   // zeroes the elements of a fragment whose reduction index (16*ks + 8*(lane/32) + 0..7 inside the
-  // block) is not below tail_valid
+  // block) is not below k_valid
   auto mask_fragment = [&](u32x4& f, int ks) {
-    const int n = tail_valid - (16 * ks + 8 * (lane / 32));  // valid elements among the lane's 8
+    const int n = k_valid - (16 * ks + 8 * (lane / 32));  // valid elements among the lane's 8
     f.x &= n >= 2 ? ~0u : (n == 1 ? 0xffffu : 0u);
     f.y &= n >= 4 ? ~0u : (n == 3 ? 0xffffu : 0u);
     f.z &= n >= 6 ? ~0u : (n == 5 ? 0xffffu : 0u);
@@ -356,7 +374,7 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
         read_a(at0 + ((u + 1) / 4) * TILE, ks1, af[(u + 1) & 1]);
       }
       __builtin_amdgcn_sched_barrier(0);
-      if (RAGGED && TRANS && red_tail) {  // ragged reduction block: nothing past the end may reach the MFMAs
+      if (RAGGED && red_tail) {  // ragged reduction block: nothing past the end may reach the MFMAs
         mask_fragment(af[u & 1][0], ks);
         mask_fragment(af[u & 1][1], ks);
         if (u < 4) {
@@ -420,7 +438,7 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
           const int lane_i = lane % 32;
           const int64_t m = (int64_t)rb * BS + mt * 32 + (CM ? lane_i : reg_i);
           const int64_t n = n0 + ns * 64 + nt * 32 + (CM ? reg_i : lane_i);
-          if (RAGGED && m >= g.M) continue;  // ragged last row block
+          if (RAGGED && (m >= g.M || n >= g.N)) continue;  // ragged last row block / column slice
           if (part)  // unscaled fp32 partial in C's own element order; the reduce pass scales and rounds
             part[CM ? n * g.M + m : m * g.N + n] = acc[rr][mt][nt][v];
           else
@@ -450,7 +468,11 @@ constexpr int G_STAGE = (R + GW) * TILE;   // 80 KB
 constexpr int G_SMEM = 2 * G_STAGE;        // all of the 160 KB; everything else lives in registers
 constexpr int G_MAX_CB = 32768;            // per-column flags share the first stage before the loads start
 
-template <typename T>
+// EDGE = the output width or the reduction length is not a multiple of 64 (both multiples of 8): the
+// overhanging 16-byte chunks / rows of the last column block / reduction block are fetched from inside the
+// matrix instead, as in the DSD kernel, the fragments of the last reduction block are zeroed past the end,
+// and nothing is stored past the last column.  (A ragged M costs nothing worth a separate instance.)
+template <typename T, bool EDGE>
 __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tiles_m, int gmax, int Mb,
                                                             int Cb) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -564,7 +586,7 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
       const uint32_t f = (uint32_t)__builtin_amdgcn_readfirstlane((int)flags[c]);
       for (int r = 0; r < R; ++r) {
         if (rb0 + r >= Mb) break;
-        if (!((f >> r) & 1u) && (int64_t)(rb0 + r) * BS + row < g.M)
+        if (!((f >> r) & 1u) && (int64_t)(rb0 + r) * BS + row < g.M && (!EDGE || (int64_t)c * BS + ch * 8 < g.N))
           *reinterpret_cast<u32x4*>(g.c + ((int64_t)(rb0 + r) * BS + row) * g.c_sr + (int64_t)c * BS + ch * 8) = z;
       }
     }
@@ -585,22 +607,41 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
       b_off[ks] = (16 * ks + row) * 128 + b_ch * 16 + (j % 2) * 8;           // ^ 64 for the second 32 columns
     }
   }
-  const int nsteps = (int)(g.K / BS);
+  const int nsteps = (int)((g.K + BS - 1) / BS);
   // loads: wave-uniform tile bases plus this lane's 16 bytes of the wave's 8 tile rows
   const char* a_base = reinterpret_cast<const char*>(g.a.ptr + (int64_t)rb0 * BS * g.a.sr);
   const char* b_base = reinterpret_cast<const char*>(g.b.ptr);
   // M need not be a multiple of 64: rows of the last row block past M are fetched from its last valid row
   // (rows are independent, theirs are never stored)
-  uint32_t a_lane, a_lane_t, b_lane;
-  const int r_tail = (g.M % BS) ? Mb - 1 - rb0 : -1;
+  const int m_valid = (int)(g.M % BS), n_valid = (int)(g.N % BS), k_valid = (int)(g.K % BS);
+  const int r_tail = m_valid ? Mb - 1 - rb0 : -1;
+  const int c_tail = (EDGE && n_valid) ? Cb - 1 : -1;        // column block that is ragged
+  const int s_tail = (EDGE && k_valid) ? nsteps - 1 : -1;    // reduction block that is ragged
+  uint32_t a_lane, a_lane_m, b_lane;
+  // EDGE: what to add (mod 2^32) to a lane's offset for a ragged reduction block / column block; the row and
+  // the chunk term of an offset are redirected independently, so the corrections add up
+  uint32_t a_delta_k, b_delta_c, b_delta_k;
   {
     const int row = wave * 8 + lane / 8;
     const int pch = lane % 8;
-    a_lane = (uint32_t)(row * g.a.sr + (pch ^ ((row >> 1) & 7)) * 8) * 2u;
-    const int valid = (int)(g.M % BS);
-    const int rc = (r_tail >= 0 && row >= valid) ? valid - 1 : row;
-    a_lane_t = (uint32_t)(rc * g.a.sr + (pch ^ ((row >> 1) & 7)) * 8) * 2u;
-    b_lane = (uint32_t)(row * g.b.sc + (pch ^ (((row >> 1) & 1) << 2)) * 8) * 2u;
+    auto a_at = [&](bool clamp_m, bool clamp_k) {
+      const int rc = (clamp_m && row >= m_valid) ? m_valid - 1 : row;
+      int c = pch ^ ((row >> 1) & 7);
+      if (clamp_k && c * 8 >= k_valid) c = 0;
+      return (uint32_t)(rc * g.a.sr + c * 8) * 2u;
+    };
+    auto b_at = [&](bool clamp_c, bool clamp_k) {  // rows of a W tile are reduction indices
+      const int rc = (clamp_k && row >= k_valid) ? k_valid - 1 : row;
+      int c = pch ^ (((row >> 1) & 1) << 2);
+      if (clamp_c && c * 8 >= n_valid) c = 0;
+      return (uint32_t)(rc * g.b.sc + c * 8) * 2u;
+    };
+    a_lane = a_at(false, false);
+    a_lane_m = a_at(r_tail >= 0, false);
+    a_delta_k = a_at(false, s_tail >= 0) - a_lane;
+    b_lane = b_at(false, false);
+    b_delta_c = b_at(c_tail >= 0, false) - b_lane;
+    b_delta_k = b_at(false, s_tail >= 0) - b_lane;
   }
   const int64_t a_tile_stride = (int64_t)BS * g.a.sr * 2;
   const int64_t b_step_stride = (int64_t)BS * g.b.sc * 2;
@@ -608,12 +649,30 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
     char* st = smem + stage * G_STAGE + wave * 1024;
     const char* ap = a_base + step * (BS * 2);
     const char* bp = b_base + step * b_step_stride;
+    const bool red_tail = EDGE && step == s_tail;
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      if (rowmask & (1u << r)) load16_to_lds(ap + r * a_tile_stride, r == r_tail ? a_lane_t : a_lane, st + r * TILE);
+      if (rowmask & (1u << r)) {
+        uint32_t off = r == r_tail ? a_lane_m : a_lane;
+        if (EDGE) off += red_tail ? a_delta_k : 0u;
+        load16_to_lds(ap + r * a_tile_stride, off, st + r * TILE);
+      }
 #pragma unroll
     for (int j = 0; j < GW; ++j)
-      if (j < ncols) load16_to_lds(bp + (int64_t)cols[j] * (BS * 2), b_lane, st + G_BOFF + j * TILE);
+      if (j < ncols) {
+        uint32_t off = b_lane;
+        if (EDGE) off += (cols[j] == c_tail ? b_delta_c : 0u) + (red_tail ? b_delta_k : 0u);
+        load16_to_lds(bp + (int64_t)cols[j] * (BS * 2), off, st + G_BOFF + j * TILE);
+      }
+  };
+  // zeroes the elements of a fragment whose reduction index (16*ks + 8*(lane/32) + 0..7 inside the
+  // block) is not below k_valid
+  auto mask_fragment = [&](u32x4& f, int ks) {
+    const int n = k_valid - (16 * ks + 8 * (lane / 32));
+    f.x &= n >= 2 ? ~0u : (n == 1 ? 0xffffu : 0u);
+    f.y &= n >= 4 ? ~0u : (n == 3 ? 0xffffu : 0u);
+    f.z &= n >= 6 ? ~0u : (n == 5 ? 0xffffu : 0u);
+    f.w &= n >= 8 ? ~0u : (n == 7 ? 0xffffu : 0u);
   };
   // the two waves of a SIMD (w and w + 4) issue their loads half a step apart
   const bool late = wave >= 4;
@@ -654,8 +713,16 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
           bf[u & 1][h] = u32x4{lo.x, lo.y, hi.x, hi.y};
         }
       };
+      const bool red_tail = EDGE && step == s_tail;
       auto mfma_unit = [&](auto k_c, int u) {
         constexpr int k = decltype(k_c)::value;
+        if (EDGE && red_tail) {  // nothing past the end of the reduction may reach the MFMAs
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            mask_fragment(af[u & 1][h], u % 4);
+            mask_fragment(bf[u & 1][h], u % 4);
+          }
+        }
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -696,7 +763,7 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
         for (int v = 0; v < 16; ++v) {
           const int64_t m = (int64_t)(rb0 + my_r[k]) * BS + mt * 32 + 8 * (v / 4) + 4 * (lane / 32) + (v % 4);
           const int64_t n = (int64_t)my_c[k] * BS + nt * 32 + (lane % 32);
-          if (m < g.M) g.c[m * g.c_sr + n] = T::from_float(acc[k][mt][nt][v] * g.scale);
+          if (m < g.M && (!EDGE || n < g.N)) g.c[m * g.c_sr + n] = T::from_float(acc[k][mt][nt][v] * g.scale);
         }
   }
 }
@@ -735,18 +802,18 @@ int launch_dsd_r(const GemmArgs& g, int splits, hipStream_t stream) {
 
 template <typename T, bool TRANS, bool CM>
 int launch_dsd(const GemmArgs& g, int splits, hipStream_t stream) {
-  const bool ragged = TRANS ? (g.K % BS != 0) : (g.M % BS != 0);
+  const bool ragged = g.M % BS != 0 || g.N % BS != 0 || g.K % BS != 0;
   return ragged ? launch_dsd_r<T, TRANS, CM, true>(g, splits, stream)
                 : launch_dsd_r<T, TRANS, CM, false>(g, splits, stream);
 }
 
-template <typename T>
+template <typename T, bool EDGE>
 int launch_sdd_group(const GemmArgs& g, hipStream_t stream) {
   static bool configured[kMaxDevices] = {};
-  if (int rc = allow_big_lds(reinterpret_cast<const void*>(&sdd_group_kernel<T>), G_SMEM, configured)) return rc;
-  const int Mb = (int)((g.M + BS - 1) / BS), Cb = (int)(g.N / BS);
+  if (int rc = allow_big_lds(reinterpret_cast<const void*>(&sdd_group_kernel<T, EDGE>), G_SMEM, configured)) return rc;
+  const int Mb = (int)((g.M + BS - 1) / BS), Cb = (int)((g.N + BS - 1) / BS);
   const int tiles_m = (Mb + R - 1) / R, gmax = (Cb + R - 1) / R;
-  hipLaunchKernelGGL(sdd_group_kernel<T>, dim3((unsigned)(tiles_m * gmax)), dim3(THREADS), G_SMEM, stream, g,
+  hipLaunchKernelGGL((sdd_group_kernel<T, EDGE>), dim3((unsigned)(tiles_m * gmax)), dim3(THREADS), G_SMEM, stream, g,
                      tiles_m, gmax, Mb, Cb);
   return check_launch("sdd_group_kernel");
 }
@@ -754,14 +821,17 @@ int launch_sdd_group(const GemmArgs& g, hipStream_t stream) {
 int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
   if (g.row_ptr && g.bs != BS) return SD_ERR_UNSUPPORTED;
   const bool layout_ok = g.a.sc == 1 && g.b.sr == 1 && g.b.sc != 1 && g.c_sc == 1;
-  const bool shape_ok = g.M > 0 && g.N > 0 && g.N % BS == 0 && g.K > 0 && g.K % BS == 0;  // any M
+  const bool shape_ok = g.M > 0 && g.N > 0 && g.N % 8 == 0 && g.K > 0 && g.K % 8 == 0;  // any M
   const bool align_ok = aligned16(g.a.ptr) && aligned16(g.b.ptr) && aligned16(g.c) && g.a.sr % 8 == 0 &&
                         g.b.sc % 8 == 0 && g.c_sr % 8 == 0 && g.a.sr < (1 << 22) &&
                         g.b.sc < (1 << 22);  // per-lane byte offsets are 32-bit
-  const int64_t tiles = (((g.M + BS - 1) / BS + R - 1) / R) * ((g.N / BS + R - 1) / R);
+  const int64_t Cb = (g.N + BS - 1) / BS;
+  const int64_t tiles = (((g.M + BS - 1) / BS + R - 1) / R) * ((Cb + R - 1) / R);
   if (!layout_ok || !shape_ok || !align_ok || tiles > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
-  if (g.N / BS > G_MAX_CB) return SD_ERR_UNSUPPORTED;
-  return dtype == SD_BF16 ? launch_sdd_group<BF16>(g, stream) : launch_sdd_group<F16>(g, stream);
+  if (Cb > G_MAX_CB) return SD_ERR_UNSUPPORTED;
+  const bool edge = g.N % BS != 0 || g.K % BS != 0;
+  if (dtype == SD_BF16) return edge ? launch_sdd_group<BF16, true>(g, stream) : launch_sdd_group<BF16, false>(g, stream);
+  return edge ? launch_sdd_group<F16, true>(g, stream) : launch_sdd_group<F16, false>(g, stream);
 }
 
 }  // namespace
@@ -776,9 +846,9 @@ int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   const bool nt = g.a.sc == 1 && g.b.sc == 1;         // reduction-contiguous operands
   const bool tn = !nt && g.a.sr == 1 && g.b.sr == 1;  // reduction-strided operands
   const bool cm = g.c_sc != 1;                        // column-major C
-  // ragged edges: the rows of a reduction-contiguous A (M), the reduction length of reduction-strided operands (K)
-  const bool shape_ok = g.M > 0 && (nt || g.M % BS == 0) && g.N > 0 && g.N % BS == 0 && g.K > 0 &&
-                        (tn || g.K % BS == 0) && (g.K + BS - 1) / BS < 65536;
+  // ragged edges: any extent along a strided index, multiples of 8 (the 16 bytes of a load) along a contiguous one
+  const bool shape_ok = g.M > 0 && (nt || g.M % 8 == 0) && g.N > 0 && (nt || g.N % 8 == 0) && g.K > 0 &&
+                        (tn || g.K % 8 == 0) && (g.K + BS - 1) / BS < 65536;
   const int64_t lda = nt ? g.a.sr : g.a.sc, ldb = nt ? g.b.sr : g.b.sc;
   const bool align_ok = aligned16(g.a.ptr) && aligned16(g.b.ptr) && lda % 8 == 0 && ldb % 8 == 0 &&
                         lda < (1 << 22) && ldb < (1 << 22);  // per-lane byte offsets are 32-bit

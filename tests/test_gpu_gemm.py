@@ -315,12 +315,16 @@ def test_sdd_column_groups(M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(1000, 256, 512), (19700 // 4, 384, 768), (70, 128, 192), (4097, 512, 256),
-                                   (8200, 128, 576)])
+                                   (8200, 128, 576),
+                                   # feature dimensions that are multiples of 8 but not of 64
+                                   (4096, 1024, 784), (1000, 1000, 1000), (70, 72, 200), (256, 264, 72),
+                                   (300, 8, 8), (8200, 72, 200), (130, 320, 56), (64, 64, 4104)])
 @pytest.mark.parametrize("p", [0.0, 0.5])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_ragged_row_count_stays_on_the_specialised_kernels(M, N, K, p, dtype):
-    """M (batch x sequence) is rarely a multiple of 64: forward, dX and the row-major dW all run on the
-    specialised kernels with a ragged last row block, and match the oracle."""
+def test_ragged_shapes_stay_on_the_specialised_kernels(M, N, K, p, dtype):
+    """M (batch x sequence) is rarely a multiple of 64, and feature counts such as 784 or 1000 are not either:
+    forward, dX and dW all run on the specialised kernels with ragged last blocks along any of M, N, K
+    (any M; N and K multiples of 8, the 16 bytes of one load), and match the oracle."""
     from flash_dropout.hip import GEMM
 
     ext = GEMM()
@@ -337,8 +341,11 @@ def test_ragged_row_count_stays_on_the_specialised_kernels(M, N, K, p, dtype):
     assert ext.last_kernel() == "specialised"
     dB = ext.gemm_dsd_lists(A.T, dC.T, lists.transposed(), 64, s, transposed_out=True).T
     assert ext.last_kernel() == "specialised"
+    dBt = ext.gemm_dsd_lists(A.T, dC.T, lists.transposed(), 64, s)  # [K, N] row-major
+    assert ext.last_kernel() == "specialised"
     rC, rdA, rdB = _oracle_products(A, B, dC, mk, 64, p)
-    for got, ref, what in ((C, rC, "C"), (dA, rdA, "dA"), (dB, rdB, "dB")):
+    for got, ref, what in ((C, rC, "C"), (dA, rdA, "dA"), (dB, rdB, "dB"), (dBt, rdB.T, "dBt")):
+        assert tuple(got.shape) == ref.shape, what
         assert rel_fro(got, ref) <= REL_FRO_TOL, what
     keep = O.expand_keep(mk.numpy(), 64, M, K)
     assert (to_np(dA)[~keep] == 0).all()
