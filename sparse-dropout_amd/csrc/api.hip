@@ -116,6 +116,8 @@ const char* sd_last_error(void) { return last_error_buf(); }
 
 const char* sd_last_kernel(void) { return last_kernel; }
 
+int sd_set_tile_policy(int policy) { return sd::set_tile_policy(policy); }
+
 int64_t sd_workspace_bytes(int64_t mb, int64_t kb) {
   if (mb < 0 || kb < 0) return 0;
   // row_ptr[mb+1] then col_idx[mb*kb], the first padded to a 16-byte boundary

@@ -121,5 +121,9 @@ int fast_splits(int64_t M, int64_t N, int64_t K);
 int launch_splitk_reduce(const GemmArgs& g, int splits, bool trans_out, int dtype, hipStream_t stream);
 // returns SD_ERR_UNSUPPORTED (without setting an error message) when the fast path does not apply
 int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream);
+// which workgroup shape the DSD kernel runs in: chosen from the shape, or forced (tuning and tests);
+// returns the previous policy, -1 for an unknown one
+enum { kTileAuto = 0, kTileBig = 1, kTileMid = 2 };
+int set_tile_policy(int policy);
 
 }  // namespace sd

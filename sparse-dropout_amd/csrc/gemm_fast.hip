@@ -32,6 +32,7 @@
 // Only kept output tiles are computed; the reduction (over N) is dense.  dY tiles are reduction-contiguous
 // (swizzled as in the forward), W tiles reduction-strided (read with ds_read_b64_tr_b16 as in dW).  See
 // sdd_group_kernel for how tiles are grouped into workgroups; dropped tiles are written as zeros.
+#include <atomic>
 #include <type_traits>
 
 #include "common.h"
@@ -44,15 +45,35 @@ constexpr int BS = 64;        // mask block = tile edge along M and K
 constexpr int BN = 256;       // output columns per workgroup
 constexpr int THREADS = 512;  // 8 waves
 constexpr int TILE = BS * BS * 2;              // bytes of one 64 x 64 tile (rows of 128 B)
-constexpr int STAGE = (BN / BS) * TILE + R * TILE;  // W tile (32 KB) + up to 4 X tiles (32 KB)
-constexpr int A_OFF = (BN / BS) * TILE;
 constexpr int MAX_STEPS = 1024;
 // step table: one uint32 per step of the union walk, reduction block | keep flags << 16, followed by
 // STEP_PAD zero entries so that look-ahead reads past the end are harmless
 constexpr int STEP_PAD = 4;
-constexpr int SMEM_STEPS = 2 * STAGE;
-constexpr int SMEM_SCRATCH = SMEM_STEPS + 4 * (MAX_STEPS + STEP_PAD);  // uint32 per K block while merging
-constexpr int SMEM_BYTES = SMEM_SCRATCH + 4 * MAX_STEPS + 16;
+// Shape of a DSD workgroup: RH pairs of row blocks x NS column slices of NT 32-column MFMA tiles; wave
+// (rh, ns) multiplies its slice of the W tile with the kept X tiles of its pair.
+//   DsdBig  256 rows x 256 columns, 8 waves: the least operand traffic per MFMA; what large products run on
+//   DsdMid  128 rows x 128 columns, 4 waves: four times as many workgroups, for products whose 256 x 256
+//           tiles would leave most of the 256 CUs without one.  A wave's 128 x 32 slice needs 1.25 KB of
+//           LDS fragment reads per MFMA against 0.75 KB in the big shape, which is what bounds it
+template <int RH_, int NS_, int NT_>
+struct DsdShape {
+  static constexpr int RH = RH_, NS = NS_, NT = NT_;
+  static constexpr int R = 2 * RH;           // row blocks per workgroup
+  static constexpr int NW = RH * NS;         // waves
+  static constexpr int THREADS = 64 * NW;
+  static constexpr int BN = NS * NT * 32;    // output columns per workgroup
+  static constexpr int B_TILE = BN * BS * 2; // bytes of the W tile of one step
+  static constexpr int A_OFF = B_TILE;       // X tiles follow it
+  static constexpr int STAGE = B_TILE + R * TILE;
+  static constexpr int BL = B_TILE / 1024 / NW;  // wave-wide 1 KB loads per wave for the W tile
+  static constexpr int AL = TILE / 1024 / NW;    // ... for one X tile
+  static constexpr int SMEM_STEPS = 2 * STAGE;
+  static constexpr int SMEM_SCRATCH = SMEM_STEPS + 4 * (MAX_STEPS + STEP_PAD);  // uint32 per K block while merging
+  static constexpr int SMEM_BYTES = SMEM_SCRATCH + 4 * MAX_STEPS + 16;
+  static_assert(BL >= 1 && AL >= 1 && BL * NW * 1024 == B_TILE && AL * NW * 1024 == TILE, "loads must divide evenly");
+};
+using DsdBig = DsdShape<2, 4, 2>;
+using DsdMid = DsdShape<1, 4, 1>;
 __device__ inline int step_block(uint32_t e) { return (int)(e & 0xffffu); }
 __device__ inline uint32_t step_flags(uint32_t e) { return e >> 16; }
 __device__ inline uint32_t uniform(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane(v); }
@@ -117,21 +138,23 @@ __device__ inline u32x2 lds_read_tr(const char* p) {
 // CM = C is column-major: the MFMA operands are swapped so that lanes run along C's rows
 // RAGGED = some of M, N, K is not a multiple of 64; a separate instance so that the aligned case carries
 // none of the edge handling
-template <typename T, bool TRANS, bool CM, bool RAGGED>
-__global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, int tiles_n,
-                                                      int Mb, int Kb_all) {
+template <typename T, bool TRANS, bool CM, bool RAGGED, typename S>
+__global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m, int tiles_n,
+                                                         int Mb, int Kb_all) {
+  constexpr int R = S::R, BN = S::BN, THREADS = S::THREADS, NT = S::NT, STAGE = S::STAGE, A_OFF = S::A_OFF;
+  constexpr int BL = S::BL, AL = S::AL;
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  uint32_t* step_e = reinterpret_cast<uint32_t*>(smem + SMEM_STEPS);
-  uint32_t* scratch = reinterpret_cast<uint32_t*>(smem + SMEM_SCRATCH);
-  int* nsteps_p = reinterpret_cast<int*>(smem + SMEM_SCRATCH + 4 * MAX_STEPS);
+  uint32_t* step_e = reinterpret_cast<uint32_t*>(smem + S::SMEM_STEPS);
+  uint32_t* scratch = reinterpret_cast<uint32_t*>(smem + S::SMEM_SCRATCH);
+  int* nsteps_p = reinterpret_cast<int*>(smem + S::SMEM_SCRATCH + 4 * MAX_STEPS);
 
   int tm, tn;
   tile_of_block<DSD_GROUP_M>(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int tid = threadIdx.x;
   const int lane = tid % 64;
   const int wave = tid / 64;
-  const int ns = wave % 4;  // 64-column slice
-  const int rh = wave / 4;  // row-block pair
+  const int ns = wave % S::NS;  // column slice
+  const int rh = wave / S::NS;  // row-block pair
   const int rb0 = tm * R;   // first row block
   const int64_t n0 = (int64_t)tn * BN;
   const int nvalid = (int)((g.N - n0) < BN ? (g.N - n0) : BN);  // columns of this tile inside C
@@ -153,7 +176,7 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
       }
     }
   } else {
-    const uint32_t all = (rb0 + R <= Mb) ? 0xfu : ((1u << (Mb - rb0)) - 1u);
+    const uint32_t all = (rb0 + R <= Mb) ? ((1u << R) - 1u) : ((1u << (Mb - rb0)) - 1u);
     for (int i = tid; i < Kb; i += THREADS) scratch[i] = all;
   }
   __syncthreads();
@@ -188,7 +211,7 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
     for (int ks = 0; ks < 4; ++ks) {
       const int ko = ((2 * ks + lane / 32) ^ fr_sw) * 16;
       a_off[ks] = fr_row * 128 + ko;
-      b_off[ks] = (ns * 64 + fr_row) * 128 + ko;
+      b_off[ks] = (ns * 32 * NT + fr_row) * 128 + ko;
     }
   } else {
     // rows are reduction indices.  16-lane group b = lane/16, lane = 16b + 4e + j reads 8 bytes of
@@ -198,19 +221,19 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
     const int colchunk = 2 * (b4 % 2) + j / 2;  // 16 B chunk inside a 32-column tile
     // X tile rows are 128 B (8 chunks): physical chunk = logical ^ (((row>>1)&1)<<2)
     const int a_ch = colchunk ^ (((e >> 1) & 1) << 2);
-    // W tile rows are 512 B (32 chunks): physical chunk = logical ^ ((row&3)<<2)
-    const int b_ch = (ns * 8 + colchunk) ^ (e << 2);
+    // W tile rows are 2*BN bytes (32 or 16 chunks): physical chunk = logical ^ ((row&3)<<2)
+    const int b_ch = (ns * 4 * NT + colchunk) ^ (e << 2);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       a_off[ks] = (16 * ks + row) * 128 + a_ch * 16 + (j % 2) * 8;
-      b_off[ks] = (16 * ks + row) * 512 + b_ch * 16 + (j % 2) * 8;
+      b_off[ks] = (16 * ks + row) * (2 * BN) + b_ch * 16 + (j % 2) * 8;
     }
   }
 
   // global -> LDS: every wave-wide load fills 1 KB of LDS in lane order.  Per-lane byte offsets are
   // fixed for the whole kernel; per step only a wave-uniform base moves.
-  uint32_t b_lane[4], a_lane;
-  bool b_valid[4];  // the lane's 16 bytes of the W tile lie inside the matrix (a tile may overhang N)
+  uint32_t b_lane[BL], a_lane[AL];
+  bool b_valid[BL];  // the lane's 16 bytes of the W tile lie inside the matrix (a tile may overhang N)
   // Ragged edges (all in units of 8 elements, the 16 bytes of one lane's load).  A 64-block that overhangs
   // the matrix along the strided index of its operand is fetched with the overhanging rows redirected to
   // its last valid row; one that overhangs along the contiguous index with the overhanging 16-byte chunks
@@ -223,7 +246,7 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
   const int kb_tail = (RAGGED && k_valid) ? Kb_all - 1 : -1;    // reduction block that is ragged
   // what to add (mod 2^32) to a lane's offset for a block ragged along M / along the reduction: the row and
   // the chunk term of an offset are redirected independently, so the two corrections add up
-  uint32_t a_delta_m, a_delta_k, b_delta_k[4];
+  uint32_t a_delta_m[AL], a_delta_k[AL], b_delta_k[BL];
   const char* a_tile0;  // first X tile of the patch at reduction block 0
   const char* b_tile0;  // W tile at reduction block 0
   int64_t red_stride;   // bytes between consecutive reduction blocks
@@ -239,41 +262,48 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
       return (uint32_t)(rc * ld + c * 8) * 2u;
     };
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) {
-      const int row = (wave * 4 + jj) * 8 + ld_row;
+    for (int jj = 0; jj < BL; ++jj) {
+      const int row = (wave * BL + jj) * 8 + ld_row;
       b_lane[jj] = chunk_at(row, g.b.sr, 0, false, false);
       b_delta_k[jj] = chunk_at(row, g.b.sr, 0, false, kb_tail >= 0) - b_lane[jj];
       b_valid[jj] = row < nvalid;
     }
-    const int row = wave * 8 + ld_row;
-    a_lane = chunk_at(row, g.a.sr, 0, false, false);
-    a_delta_m = chunk_at(row, g.a.sr, m_valid, r_tail >= 0, false) - a_lane;
-    a_delta_k = chunk_at(row, g.a.sr, 0, false, kb_tail >= 0) - a_lane;
+#pragma unroll
+    for (int i = 0; i < AL; ++i) {
+      const int row = (wave * AL + i) * 8 + ld_row;
+      a_lane[i] = chunk_at(row, g.a.sr, 0, false, false);
+      a_delta_m[i] = chunk_at(row, g.a.sr, m_valid, r_tail >= 0, false) - a_lane[i];
+      a_delta_k[i] = chunk_at(row, g.a.sr, 0, false, kb_tail >= 0) - a_lane[i];
+    }
     a_tile0 = reinterpret_cast<const char*>(g.a.ptr + (int64_t)rb0 * BS * g.a.sr);
     b_tile0 = reinterpret_cast<const char*>(g.b.ptr + n0 * g.b.sr);
     red_stride = BS * 2;
     a_rstride = (uint32_t)(BS * g.a.sr) * 2u;
   } else {
-    // W tile: 2 reduction rows of 512 B per load; X tiles: 8 reduction rows of 128 B per load
+    // W tile: reduction rows of 2*BN bytes, 2 or 4 of them per load; X tiles: 8 reduction rows of 128 B per load
+    constexpr int CPR = BN / 8;  // 16-byte chunks per W tile row
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) {
-      const int row = (wave * 4 + jj) * 2 + lane / 32;
-      const int col = ((lane % 32) ^ ((row & 3) << 2)) * 8;
+    for (int jj = 0; jj < BL; ++jj) {
+      const int row = (wave * BL + jj) * (64 / CPR) + lane / CPR;
+      const int col = ((lane % CPR) ^ ((row & 3) << 2)) * 8;
       b_lane[jj] = (uint32_t)(row * g.b.sc + col) * 2u;
       b_valid[jj] = col < nvalid;
       const int rc = (kb_tail >= 0 && row >= k_valid) ? k_valid - 1 : row;
       b_delta_k[jj] = (uint32_t)(rc * g.b.sc + col) * 2u - b_lane[jj];
     }
-    const int row = wave * 8 + lane / 8;
-    auto chunk_at = [&](bool clamp_m, bool clamp_k) {
+    auto chunk_at = [&](int row, bool clamp_m, bool clamp_k) {
       const int rc = (clamp_k && row >= k_valid) ? k_valid - 1 : row;
       int c = (lane % 8) ^ (((row >> 1) & 1) << 2);
       if (clamp_m && c * 8 >= m_valid) c = 0;
       return (uint32_t)(rc * g.a.sc + c * 8) * 2u;
     };
-    a_lane = chunk_at(false, false);
-    a_delta_m = chunk_at(r_tail >= 0, false) - a_lane;
-    a_delta_k = chunk_at(false, kb_tail >= 0) - a_lane;
+#pragma unroll
+    for (int i = 0; i < AL; ++i) {
+      const int row = (wave * AL + i) * 8 + lane / 8;
+      a_lane[i] = chunk_at(row, false, false);
+      a_delta_m[i] = chunk_at(row, r_tail >= 0, false) - a_lane[i];
+      a_delta_k[i] = chunk_at(row, false, kb_tail >= 0) - a_lane[i];
+    }
     a_tile0 = reinterpret_cast<const char*>(g.a.ptr + (int64_t)rb0 * BS);
     b_tile0 = reinterpret_cast<const char*>(g.b.ptr + n0);
     red_stride = (int64_t)BS * g.a.sc * 2;  // == BS * g.b.sc * 2 only if the leading dimensions agree
@@ -289,19 +319,21 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
     const char* ap = a_tile0 + kb * red_stride;
     const bool red_tail = RAGGED && kb == kb_tail;  // wave-uniform
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj)
-      if (b_valid[jj])
-        {
+    for (int jj = 0; jj < BL; ++jj)
+      if (b_valid[jj]) {
         uint32_t off = b_lane[jj];
         if (RAGGED) off += red_tail ? b_delta_k[jj] : 0u;
-        load16_to_lds(bp, off, st + (wave * 4 + jj) * 1024);
+        load16_to_lds(bp, off, st + (wave * BL + jj) * 1024);
       }
 #pragma unroll
     for (int r = 0; r < R; ++r)
       if (fl & (1u << r)) {
-        uint32_t off = a_lane;
-        if (RAGGED) off += (r == r_tail ? a_delta_m : 0u) + (red_tail ? a_delta_k : 0u);
-        load16_to_lds(ap + r * a_rstride, off, st + A_OFF + r * TILE + wave * 1024);
+#pragma unroll
+        for (int i = 0; i < AL; ++i) {
+          uint32_t off = a_lane[i];
+          if (RAGGED) off += (r == r_tail ? a_delta_m[i] : 0u) + (red_tail ? a_delta_k[i] : 0u);
+          load16_to_lds(ap + r * a_rstride, off, st + A_OFF + r * TILE + (wave * AL + i) * 1024);
+        }
       }
   };
   // zeroes the elements of a fragment whose reduction index (16*ks + 8*(lane/32) + 0..7 inside the
@@ -314,13 +346,13 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
     f.w &= n >= 8 ? ~0u : (n == 7 ? 0xffffu : 0u);
   };
 
-  f32x16 acc[2][2][2];  // [row block of the pair][m tile][n tile]
+  f32x16 acc[2][2][NT];  // [row block of the pair][m tile][n tile]
 #pragma unroll
   for (int a = 0; a < 2; ++a)
 #pragma unroll
     for (int b = 0; b < 2; ++b)
 #pragma unroll
-      for (int c = 0; c < 2; ++c)
+      for (int c = 0; c < NT; ++c)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[a][b][c][v] = 0.f;
 
@@ -338,14 +370,14 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
       }
     }
   };
-  auto read_b = [&](const char* st, int ks, u32x4 (&dst)[2][4]) {
+  auto read_b = [&](const char* st, int ks, u32x4 (&dst)[NT][4]) {
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
+    for (int nt = 0; nt < NT; ++nt) {
       if (!TRANS) {
         dst[nt][ks] = *reinterpret_cast<const u32x4*>(st + b_off[ks] + nt * 32 * 128);
       } else {
         const char* p = st + (b_off[ks] ^ (nt * 64));
-        const u32x2 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * 512);
+        const u32x2 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * 2 * BN);
         dst[nt][ks] = u32x4{lo.x, lo.y, hi.x, hi.y};
       }
     }
@@ -360,9 +392,9 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
     constexpr int MINE = decltype(mine_c)::value;
     constexpr int NR = (MINE == 3) ? 2 : 1;
     constexpr int R0 = (MINE == 2) ? 1 : 0;
-    u32x4 bf[2][4];
-    u32x4 af[2][2];
+    u32x4 bf[NT][4];
     const char* at0 = st + A_OFF + (2 * rh + R0) * TILE;
+    u32x4 af[2][2];
     read_b(st, 0, bf);
     read_a(at0, 0, af[0]);
 #pragma unroll
@@ -378,14 +410,14 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
         mask_fragment(af[u & 1][0], ks);
         mask_fragment(af[u & 1][1], ks);
         if (u < 4) {
-          mask_fragment(bf[0][ks], ks);
-          mask_fragment(bf[1][ks], ks);
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) mask_fragment(bf[nt][ks], ks);
         }
       }
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
+        for (int nt = 0; nt < NT; ++nt)
           acc[rr][mt][nt] = CM ? T::mfma32(bf[nt][ks], af[u & 1][mt], acc[rr][mt][nt])
                                : T::mfma32(af[u & 1][mt], bf[nt][ks], acc[rr][mt][nt]);
       __builtin_amdgcn_sched_barrier(0);
@@ -422,7 +454,7 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
   // ---- epilogue: scale, round once, store ---------------------------------------------------------
   // accumulator register v of lane l is element (8*(v/4) + 4*(l/32) + v%4, l%32) of the 32x32 product
   // (first MFMA operand's rows) x (second operand's rows); lanes run along C's contiguous index.
-  if (ns * 64 >= nvalid) return;  // this wave's column slice overhangs N: nothing of it is stored
+  if (ns * 32 * NT >= nvalid) return;  // this wave's column slice overhangs N: nothing of it is stored
   float* part = nsplit > 1 ? g.ws + (int64_t)split * g.M * g.N : nullptr;
 #pragma unroll
   for (int rr = 0; rr < 2; ++rr) {
@@ -431,13 +463,13 @@ __global__ __launch_bounds__(THREADS) void dsd_kernel(GemmArgs g, int tiles_m, i
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
+      for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int reg_i = 8 * (v / 4) + 4 * (lane / 32) + (v % 4);
           const int lane_i = lane % 32;
           const int64_t m = (int64_t)rb * BS + mt * 32 + (CM ? lane_i : reg_i);
-          const int64_t n = n0 + ns * 64 + nt * 32 + (CM ? reg_i : lane_i);
+          const int64_t n = n0 + ns * 32 * NT + nt * 32 + (CM ? reg_i : lane_i);
           if (RAGGED && (m >= g.M || n >= g.N)) continue;  // ragged last row block / column slice
           if (part)  // unscaled fp32 partial in C's own element order; the reduce pass scales and rounds
             part[CM ? n * g.M + m : m * g.N + n] = acc[rr][mt][nt][v];
@@ -785,26 +817,61 @@ int allow_big_lds(const void* kernel, int bytes, bool (&done)[kMaxDevices]) {
   return SD_OK;
 }
 
-template <typename T, bool TRANS, bool CM, bool RAGGED>
-int launch_dsd_r(const GemmArgs& g, int splits, hipStream_t stream) {
+template <typename T, bool TRANS, bool CM, bool RAGGED, typename S>
+int launch_dsd_s(const GemmArgs& g, int splits, hipStream_t stream) {
   static bool configured[kMaxDevices] = {};
-  if (int rc = allow_big_lds(reinterpret_cast<const void*>(&dsd_kernel<T, TRANS, CM, RAGGED>), SMEM_BYTES,
+  if (int rc = allow_big_lds(reinterpret_cast<const void*>(&dsd_kernel<T, TRANS, CM, RAGGED, S>), S::SMEM_BYTES,
                              configured))
     return rc;
   const int Mb = (int)((g.M + BS - 1) / BS), Kb = (int)((g.K + BS - 1) / BS);
-  const int tiles_m = (Mb + R - 1) / R, tiles_n = (int)((g.N + BN - 1) / BN);
-  hipLaunchKernelGGL((dsd_kernel<T, TRANS, CM, RAGGED>), dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits),
-                     dim3(THREADS), SMEM_BYTES, stream, g, tiles_m, tiles_n, Mb, Kb);
+  const int tiles_m = (Mb + S::R - 1) / S::R, tiles_n = (int)((g.N + S::BN - 1) / S::BN);
+  hipLaunchKernelGGL((dsd_kernel<T, TRANS, CM, RAGGED, S>), dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits),
+                     dim3(S::THREADS), S::SMEM_BYTES, stream, g, tiles_m, tiles_n, Mb, Kb);
   if (int rc = check_launch("dsd_kernel")) return rc;
   if (splits > 1) return launch_splitk_reduce(g, splits, CM, T::id, stream);
   return SD_OK;
 }
 
 template <typename T, bool TRANS, bool CM>
-int launch_dsd(const GemmArgs& g, int splits, hipStream_t stream) {
+int launch_dsd(const GemmArgs& g, bool mid, int splits, hipStream_t stream) {
   const bool ragged = g.M % BS != 0 || g.N % BS != 0 || g.K % BS != 0;
-  return ragged ? launch_dsd_r<T, TRANS, CM, true>(g, splits, stream)
-                : launch_dsd_r<T, TRANS, CM, false>(g, splits, stream);
+  if (mid)
+    return ragged ? launch_dsd_s<T, TRANS, CM, true, DsdMid>(g, splits, stream)
+                  : launch_dsd_s<T, TRANS, CM, false, DsdMid>(g, splits, stream);
+  return ragged ? launch_dsd_s<T, TRANS, CM, true, DsdBig>(g, splits, stream)
+                : launch_dsd_s<T, TRANS, CM, false, DsdBig>(g, splits, stream);
+}
+
+std::atomic<int> tile_policy{0};
+
+// workgroups a tile shape gives and how many ways the reduction is then split
+struct DsdPlan {
+  bool mid;
+  int splits;
+};
+template <typename S>
+int64_t dsd_tiles(int64_t M, int64_t N) {
+  return ((M + BS * S::R - 1) / (BS * S::R)) * ((N + S::BN - 1) / S::BN);
+}
+// One round of workgroups (one per CU) when the output alone gives fewer than half of that and the
+// reduction is long enough to pay for the extra pass: at least 8 reduction blocks per split.
+int splits_for(int64_t tiles, int64_t M, int64_t N, int64_t K) {
+  const int64_t kb = K / BS;
+  if (tiles >= 128 || kb < 32) return 1;
+  int64_t want = 256 / tiles;
+  if (want > kb / 8) want = kb / 8;
+  while (want > 1 && want * M * N * 4 > (256LL << 20)) --want;
+  return want < 2 ? 1 : (int)want;
+}
+DsdPlan plan_dsd(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0) return {false, 1};
+  const int policy = tile_policy.load(std::memory_order_relaxed);
+  const int64_t big = dsd_tiles<DsdBig>(M, N), midt = dsd_tiles<DsdMid>(M, N);
+  // the 256 x 256 shape whenever it gives at least half of the CUs a workgroup, and for long reductions,
+  // which it splits over workgroups (measured: 2048^3 runs 15-25 % faster on 128 x 128 tiles than on 64 big
+  // tiles x 4 splits; a 384 x 1536 weight gradient over 16384 rows 25 % slower than on 12 big tiles x 21 splits)
+  const bool mid = policy == kTileMid || (policy == kTileAuto && big < 128 && K / BS <= 64);
+  return {mid, splits_for(mid ? midt : big, M, N, K)};
 }
 
 template <typename T, bool EDGE>
@@ -852,11 +919,12 @@ int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   const int64_t lda = nt ? g.a.sr : g.a.sc, ldb = nt ? g.b.sr : g.b.sc;
   const bool align_ok = aligned16(g.a.ptr) && aligned16(g.b.ptr) && lda % 8 == 0 && ldb % 8 == 0 &&
                         lda < (1 << 22) && ldb < (1 << 22);  // per-lane byte offsets are 32-bit
-  const int64_t tiles = (((g.M + BS - 1) / BS + R - 1) / R) * ((g.N + BN - 1) / BN);
+  const DsdPlan plan = plan_dsd(g.M, g.N, g.K);
+  const int64_t tiles = plan.mid ? dsd_tiles<DsdMid>(g.M, g.N) : dsd_tiles<DsdBig>(g.M, g.N);
   if (!(nt || tn) || !shape_ok || !align_ok || tiles > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
   // few output tiles and a long reduction (the weight gradient of a tall matrix): split the reduction
   // over workgroups when the caller gave scratch for the fp32 partials
-  int splits = fast_splits(g.M, g.N, g.K);
+  int splits = plan.splits;
   const int64_t part_bytes = g.M * g.N * 4;
   if (splits > 1 && (g.ws == nullptr || g.ws_bytes < part_bytes * splits))
     splits = g.ws ? (int)(g.ws_bytes / part_bytes) : 1;
@@ -867,25 +935,20 @@ int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
     const int gs = generic_splits(g.M, g.N, g.K, g.bs, mode);
     if (gs > 1 && g.ws_bytes >= (int64_t)gs * part_bytes) return SD_ERR_UNSUPPORTED;
   }
+  const bool mid = plan.mid;
   if (dtype == SD_BF16) {
-    if (nt) return cm ? launch_dsd<BF16, false, true>(g, splits, stream) : launch_dsd<BF16, false, false>(g, splits, stream);
-    return cm ? launch_dsd<BF16, true, true>(g, splits, stream) : launch_dsd<BF16, true, false>(g, splits, stream);
+    if (nt) return cm ? launch_dsd<BF16, false, true>(g, mid, splits, stream) : launch_dsd<BF16, false, false>(g, mid, splits, stream);
+    return cm ? launch_dsd<BF16, true, true>(g, mid, splits, stream) : launch_dsd<BF16, true, false>(g, mid, splits, stream);
   }
-  if (nt) return cm ? launch_dsd<F16, false, true>(g, splits, stream) : launch_dsd<F16, false, false>(g, splits, stream);
-  return cm ? launch_dsd<F16, true, true>(g, splits, stream) : launch_dsd<F16, true, false>(g, splits, stream);
+  if (nt) return cm ? launch_dsd<F16, false, true>(g, mid, splits, stream) : launch_dsd<F16, false, false>(g, mid, splits, stream);
+  return cm ? launch_dsd<F16, true, true>(g, mid, splits, stream) : launch_dsd<F16, true, false>(g, mid, splits, stream);
 }
 
-// One round of workgroups (one per CU) when the output alone gives fewer than half of that and the
-// reduction is long enough to pay for the extra pass: at least 8 reduction blocks per split.
-int fast_splits(int64_t M, int64_t N, int64_t K) {
-  if (M <= 0 || N <= 0 || K <= 0) return 1;
-  const int64_t tiles = ((M + BS * R - 1) / (BS * R)) * ((N + BN - 1) / BN);
-  const int64_t kb = K / BS;
-  if (tiles >= 128 || kb < 32) return 1;
-  int64_t want = 256 / tiles;
-  if (want > kb / 8) want = kb / 8;
-  while (want > 1 && want * M * N * 4 > (256LL << 20)) --want;
-  return want < 2 ? 1 : (int)want;
+int set_tile_policy(int policy) {
+  if (policy != kTileAuto && policy != kTileBig && policy != kTileMid) return -1;
+  return tile_policy.exchange(policy, std::memory_order_relaxed);
 }
+
+int fast_splits(int64_t M, int64_t N, int64_t K) { return plan_dsd(M, N, K).splits; }
 
 }  // namespace sd

@@ -19,6 +19,7 @@ SIGNATURES = {
     "sd_version": (c_int, []),
     "sd_last_error": (c_char_p, []),
     "sd_last_kernel": (c_char_p, []),
+    "sd_set_tile_policy": (c_int, [c_int]),
     "sd_workspace_bytes": (c_int64, [c_int64, c_int64]),
     "sd_build_lists": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64,
                                c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),

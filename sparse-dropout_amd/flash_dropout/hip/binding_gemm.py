@@ -135,6 +135,17 @@ class GEMM:
         """"specialised" or "generic": the kernel family this thread's last GEMM call ran on."""
         return self.lib.sd_last_kernel().decode()
 
+    TILE_POLICIES = {"auto": 0, "big": 1, "mid": 2}
+
+    def set_tile_policy(self, policy: str) -> str:
+        """Workgroup shape of the specialised DSD / dense kernels for every later call of the process:
+        "auto" (from the shape), "big" (256 x 256 output tiles) or "mid" (128 x 128).  Returns the
+        previous setting.  A tuning and test hook."""
+        if policy not in self.TILE_POLICIES:
+            raise ValueError(f"tile policy {policy!r}: expected one of {sorted(self.TILE_POLICIES)}")
+        prev = self.lib.sd_set_tile_policy(self.TILE_POLICIES[policy])
+        return {v: k for k, v in self.TILE_POLICIES.items()}[prev]
+
     # ------------------------------------------------------------------ plumbing
     def _call(self, fn, *args) -> None:
         rc = fn(*args)

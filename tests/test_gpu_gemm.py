@@ -17,6 +17,18 @@ from oracle import sparsedrop_oracle as O
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True, params=["auto", "big", "mid"])
+def tile_policy(request):
+    """Every test of this file runs with the DSD workgroup shape chosen from the problem shape and with
+    each of the two shapes forced, so both are checked on every shape and edge case below."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    prev = ext.set_tile_policy(request.param)
+    yield request.param
+    ext.set_tile_policy(prev)
+
+
 def _three_products(A, B, dC, mask, bs, p):
     """The three calls exactly as the reference's autograd function issues them."""
     from flash_dropout.hip import GEMM
