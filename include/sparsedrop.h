@@ -228,6 +228,30 @@ int sd_col2im(const void* cols, int64_t cols_ld, void* dx, int64_t dx_stride_n,
               const uint8_t* mask, int64_t mask_stride_r, int64_t mask_stride_c, int64_t block_size,
               int dtype, void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Implicit-GEMM forward of the block-dropout convolution: the product sd_im2col + sd_gemm_dsd_lists
+ * compute, y[(n*P+p)*Q+q, k] = scale * sum over the kept blocks (row_ptr/col_idx, block_size 64, over the
+ * [N*P*Q / 64, ceil(C*R*S / 64)] grid of the patch matrix) of cols[m, j] * weight[k, j], without the patch
+ * matrix ever existing in memory: each workgroup keeps the input rows its 256 output positions touch in LDS
+ * and builds the kept 64 x 64 patch tiles from them.  weight is the [k_out, C*R*S] matrix (the kernel
+ * viewed as in flash_dropout/functional/im2col_conv2d.py:21-24), y is [N*P*Q, k_out] row-major with
+ * leading dimension y_ld.  This is what report.pdf section 5.3 proposes as future work; the reference has
+ * no counterpart (its conv variants are stubs, layers/dropout_conv.py:86-99).
+ *
+ * Taken: stride 1, dilation 1, unit w stride of x, W a multiple of 8, Q a divisor of 64, P*Q a multiple of
+ * 256, C*R*S a multiple of 8, R*S <= 30, and the input rows of 256 output positions (all channels) plus a
+ * column table fitting in LDS (C * (256/Q + R - 1) * W * 2 + ceil(C*R*S/64)*256 <= about 55 KB).
+ * Anything else returns SD_ERR_UNSUPPORTED with nothing launched: use sd_im2col + sd_gemm_dsd_lists.
+ * ------------------------------------------------------------------------------------------- */
+int sd_conv2d_dsd_lists(const void* x, int64_t x_stride_n, int64_t x_stride_c, int64_t x_stride_h,
+                        int64_t x_stride_w, const void* weight, int64_t weight_ld,
+                        void* y, int64_t y_ld,
+                        int64_t n, int64_t c, int64_t h, int64_t w, int64_t k_out, int64_t r, int64_t s,
+                        int64_t pad_h, int64_t pad_w, int64_t stride_h, int64_t stride_w,
+                        int64_t dil_h, int64_t dil_w,
+                        const int32_t* row_ptr, const int32_t* col_idx, int64_t block_size, float scale,
+                        int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -307,4 +307,52 @@ int sd_col2im(const void* cols, int64_t ld, void* dx, int64_t sn, int64_t sc, in
                 dil_w, mask, msr, msc, bs, dtype, (hipStream_t)stream);
 }
 
+int sd_conv2d_dsd_lists(const void* x, int64_t sn, int64_t sc, int64_t sh, int64_t sw, const void* weight,
+                        int64_t wld, void* y, int64_t yld, int64_t n, int64_t c, int64_t h, int64_t w,
+                        int64_t k_out, int64_t r, int64_t s, int64_t pad_h, int64_t pad_w, int64_t stride_h,
+                        int64_t stride_w, int64_t dil_h, int64_t dil_w, const int32_t* row_ptr,
+                        const int32_t* col_idx, int64_t bs, float scale, int dtype, void* stream) {
+  SD_REQUIRE(dtype == SD_F16 || dtype == SD_BF16, "dtype must be SD_F16 or SD_BF16 (got %d)", dtype);
+  SD_REQUIRE(x && weight && y && row_ptr && col_idx, "null pointer argument");
+  SD_REQUIRE(n > 0 && c > 0 && h > 0 && w > 0 && k_out > 0 && r > 0 && s > 0, "sizes must be positive");
+  SD_REQUIRE(stride_h > 0 && stride_w > 0 && dil_h > 0 && dil_w > 0 && pad_h >= 0 && pad_w >= 0,
+             "strides and dilations must be positive, paddings non-negative");
+  if (int rc = check_sparse(bs, scale)) return rc;
+  const int64_t P = (h + 2 * pad_h - dil_h * (r - 1) - 1) / stride_h + 1;
+  const int64_t Q = (w + 2 * pad_w - dil_w * (s - 1) - 1) / stride_w + 1;
+  SD_REQUIRE(P > 0 && Q > 0, "the kernel does not fit the padded input");
+  SD_REQUIRE(wld >= c * r * s && yld >= k_out, "leading dimensions too small");
+  if (bs != 64 || Q > 64 || 64 % Q != 0 || c * r * s > (1 << 16) || h > (1 << 20) || w > (1 << 12) || r > 64 || s > 64)
+    return SD_ERR_UNSUPPORTED;
+  ImplicitConv cg;
+  cg.x = static_cast<const uint16_t*>(x);
+  cg.sn = sn;
+  cg.sc = sc;
+  cg.sh = sh;
+  cg.C = (int)c;
+  cg.H = (int)h;
+  cg.W = (int)w;
+  cg.Q = (int)Q;
+  cg.RS = (int)(r * s);
+  cg.S = (int)s;
+  cg.pad_h = (int)pad_h;
+  cg.pad_w = (int)pad_w;
+  cg.rpb = (int)(64 / Q);
+  cg.blocks_per_img = (int)(P * Q / 64);
+  cg.PR = (int)(4 * (64 / Q) + r - 1);
+  cg.PW = (int)(w + 8);
+  cg.K = (int)(c * r * s);
+  auto magic = [](int64_t d) { return d <= 1 ? 0u : (uint32_t)(((1ull << 32) + (uint64_t)d - 1) / (uint64_t)d); };
+  cg.m_spc = magic(cg.PR * (w / 8));
+  cg.m_spr = magic(w / 8);
+  cg.m_RS = magic(r * s);
+  cg.m_S = magic(s);
+  cg.m_Q = magic(Q);
+  GemmArgs g = make_args(nullptr, 0, 0, weight, wld, 1, y, yld, 1, n * P * Q, k_out, c * r * s, bs, scale, row_ptr,
+                         col_idx);
+  const int rc = launch_conv_implicit(g, cg, P, stride_h, stride_w, dil_h, dil_w, r, sw, dtype, (hipStream_t)stream);
+  if (rc == SD_OK) last_kernel = "specialised";
+  return rc;
+}
+
 }  // extern "C"

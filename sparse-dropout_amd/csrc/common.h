@@ -108,6 +108,23 @@ struct GemmArgs {
   int64_t ws_bytes;
 };
 
+// Geometry of a stride-1, dilation-1 convolution whose patch matrix the DSD kernel gathers itself
+// (implicit GEMM): x[n][c][h][w] with unit w stride, row block = 64 / Q whole output rows of one image.
+struct ImplicitConv {
+  const uint16_t* x;
+  int64_t sn, sc, sh;  // element strides of x
+  int C, H, W, Q;      // channels, input height and width, output width
+  int RS, S;           // taps per channel, kernel width
+  int pad_h, pad_w;
+  int rpb;             // output rows per 64-row block (64 / Q)
+  int blocks_per_img;  // P * Q / 64
+  int PR;              // input rows a workgroup's 4 row blocks touch: 4 * rpb + R - 1
+  int PW;              // halfs per row of the LDS copy: 8 zeros, then the W of the image
+  int K;               // C * R * S
+  // ceil(2^32 / d) for the divisors the kernel needs (0 for d = 1): x / d == umulhi(x, m) while x * d < 2^32
+  uint32_t m_spc, m_spr, m_RS, m_S, m_Q;  // d = PR * W / 8, W / 8, R * S, S, Q
+};
+
 enum Mode { kDense = 0, kDsd = 1, kSdd = 2 };
 
 // launchers (one per translation unit)
@@ -121,6 +138,11 @@ int fast_splits(int64_t M, int64_t N, int64_t K);
 int launch_splitk_reduce(const GemmArgs& g, int splits, bool trans_out, int dtype, hipStream_t stream);
 // returns SD_ERR_UNSUPPORTED (without setting an error message) when the fast path does not apply
 int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream);
+// forward of the block-dropout convolution without the patch matrix: g.a is unused, g.b the [K_out, C*R*S]
+// weight matrix, g.c the [N*P*Q, K_out] output, the lists over the patch matrix's block grid.  Returns
+// SD_ERR_UNSUPPORTED (without an error message) for geometries it does not take.
+int launch_conv_implicit(const GemmArgs& g, const ImplicitConv& cg, int64_t P, int64_t stride_h, int64_t stride_w,
+                         int64_t dil_h, int64_t dil_w, int64_t R, int64_t x_sw, int dtype, hipStream_t stream);
 // which workgroup shape the DSD kernel runs in: chosen from the shape, or forced (tuning and tests);
 // returns the previous policy, -1 for an unknown one
 enum { kTileAuto = 0, kTileBig = 1, kTileMid = 2 };

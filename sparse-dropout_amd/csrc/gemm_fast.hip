@@ -74,6 +74,10 @@ struct DsdShape {
 };
 using DsdBig = DsdShape<2, 4, 2>;
 using DsdMid = DsdShape<1, 4, 1>;
+// 256 rows x 128 columns, 8 waves: the shape of the implicit-GEMM convolution, whose input patch has to
+// fit in LDS next to the stages
+using DsdConv = DsdShape<2, 4, 1>;
+constexpr int CONV_PATCH_MAX = 163840 - DsdConv::SMEM_BYTES - 16;  // bytes left for patch + column table
 __device__ inline int step_block(uint32_t e) { return (int)(e & 0xffffu); }
 __device__ inline uint32_t step_flags(uint32_t e) { return e >> 16; }
 __device__ inline uint32_t uniform(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane(v); }
@@ -138,9 +142,15 @@ __device__ inline u32x2 lds_read_tr(const char* p) {
 // CM = C is column-major: the MFMA operands are swapped so that lanes run along C's rows
 // RAGGED = some of M, N, K is not a multiple of 64; a separate instance so that the aligned case carries
 // none of the edge handling
-template <typename T, bool TRANS, bool CM, bool RAGGED, typename S>
+// IMPLICIT = A is the patch matrix of a convolution, never materialised: the workgroup copies the input rows
+// its 256 output positions touch (all channels) into LDS once, and per step builds the kept 64 x 64 tiles of
+// the patch matrix from that copy, in the layout the fragment reads expect, instead of loading them.  A
+// table in LDS maps a patch-matrix column (c, r, s) to its offset in the copy; whether
+// a tap falls outside the image never has to be asked: the copy carries a halo of zeros.
+template <typename T, bool TRANS, bool CM, bool RAGGED, typename S, bool IMPLICIT = false>
 __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m, int tiles_n,
-                                                         int Mb, int Kb_all) {
+                                                         int Mb, int Kb_all, ImplicitConv cg) {
+  static_assert(!IMPLICIT || (!TRANS && S::R == 4 && S::THREADS == 512), "the gather assumes 512 threads x 4 row blocks");
   constexpr int R = S::R, BN = S::BN, THREADS = S::THREADS, NT = S::NT, STAGE = S::STAGE, A_OFF = S::A_OFF;
   constexpr int BL = S::BL, AL = S::AL;
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -198,6 +208,68 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   }
   __syncthreads();
   const int nsteps = *nsteps_p;
+
+  // ---- implicit GEMM: input rows -> LDS with a zero halo, column table -------------------------------
+  // Patch layout: [channel][input row][8 zero halfs | W image halfs]; the zero group in front of a row is
+  // the left halo of that row and the right halo of the row before it, rows outside the image are zeros,
+  // so a tap never needs a bounds test: element (m, k) of the patch matrix is
+  // patch[base(m) + ktab[k]] with base(m) = (output row of m inside the workgroup) * PW + 8 + q - pad_w
+  // and ktab[k] = ((c * PR + r) * PW + s) for column k = (c, r, s), both kept as byte offsets.
+  uint16_t* patch = reinterpret_cast<uint16_t*>(smem + ((S::SMEM_BYTES + 15) & ~15));
+  uint16_t* ktab = nullptr;
+  uint32_t gat_base[4];  // byte offset of (this thread's tile row, tap 0) in the patch, per row block
+  const int gat_row = tid / 8, gat_pc = tid % 8;  // the tile row and physical 16-byte chunk this thread builds
+  if constexpr (IMPLICIT) {
+    auto div = [](int x, uint32_t magic) { return magic ? (int)__umulhi((uint32_t)x, magic) : x; };
+    const int img = rb0 / cg.blocks_per_img;
+    const int p0 = (rb0 - img * cg.blocks_per_img) * cg.rpb;  // first output row of the workgroup
+    const int h0 = p0 - cg.pad_h;                              // input row of patch row 0
+    const int spr = cg.W / 8, spc = cg.PR * spr;               // 16-byte segments per row, per channel
+    const int total = cg.C * spc;
+    const int rows = cg.C * cg.PR;
+    ktab = patch + rows * cg.PW + 8;
+    const uint16_t* ximg = cg.x + (int64_t)img * cg.sn;
+    constexpr int MAXSEG = (CONV_PATCH_MAX / 16 + THREADS - 1) / THREADS;
+    u32x4 v[MAXSEG];
+    int dst[MAXSEG];
+#pragma unroll
+    for (int j = 0; j < MAXSEG; ++j) {  // all loads first, so that their latencies overlap
+      const int seg = tid + j * THREADS;
+      const int c = div(seg, cg.m_spc), rem = seg - c * spc;
+      const int row = div(rem, cg.m_spr), w8 = rem - row * spr;
+      const int h = h0 + row;
+      dst[j] = seg < total ? (c * cg.PR + row) * cg.PW + 8 + w8 * 8 : -1;
+      v[j] = u32x4{0u, 0u, 0u, 0u};
+      if (seg < total && h >= 0 && h < cg.H)
+        v[j] = *reinterpret_cast<const u32x4*>(ximg + c * cg.sc + h * cg.sh + w8 * 8);
+    }
+    for (int m = tid; m <= rows; m += THREADS)  // the halo groups, one more after the last row
+      *reinterpret_cast<u32x4*>(patch + m * cg.PW) = u32x4{0u, 0u, 0u, 0u};
+    for (int k = tid; k < Kb_all * BS; k += THREADS) {
+      const int c = div(k, cg.m_RS), tap = k - c * cg.RS;
+      const int rr = div(tap, cg.m_S), ss = tap - rr * cg.S;
+      // columns past the last one read anything readable: their fragments are zeroed before the MFMAs
+      ktab[k] = k < cg.K ? (uint16_t)(((c * cg.PR + rr) * cg.PW + ss) * 2) : (uint16_t)0;
+    }
+    const int prow = div(gat_row, cg.m_Q), q = gat_row - prow * cg.Q;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) gat_base[r] = (uint32_t)(((r * cg.rpb + prow) * cg.PW + 8 + q - cg.pad_w) * 2);
+#pragma unroll
+    for (int j = 0; j < MAXSEG; ++j)
+      if (dst[j] >= 0) *reinterpret_cast<u32x4*>(patch + dst[j]) = v[j];
+    __syncthreads();
+  }
+  // builds this thread's 16 bytes of the patch-matrix tile (row block r of the workgroup, reduction block kb)
+  auto gather_tile = [&](int r, int kb, char* tile) {
+    const int lc = gat_pc ^ ((gat_row >> 1) & 7);  // logical chunk: columns kb*64 + lc*8 .. +7
+    const u16x8 off = *reinterpret_cast<const u16x8*>(ktab + kb * BS + lc * 8);
+    const char* pb = reinterpret_cast<const char*>(patch) + gat_base[r];
+    uint32_t v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = *reinterpret_cast<const uint16_t*>(pb + off[e]);
+    *reinterpret_cast<u32x4*>(tile + gat_row * 128 + gat_pc * 16) =
+        u32x4{v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16)};
+  };
 
   // ---- per-lane constants ---------------------------------------------------------------------
   // fragment reads
@@ -328,6 +400,10 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
 #pragma unroll
     for (int r = 0; r < R; ++r)
       if (fl & (1u << r)) {
+        if constexpr (IMPLICIT) {
+          gather_tile(r, kb, st + A_OFF + r * TILE);
+          continue;
+        }
 #pragma unroll
         for (int i = 0; i < AL; ++i) {
           uint32_t off = a_lane[i];
@@ -826,7 +902,7 @@ int launch_dsd_s(const GemmArgs& g, int splits, hipStream_t stream) {
   const int Mb = (int)((g.M + BS - 1) / BS), Kb = (int)((g.K + BS - 1) / BS);
   const int tiles_m = (Mb + S::R - 1) / S::R, tiles_n = (int)((g.N + S::BN - 1) / S::BN);
   hipLaunchKernelGGL((dsd_kernel<T, TRANS, CM, RAGGED, S>), dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits),
-                     dim3(S::THREADS), S::SMEM_BYTES, stream, g, tiles_m, tiles_n, Mb, Kb);
+                     dim3(S::THREADS), S::SMEM_BYTES, stream, g, tiles_m, tiles_n, Mb, Kb, ImplicitConv{});
   if (int rc = check_launch("dsd_kernel")) return rc;
   if (splits > 1) return launch_splitk_reduce(g, splits, CM, T::id, stream);
   return SD_OK;
@@ -901,7 +977,42 @@ int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
   return edge ? launch_sdd_group<F16, true>(g, stream) : launch_sdd_group<F16, false>(g, stream);
 }
 
+template <typename T, bool RAGGED>
+int launch_conv_t(const GemmArgs& g, const ImplicitConv& cg, int smem, hipStream_t stream) {
+  static bool configured[kMaxDevices] = {};
+  auto* kernel = &dsd_kernel<T, false, false, RAGGED, DsdConv, true>;
+  if (int rc = allow_big_lds(reinterpret_cast<const void*>(kernel), 163840, configured)) return rc;
+  const int Mb = (int)(g.M / BS), Kb = (int)((g.K + BS - 1) / BS);
+  const int tiles_m = Mb / DsdConv::R, tiles_n = (int)((g.N + DsdConv::BN - 1) / DsdConv::BN);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)(tiles_m * tiles_n), 1u), dim3(DsdConv::THREADS), smem, stream, g,
+                     tiles_m, tiles_n, Mb, Kb, cg);
+  return check_launch("dsd_kernel (implicit conv)");
+}
+
 }  // namespace
+
+int launch_conv_implicit(const GemmArgs& g, const ImplicitConv& cg, int64_t P, int64_t stride_h, int64_t stride_w,
+                         int64_t dil_h, int64_t dil_w, int64_t R, int64_t x_sw, int dtype, hipStream_t stream) {
+  if (g.bs != BS || g.row_ptr == nullptr) return SD_ERR_UNSUPPORTED;
+  const bool geom_ok = stride_h == 1 && stride_w == 1 && dil_h == 1 && dil_w == 1 && x_sw == 1 && cg.Q > 0 &&
+                       cg.Q <= BS && BS % cg.Q == 0 && (P * cg.Q) % (BS * DsdConv::R) == 0 && cg.W % 8 == 0 &&
+                       cg.pad_h >= 0 && cg.pad_w >= 0 && cg.pad_w <= 8 && cg.S - 1 - cg.pad_w <= 8 && R * cg.S == cg.RS &&
+                       cg.PW == cg.W + 8;
+  if (!geom_ok) return SD_ERR_UNSUPPORTED;
+  const int64_t patch_elems = (int64_t)cg.C * cg.PR * cg.PW + 8;  // rows with their halo groups, one more after the last
+  const int64_t Kb = (g.K + BS - 1) / BS;
+  const int64_t extra = patch_elems * 2 + Kb * BS * 2;
+  if (extra > CONV_PATCH_MAX || Kb > MAX_STEPS) return SD_ERR_UNSUPPORTED;
+  const bool align_ok = aligned16(cg.x) && cg.sn % 8 == 0 && cg.sc % 8 == 0 && cg.sh % 8 == 0 && aligned16(g.b.ptr) &&
+                        g.b.sc == 1 && g.b.sr % 8 == 0 && g.b.sr < (1 << 22) && g.c_sc == 1 && g.K % 8 == 0 &&
+                        g.M % (BS * DsdConv::R) == 0 && g.M / (BS * DsdConv::R) * ((g.N + 127) / 128) < 0x7fffffffLL;
+  if (!align_ok) return SD_ERR_UNSUPPORTED;
+  const int smem = ((DsdConv::SMEM_BYTES + 15) & ~15) + (int)extra;
+  const bool ragged = g.N % BS != 0 || g.K % BS != 0;
+  if (dtype == SD_BF16)
+    return ragged ? launch_conv_t<BF16, true>(g, cg, smem, stream) : launch_conv_t<BF16, false>(g, cg, smem, stream);
+  return ragged ? launch_conv_t<F16, true>(g, cg, smem, stream) : launch_conv_t<F16, false>(g, cg, smem, stream);
+}
 
 int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   if (mode == kSdd) return try_sdd(g, dtype, stream);

@@ -20,6 +20,11 @@ import torch.nn.functional as F
 from ..hip.binding_gemm import GEMM, KeptLists, _block_size
 
 
+# Use the implicit-GEMM forward (sd_conv2d_dsd_lists) where the library takes the geometry.  Module-level
+# switch so that tests and benchmarks can compare both routes.
+IMPLICIT_FORWARD = True
+
+
 def _pair(v) -> tuple[int, int]:
     if isinstance(v, int):
         return (v, v)
@@ -45,9 +50,16 @@ class _Im2colConv2d(torch.autograd.Function):
         if block_size:  # block dropout: mask given, or drawn in the list-building launch
             mask, lists, kernel_bs = ext.kept_lists(n * po * qo, c * r * s, block_size, mask, p, seed,
                                                     input.device)
-            cols = ext.im2col(input, (r, s), padding, stride, dilation, lists, kernel_bs)
-            y2 = ext.gemm_dsd_lists(cols, w2, lists, kernel_bs, 1.0 / (1.0 - p))
-            ctx.save_for_backward(cols, w2, mask, lists.row_ptr, lists.col_idx, lists.col_ptr, lists.row_idx)
+            # implicit GEMM where the library takes the geometry: no patch matrix in the forward, and the
+            # input is what is kept for the backward (the patch matrix is 9x its size for a 3x3 kernel)
+            y2 = ext.conv2d_dsd_lists(input, w2, lists, kernel_bs, 1.0 / (1.0 - p), (r, s), padding, stride,
+                                      dilation) if IMPLICIT_FORWARD else None
+            ctx.implicit = y2 is not None
+            if y2 is None:
+                cols = ext.im2col(input, (r, s), padding, stride, dilation, lists, kernel_bs)
+                y2 = ext.gemm_dsd_lists(cols, w2, lists, kernel_bs, 1.0 / (1.0 - p))
+            ctx.save_for_backward(input if ctx.implicit else cols, w2, mask, lists.row_ptr, lists.col_idx,
+                                  lists.col_ptr, lists.row_idx)
             ctx.list_shape = lists.shape
         else:
             cols = ext.im2col(input, (r, s), padding, stride, dilation)
@@ -74,6 +86,8 @@ class _Im2colConv2d(torch.autograd.Function):
                 dcols = ext.gemm_sdd_lists(dy2, w2.t(), lists, kernel_bs, scale)
                 dx = ext.col2im(dcols, x_shape, (r, s), padding, stride, dilation, mask, block_size, ch_last)
             if ctx.needs_input_grad[1]:
+                if ctx.implicit:  # the forward kept the input, not the patch matrix: gather the kept blocks now
+                    cols = ext.im2col(cols, (r, s), padding, stride, dilation, lists, kernel_bs)
                 dk = ext.gemm_dsd_lists(cols.t(), dy2.t(), lists.transposed(), kernel_bs, scale,
                                         transposed_out=True).t().reshape(k_shape)
         else:

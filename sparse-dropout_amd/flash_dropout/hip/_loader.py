@@ -41,6 +41,10 @@ SIGNATURES = {
                                   c_int64, c_int64, c_float, c_int, c_void_p, c_int64, c_void_p]),
     "sd_gemm_sdd_lists": (c_int, [*_mat, *_mat, *_mat, c_void_p, c_void_p, c_int64, c_int64,
                                   c_int64, c_int64, c_float, c_int, c_void_p]),
+    "sd_conv2d_dsd_lists": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64,
+                                    c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                    c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                    c_void_p, c_void_p, c_int64, c_float, c_int, c_void_p]),
     "sd_im2col": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64,
                           *([c_int64] * 12), c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "sd_col2im": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64,

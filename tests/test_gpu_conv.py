@@ -120,6 +120,82 @@ def test_blockdrop_conv_forward_backward(cfg, p):
     assert rel_fro(kg.grad, rdk) <= REL_FRO_TOL
 
 
+IMPLICIT_GEOMS = [
+    # (geometry, taken by the implicit kernel)
+    (dict(n=4, c=64, h=32, w=32, k=128, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),   # the conv configuration's layer
+    (dict(n=2, c=16, h=16, w=16, k=40, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),    # 144 columns, 40 outputs: ragged both ways; 4 output rows per block
+    (dict(n=3, c=8, h=32, w=32, k=64, r=5, s=5, padding=(2, 2), stride=(1, 1), dilation=(1, 1)), True),     # 25 taps
+    (dict(n=2, c=64, h=32, w=32, k=256, r=1, s=1, padding=(0, 0), stride=(1, 1), dilation=(1, 1)), True),   # 1x1: one reduction block, two column tiles
+    (dict(n=2, c=32, h=16, w=64, k=64, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),    # one output row per block
+    (dict(n=5, c=24, h=32, w=8, k=72, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),     # 8 output rows per block
+    (dict(n=2, c=16, h=36, w=32, k=64, r=5, s=1, padding=(0, 0), stride=(1, 1), dilation=(1, 1)), True),    # no padding: P = 32 from H = 36
+    (dict(n=2, c=16, h=16, w=16, k=64, r=3, s=3, padding=(2, 2), stride=(1, 1), dilation=(1, 1)), False),   # Q = 18
+    (dict(n=2, c=8, h=32, w=32, k=64, r=3, s=3, padding=(1, 1), stride=(2, 2), dilation=(1, 1)), False),    # stride
+    (dict(n=1, c=16, h=8, w=16, k=64, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), False),    # P*Q = 128
+    (dict(n=1, c=256, h=32, w=32, k=64, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), False),  # input rows do not fit in LDS
+]
+
+
+@pytest.mark.parametrize("cfg,taken", IMPLICIT_GEOMS)
+@pytest.mark.parametrize("p", [0.0, 0.5])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_implicit_gemm_conv_forward(cfg, taken, p, dtype):
+    """sd_conv2d_dsd_lists (no patch matrix) against the oracle and against im2col + DSD on the same lists;
+    geometries it does not take must come back as None with nothing written."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(cfg["c"] + cfg["k"])
+    x = torch.randn(cfg["n"], cfg["c"], cfg["h"], cfg["w"], generator=gen).to(dtype)
+    fan_in = cfg["c"] * cfg["r"] * cfg["s"]
+    k = ((torch.rand(cfg["k"], cfg["c"], cfg["r"], cfg["s"], generator=gen) * 2 - 1) * fan_in ** -0.5).to(dtype)
+    p_, q_ = O.conv_out_hw(cfg["h"], cfg["w"], cfg["r"], cfg["s"], **_geo(cfg))
+    rows = cfg["n"] * p_ * q_
+    mask = cpu_mask(O.mask_shape(rows, fan_in, 64), p, gen)
+    lists = ext.build_lists(mask.cuda())
+    xg, w2 = x.cuda(), k.cuda().reshape(cfg["k"], fan_in)
+    s = 1 / (1 - p)
+    y = ext.conv2d_dsd_lists(xg, w2, lists, 64, s, (cfg["r"], cfg["s"]), **_geo(cfg))
+    if not taken:
+        assert y is None
+        return
+    assert y is not None and tuple(y.shape) == (rows, cfg["k"])
+    assert ext.last_kernel() == "specialised"
+    cols = ext.im2col(xg, (cfg["r"], cfg["s"]), **_geo(cfg))
+    explicit = ext.gemm_dsd_lists(cols, w2, lists, 64, s)
+    assert rel_fro(y, to_np(explicit)) <= 1e-3
+    ry = O.conv2d_blockdrop(to_np(x), to_np(k), mask.numpy(), 64, p, dtype=np.float32, **_geo(cfg))
+    ry2 = np.transpose(ry, (0, 2, 3, 1)).reshape(rows, cfg["k"])
+    assert rel_fro(y, ry2) <= REL_FRO_TOL
+
+
+def test_implicit_and_explicit_conv_routes_agree():
+    """The autograd function with the implicit forward (input kept, kept patch blocks re-gathered for the weight
+    gradient) and with the explicit one (patch matrix kept) give the same three results."""
+    import sys
+
+    import flash_dropout.functional as F
+
+    mod = sys.modules["flash_dropout.functional.im2col_conv2d"]  # the package re-exports a function of that name
+    gen = torch.Generator().manual_seed(9)
+    x = torch.randn(4, 64, 32, 32, generator=gen).half().cuda()
+    k = (torch.randn(128, 64, 3, 3, generator=gen) * 0.04).half().cuda()
+    dy = torch.randn(4, 128, 32, 32, generator=gen).half().cuda()
+    mask = (torch.rand(64, 9, generator=gen) < 0.5).cuda()
+    out = {}
+    for implicit in (True, False):
+        prev, mod.IMPLICIT_FORWARD = mod.IMPLICIT_FORWARD, implicit
+        try:
+            xg, kg = x.clone().requires_grad_(), k.clone().requires_grad_()
+            y = F.blockwise_dropout_conv2d_mask(xg, mask, 64, 0.5, kg, padding=(1, 1))
+            y.backward(dy)
+            out[implicit] = (y.detach(), xg.grad, kg.grad)
+        finally:
+            mod.IMPLICIT_FORWARD = prev
+    for a, b, what in zip(out[True], out[False], ("y", "dx", "dk")):
+        assert rel_fro(a, to_np(b)) <= 1e-3, what
+
+
 def test_dense_im2col_conv_matches_conv2d():
     """The reference's implied check for its im2col path: equal to F.conv2d (benchmark/conv.py:20-75)."""
     import flash_dropout.functional as F
