@@ -197,6 +197,17 @@ int sd_gemm_sdd_lists(const void* A, int64_t a_stride_r, int64_t a_stride_c,
                       int64_t M, int64_t N, int64_t K, int64_t block_size, float scale, int dtype,
                       void* stream);
 
+/* sd_gemm_sdd_lists for a consumer that reads kept tiles only (sd_col2im with the same mask does): the
+ * dropped tiles of C are left untouched instead of being written as zeros, which for half of a large C
+ * dropped is a third of the call's memory traffic.  The reference always writes them
+ * (matmul_sdd.cuh:44-65); no counterpart there. */
+int sd_gemm_sdd_lists_kept(const void* A, int64_t a_stride_r, int64_t a_stride_c,
+                           const void* B, int64_t b_stride_r, int64_t b_stride_c,
+                           void* C, int64_t c_stride_r, int64_t c_stride_c,
+                           const int32_t* row_ptr, const int32_t* col_idx,
+                           int64_t M, int64_t N, int64_t K, int64_t block_size, float scale, int dtype,
+                           void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * (e) im2col gather feeding the same GEMMs for conv.
  *

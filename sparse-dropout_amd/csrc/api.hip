@@ -100,6 +100,7 @@ GemmArgs make_args(const void* A, int64_t asr, int64_t asc, const void* B, int64
   const bool ws_ok = ws != nullptr && ws_bytes > 0 && reinterpret_cast<uintptr_t>(ws) % 16 == 0;
   g.ws = ws_ok ? static_cast<float*>(ws) : nullptr;
   g.ws_bytes = ws_ok ? ws_bytes : 0;
+  g.kept_only = false;
   return g;
 }
 
@@ -223,6 +224,17 @@ int sd_gemm_sdd_lists(const void* A, int64_t asr, int64_t asc, const void* B, in
   if (int rc = check_sparse(bs, scale)) return rc;
   SD_REQUIRE(row_ptr && col_idx, "gemm_sdd: null list");
   GemmArgs g = make_args(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, bs, scale, row_ptr, col_idx);
+  return run(g, kSdd, dtype, (hipStream_t)stream);
+}
+
+int sd_gemm_sdd_lists_kept(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc,
+                           void* C, int64_t csr, int64_t csc, const int32_t* row_ptr, const int32_t* col_idx,
+                           int64_t M, int64_t N, int64_t K, int64_t bs, float scale, int dtype, void* stream) {
+  if (int rc = check_common(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, dtype)) return rc;
+  if (int rc = check_sparse(bs, scale)) return rc;
+  SD_REQUIRE(row_ptr && col_idx, "gemm_sdd: null list");
+  GemmArgs g = make_args(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, bs, scale, row_ptr, col_idx);
+  g.kept_only = true;
   return run(g, kSdd, dtype, (hipStream_t)stream);
 }
 

@@ -106,6 +106,7 @@ struct GemmArgs {
   const int32_t* col_idx;
   float* ws;         // optional split-K workspace (fp32 partial tiles), may be null
   int64_t ws_bytes;
+  bool kept_only;    // SDD: dropped tiles of C are left untouched instead of being zeroed
 };
 
 // Geometry of a stride-1, dilation-1 convolution whose patch matrix the DSD kernel gathers itself

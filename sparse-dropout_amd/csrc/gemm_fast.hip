@@ -687,7 +687,7 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
   for (int j = 0; j < GW; ++j) rowmask |= (kept >> (4 * j)) & 0xfu;
 
   // ---- zeros for the dropped tiles of the group's column range ----------------------------------------
-  {
+  if (!g.kept_only) {
     const int row = tid / 8, ch = tid % 8;
     const u32x4 z = {0u, 0u, 0u, 0u};
     for (int c = c_lo; c < c_hi; ++c) {

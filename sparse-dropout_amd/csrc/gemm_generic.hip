@@ -226,6 +226,7 @@ __global__ __launch_bounds__(THREADS) void gemm_generic_kernel(GemmArgs g, int t
   // reduction is split).
   // MFMA result layout: register v of lane l is element (row 8*(v/4) + 4*(l/32) + v%4, col l%32)
   // of D = (first operand rows) x (second operand rows).
+  if (MODE == kSdd && g.kept_only && !wave_kept) return;  // the caller never reads dropped tiles
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
 #pragma unroll

@@ -83,7 +83,8 @@ class _Im2colConv2d(torch.autograd.Function):
             lists = KeptLists(saved[3], saved[4], saved[5], saved[6], ctx.list_shape)
             scale = 1.0 / (1.0 - p)
             if ctx.needs_input_grad[0]:
-                dcols = ext.gemm_sdd_lists(dy2, w2.t(), lists, kernel_bs, scale)
+                # col2im skips the dropped blocks, so the SDD need not zero them
+                dcols = ext.gemm_sdd_lists(dy2, w2.t(), lists, kernel_bs, scale, kept_only=True)
                 dx = ext.col2im(dcols, x_shape, (r, s), padding, stride, dilation, mask, block_size, ch_last)
             if ctx.needs_input_grad[1]:
                 if ctx.implicit:  # the forward kept the input, not the patch matrix: gather the kept blocks now

@@ -41,6 +41,8 @@ SIGNATURES = {
                                   c_int64, c_int64, c_float, c_int, c_void_p, c_int64, c_void_p]),
     "sd_gemm_sdd_lists": (c_int, [*_mat, *_mat, *_mat, c_void_p, c_void_p, c_int64, c_int64,
                                   c_int64, c_int64, c_float, c_int, c_void_p]),
+    "sd_gemm_sdd_lists_kept": (c_int, [*_mat, *_mat, *_mat, c_void_p, c_void_p, c_int64, c_int64,
+                                  c_int64, c_int64, c_float, c_int, c_void_p]),
     "sd_conv2d_dsd_lists": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64,
                                     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,

@@ -382,8 +382,12 @@ class GEMM:
     def gemm_dsd_lists(self, A, B, lists: KeptLists, block_size, scale, out=None, transposed_out=False):
         return self._listed(self.lib.sd_gemm_dsd_lists, "K", A, B, lists, block_size, scale, out, transposed_out)
 
-    def gemm_sdd_lists(self, A, B, lists: KeptLists, block_size, scale, out=None, transposed_out=False):
-        return self._listed(self.lib.sd_gemm_sdd_lists, "N", A, B, lists, block_size, scale, out, transposed_out)
+    def gemm_sdd_lists(self, A, B, lists: KeptLists, block_size, scale, out=None, transposed_out=False,
+                       kept_only=False):
+        """``kept_only``: dropped tiles of the result are left as they are (uninitialised for a fresh buffer)
+        instead of being zeroed, for a consumer that never reads them (:meth:`col2im` with the mask)."""
+        fn = self.lib.sd_gemm_sdd_lists_kept if kept_only else self.lib.sd_gemm_sdd_lists
+        return self._listed(fn, "N", A, B, lists, block_size, scale, out, transposed_out)
 
     # ------------------------------------------------------------------ conv feed
     @staticmethod

@@ -394,3 +394,23 @@ def test_baseline_shapes_run_on_the_specialised_kernels(M, N, K):
     assert ext.last_kernel() == "specialised"
     ext.gemm_dsd(A.T, dC.T, mask128.T, 128, 2.0)
     assert ext.last_kernel() == "specialised"
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 256, 576), (1000, 128, 200), (4096, 64, 4104)])
+def test_sdd_kept_only_leaves_dropped_tiles_untouched(M, N, K):
+    """sd_gemm_sdd_lists_kept: kept tiles equal the ordinary call's, dropped tiles keep what the buffer held."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(3)
+    dC = make_operand(M, N, torch.float16, "cuda", gen=gen)
+    B = make_operand(N, K, torch.float16, "cuda", scale=N ** -0.5, gen=gen)
+    mk = cpu_mask(O.mask_shape(M, K, 64), 0.5, gen)
+    lists = ext.build_lists(mk.cuda())
+    full = ext.gemm_sdd_lists(dC, B.T, lists, 64, 2.0)
+    sentinel = 123.0
+    out = torch.full((M, K), sentinel, dtype=torch.float16, device="cuda")
+    got = ext.gemm_sdd_lists(dC, B.T, lists, 64, 2.0, out=out, kept_only=True)
+    keep = torch.from_numpy(O.expand_keep(mk.numpy(), 64, M, K)).cuda()
+    assert torch.equal(got[keep], full[keep])
+    assert (got[~keep] == sentinel).all()
