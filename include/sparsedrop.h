@@ -115,8 +115,10 @@ int sd_random_lists(uint64_t seed, uint64_t offset, float p, int64_t mb, int64_t
                     int64_t split, int64_t out_mb, int64_t out_kb, int32_t* row_ptr, int32_t* col_idx,
                     int32_t* col_ptr, int32_t* row_idx, void* stream);
 
-/* The same draw keyed by device memory: state is a device pointer to {seed, offset} (two uint64); the
- * kernels read both from there and a trailing one-thread kernel adds 1 to the offset, all on `stream`.
+/* The same draw keyed by device memory: state is a device pointer to four uint64 {seed, offset, 0, 0}; the
+ * kernels read seed and offset from there and add 1 to the offset once every workgroup has read them (the
+ * third word counts workgroups while a call runs and is zero again when it ends; the fourth is unused), all
+ * on `stream`, without a memset and for masks of up to 2^18 entries without an extra launch.
  * Nothing about the draw is baked into the launch arguments, so a captured HIP graph that contains this
  * call draws a new mask at every replay (with sd_random_lists the seed is a launch argument and a replay
  * would repeat the mask).  The reference has no counterpart: its mask comes from torch.rand on torch's

@@ -175,17 +175,32 @@ __device__ inline int block_exclusive_scan(int v, int32_t* lds, int& total) {
   return before + incl - v;
 }
 
+// `advance` (the device-resident generator state of a draw keyed by it, else null): the block that finishes
+// last moves the state on to the next draw.  Every block has read the state by the time it reports in
+// (state[2] counts arrivals and is left at zero), so no block can see the new offset.
 __global__ __launch_bounds__(kFlatThreads) void build_lists_flat(ListJob job0, ListJob job1, int blocks0,
                                                                 int blocks1, uint8_t* mask_out,
-                                                                int64_t mask_rows) {
+                                                                int64_t mask_rows, uint64_t* advance) {
   __shared__ int32_t lds[kFlatThreads / kWave];
   const int tid = threadIdx.x;
   int b = blockIdx.x;
+  auto report_in = [&]() {
+    if (advance == nullptr) return;
+    __syncthreads();
+    if (tid == 0) {
+      unsigned* arrivals = reinterpret_cast<unsigned*>(advance + 2);
+      if (atomicAdd(arrivals, 1u) == gridDim.x - 1) {
+        *arrivals = 0u;
+        advance[1] += 1;
+      }
+    }
+  };
   if (b >= blocks0 + blocks1) {  // launched only for a drawn mask: store it for the caller
     const int nb = gridDim.x - blocks0 - blocks1;
     job0.src.resolve();
     write_mask(job0.src, mask_rows, mask_out, (int64_t)(b - blocks0 - blocks1) * kFlatThreads + tid,
                (int64_t)nb * kFlatThreads);
+    report_in();
     return;
   }
   const bool second = b >= blocks0;
@@ -228,9 +243,10 @@ __global__ __launch_bounds__(kFlatThreads) void build_lists_flat(ListJob job0, L
     if (++e == len) { e = 0; ++line; }
   }
   if (tid == 0 && f0 + kFlatChunk >= total_entries) job.ptr[job.nlines] = base + chunk_total;
+  report_in();
 }
 
-// After every kernel of a draw has read the state: the next draw gets the next offset.
+// The same for the multi-launch form, after every kernel of a draw has read the state.
 __global__ void advance_state_kernel(uint64_t* state) { state[1] += 1; }
 
 __global__ __launch_bounds__(256) void mask_store_kernel(MaskSrc src, int64_t mb, uint8_t* out) {
@@ -294,9 +310,10 @@ __global__ __launch_bounds__(256) void increment_table_kernel(const int32_t* row
 
 }  // namespace
 
+// *advanced: whether the launch also moved a device-resident generator state on
 static int launch_lists(const MaskSrc& src, int64_t mb, int64_t kb, int32_t* row_ptr, int32_t* col_idx,
                         int32_t* col_ptr, int32_t* row_idx, uint8_t* mask_out, int64_t mask_rows,
-                        hipStream_t stream) {
+                        hipStream_t stream, bool* advanced = nullptr) {
   ListJob csr{src, 0, mb, kb, row_ptr, col_idx};
   ListJob csc{src, 1, kb, mb, col_ptr, row_idx};
   if (mb * kb <= (1 << 18)) {
@@ -304,7 +321,8 @@ static int launch_lists(const MaskSrc& src, int64_t mb, int64_t kb, int32_t* row
     const int blocks0 = row_ptr ? per_list : 0, blocks1 = col_ptr ? per_list : 0;
     const int blocks_mask = mask_out ? (int)ceil_div(mask_rows * src.kb, kFlatChunk) : 0;
     hipLaunchKernelGGL(build_lists_flat, dim3(blocks0 + blocks1 + blocks_mask), dim3(kFlatThreads), 0, stream,
-                       csr, csc, blocks0, blocks1, mask_out, mask_rows);
+                       csr, csc, blocks0, blocks1, mask_out, mask_rows, const_cast<uint64_t*>(src.state));
+    if (advanced) *advanced = src.state != nullptr;
     return check_launch("build_lists_flat");
   }
   if (mask_out) {
@@ -334,8 +352,10 @@ int random_lists(uint64_t seed, uint64_t offset, uint64_t* state, float p, int64
                  int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx, hipStream_t stream) {
   MaskSrc src{nullptr, 0, 0, (int32_t)split, (int32_t)stored_kb, (uint32_t)seed, (uint32_t)(seed >> 32),
               (uint32_t)offset, (uint32_t)(offset >> 32), p, state};
-  if (int rc = launch_lists(src, mb, kb, row_ptr, col_idx, col_ptr, row_idx, mask_out, stored_mb, stream)) return rc;
-  if (state) {
+  bool advanced = false;
+  if (int rc = launch_lists(src, mb, kb, row_ptr, col_idx, col_ptr, row_idx, mask_out, stored_mb, stream, &advanced))
+    return rc;
+  if (state && !advanced) {
     hipLaunchKernelGGL(advance_state_kernel, dim3(1), dim3(1), 0, stream, state);
     return check_launch("advance_state");
   }

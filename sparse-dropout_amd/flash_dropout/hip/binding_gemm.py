@@ -281,11 +281,11 @@ class GEMM:
         dev = _device(device)
         seed = int(seed) & (2 ** 64 - 1)
         as_i64 = seed if seed < 2 ** 63 else seed - 2 ** 64
-        state = torch.tensor([as_i64, 0], dtype=torch.int64, device=dev)
+        state = torch.tensor([as_i64, 0, 0, 0], dtype=torch.int64, device=dev)
         self._rng[dev.index] = (torch.initial_seed(), state)
 
     def rng_state(self, device=None) -> torch.Tensor:
-        """int64[2] device tensor {seed, offset} behind the draws that are given no explicit seed; every
+        """int64[4] device tensor {seed, offset, 0, 0} behind the draws that are given no explicit seed; every
         such draw advances the offset by one on the stream it runs on.  Create it (one draw, or
         :meth:`manual_seed`) before capturing a graph: the first use copies the seed from the host."""
         dev = _device(device)

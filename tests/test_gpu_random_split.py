@@ -148,7 +148,7 @@ def test_functional_mask_follows_torch_seed():
     ext.manual_seed(77)                 # explicit restart, independent of torch's seed
     m0, _ = ext.random_lists((5, 7), 0.4)
     m1, _ = ext.random_lists((5, 7), 0.4)
-    assert ext.rng_state().tolist() == [77, 2]
+    assert ext.rng_state().tolist() == [77, 2, 0, 0]
     assert np.array_equal(m0.cpu().numpy(), O.random_mask((5, 7), 0.4, 77, offset=0))
     assert np.array_equal(m1.cpu().numpy(), O.random_mask((5, 7), 0.4, 77, offset=1))
     # large mask: the multi-launch builder reads the same state in all of its kernels
@@ -156,7 +156,7 @@ def test_functional_mask_follows_torch_seed():
     want = O.random_mask((600, 600), 0.5, 77, offset=2)
     assert np.array_equal(m2.cpu().numpy(), want)
     _assert_lists(l2, want)
-    assert ext.rng_state().tolist() == [77, 3]
+    assert ext.rng_state().tolist() == [77, 3, 0, 0]
 
 
 def test_graph_replays_draw_fresh_masks():
