@@ -66,7 +66,7 @@ const char* sd_last_error(void);
 const char* sd_last_kernel(void);
 
 /* Workgroup shape of the specialised DSD / dense kernels: SD_TILE_AUTO picks from the shape (256 x 256
- * output tiles when they give at least half of the CUs a workgroup or the reduction is longer than 4096, split
+ * output tiles when they give three quarters of the CUs a workgroup or the reduction is longer than 4096, split
  * over workgroups then; 128 x 128 otherwise), the other two
  * force one shape for every later call of the process.  Returns the previous setting, -1 for an unknown
  * value.  A tuning and test hook; results do not depend on it beyond fp32 summation order.  No

@@ -49,16 +49,20 @@ constexpr int MAX_STEPS = 1024;
 // step table: one uint32 per step of the union walk, reduction block | keep flags << 16, followed by
 // STEP_PAD zero entries so that look-ahead reads past the end are harmless
 constexpr int STEP_PAD = 4;
-// Shape of a DSD workgroup: RH pairs of row blocks x NS column slices of NT 32-column MFMA tiles; wave
-// (rh, ns) multiplies its slice of the W tile with the kept X tiles of its pair.
-//   DsdBig  256 rows x 256 columns, 8 waves: the least operand traffic per MFMA; what large products run on
-//   DsdMid  128 rows x 128 columns, 4 waves: four times as many workgroups, for products whose 256 x 256
-//           tiles would leave most of the 256 CUs without one.  A wave's 128 x 32 slice needs 1.25 KB of
-//           LDS fragment reads per MFMA against 0.75 KB in the big shape, which is what bounds it
-template <int RH_, int NS_, int NT_>
+// Shape of a DSD workgroup: RH groups of RW row blocks x NS column slices of NT 32-column MFMA tiles; wave
+// (rh, ns) multiplies its slice of the W tile with the kept X tiles of its RW row blocks.  Waves (rh, ns)
+// with equal ns share a SIMD, so a SIMD's MFMA work per step depends on how many row blocks keep the K
+// block, not on which.
+//   DsdBig  256 rows x 256 columns, 8 waves of 2 row blocks x 64 columns: the least operand traffic per
+//           MFMA; what large products run on
+//   DsdMid  128 rows x 128 columns, 8 waves of 1 row block x 32 columns: four times as many workgroups, for
+//           products whose 256 x 256 tiles would leave most of the 256 CUs without one; two workgroups fit
+//           a CU (72 KB of LDS, under 128 VGPRs).  More LDS fragment traffic per MFMA (1.5 KB against
+//           0.75 KB), which is why the big shape wins as soon as it can fill the chip
+template <int RH_, int NS_, int NT_, int RW_ = 2>
 struct DsdShape {
-  static constexpr int RH = RH_, NS = NS_, NT = NT_;
-  static constexpr int R = 2 * RH;           // row blocks per workgroup
+  static constexpr int RH = RH_, NS = NS_, NT = NT_, RW = RW_;  // RW: row blocks a wave owns (2 or 1)
+  static constexpr int R = RW * RH;          // row blocks per workgroup
   static constexpr int NW = RH * NS;         // waves
   static constexpr int THREADS = 64 * NW;
   static constexpr int BN = NS * NT * 32;    // output columns per workgroup
@@ -73,7 +77,7 @@ struct DsdShape {
   static_assert(BL >= 1 && AL >= 1 && BL * NW * 1024 == B_TILE && AL * NW * 1024 == TILE, "loads must divide evenly");
 };
 using DsdBig = DsdShape<2, 4, 2>;
-using DsdMid = DsdShape<1, 4, 1>;
+using DsdMid = DsdShape<2, 4, 1, 1>;
 // 256 rows x 128 columns, 8 waves: the shape of the implicit-GEMM convolution, whose input patch has to
 // fit in LDS next to the stages
 using DsdConv = DsdShape<2, 4, 1>;
@@ -152,7 +156,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
                                                          int Mb, int Kb_all, ImplicitConv cg) {
   static_assert(!IMPLICIT || (!TRANS && S::R == 4 && S::THREADS == 512), "the gather assumes 512 threads x 4 row blocks");
   constexpr int R = S::R, BN = S::BN, THREADS = S::THREADS, NT = S::NT, STAGE = S::STAGE, A_OFF = S::A_OFF;
-  constexpr int BL = S::BL, AL = S::AL;
+  constexpr int BL = S::BL, AL = S::AL, RW = S::RW;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   uint32_t* step_e = reinterpret_cast<uint32_t*>(smem + S::SMEM_STEPS);
   uint32_t* scratch = reinterpret_cast<uint32_t*>(smem + S::SMEM_SCRATCH);
@@ -422,9 +426,9 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
     f.w &= n >= 8 ? ~0u : (n == 7 ? 0xffffu : 0u);
   };
 
-  f32x16 acc[2][2][NT];  // [row block of the pair][m tile][n tile]
+  f32x16 acc[RW][2][NT];  // [row block of the wave][m tile][n tile]
 #pragma unroll
-  for (int a = 0; a < 2; ++a)
+  for (int a = 0; a < RW; ++a)
 #pragma unroll
     for (int b = 0; b < 2; ++b)
 #pragma unroll
@@ -469,7 +473,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
     constexpr int NR = (MINE == 3) ? 2 : 1;
     constexpr int R0 = (MINE == 2) ? 1 : 0;
     u32x4 bf[NT][4];
-    const char* at0 = st + A_OFF + (2 * rh + R0) * TILE;
+    const char* at0 = st + A_OFF + (RW * rh + R0) * TILE;
     u32x4 af[2][2];
     read_b(st, 0, bf);
     read_a(at0, 0, af[0]);
@@ -513,14 +517,18 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
     const int stage = step & 1;
     const uint32_t e_after = step_e[step + 2];
     const bool more = step + 1 < nsteps;
-    const uint32_t mine = (step_flags(e_cur) >> (2 * rh)) & 3u;
+    const uint32_t mine = (step_flags(e_cur) >> (RW * rh)) & ((1u << RW) - 1u);
     const bool mid = late && more && mine != 0u;
     if (more && !mid) issue_loads(e_next, stage ^ 1);
     const char* st = smem + stage * STAGE;
     const bool red_tail = RAGGED && step_block(e_cur) == kb_tail;
-    if (mine == 3u) compute(std::integral_constant<int, 3>{}, st, mid, e_next, stage ^ 1, red_tail);
-    else if (mine == 1u) compute(std::integral_constant<int, 1>{}, st, mid, e_next, stage ^ 1, red_tail);
-    else if (mine == 2u) compute(std::integral_constant<int, 2>{}, st, mid, e_next, stage ^ 1, red_tail);
+    if constexpr (RW == 2) {
+      if (mine == 3u) compute(std::integral_constant<int, 3>{}, st, mid, e_next, stage ^ 1, red_tail);
+      else if (mine == 1u) compute(std::integral_constant<int, 1>{}, st, mid, e_next, stage ^ 1, red_tail);
+      else if (mine == 2u) compute(std::integral_constant<int, 2>{}, st, mid, e_next, stage ^ 1, red_tail);
+    } else {
+      if (mine) compute(std::integral_constant<int, 1>{}, st, mid, e_next, stage ^ 1, red_tail);
+    }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     e_cur = e_next;
@@ -533,8 +541,8 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   if (ns * 32 * NT >= nvalid) return;  // this wave's column slice overhangs N: nothing of it is stored
   float* part = nsplit > 1 ? g.ws + (int64_t)split * g.M * g.N : nullptr;
 #pragma unroll
-  for (int rr = 0; rr < 2; ++rr) {
-    const int rb = rb0 + 2 * rh + rr;
+  for (int rr = 0; rr < RW; ++rr) {
+    const int rb = rb0 + RW * rh + rr;
     if (rb >= Mb) continue;
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
@@ -893,6 +901,8 @@ int allow_big_lds(const void* kernel, int bytes, bool (&done)[kMaxDevices]) {
   return SD_OK;
 }
 
+std::atomic<int> tile_policy{0};
+
 template <typename T, bool TRANS, bool CM, bool RAGGED, typename S>
 int launch_dsd_s(const GemmArgs& g, int splits, hipStream_t stream) {
   static bool configured[kMaxDevices] = {};
@@ -918,7 +928,6 @@ int launch_dsd(const GemmArgs& g, bool mid, int splits, hipStream_t stream) {
                 : launch_dsd_s<T, TRANS, CM, false, DsdBig>(g, splits, stream);
 }
 
-std::atomic<int> tile_policy{0};
 
 // workgroups a tile shape gives and how many ways the reduction is then split
 struct DsdPlan {
@@ -943,10 +952,11 @@ DsdPlan plan_dsd(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0) return {false, 1};
   const int policy = tile_policy.load(std::memory_order_relaxed);
   const int64_t big = dsd_tiles<DsdBig>(M, N), midt = dsd_tiles<DsdMid>(M, N);
-  // the 256 x 256 shape whenever it gives at least half of the CUs a workgroup, and for long reductions,
-  // which it splits over workgroups (measured: 2048^3 runs 15-25 % faster on 128 x 128 tiles than on 64 big
-  // tiles x 4 splits; a 384 x 1536 weight gradient over 16384 rows 25 % slower than on 12 big tiles x 21 splits)
-  const bool mid = policy == kTileMid || (policy == kTileAuto && big < 128 && K / BS <= 64);
+  // the 256 x 256 shape when it gives three quarters of the CUs a workgroup, and for long reductions, which it
+  // splits over workgroups (measured: 1024^3 forward 29 us on 16 big tiles, 13 us on 64 mid tiles; 2048^3
+  // 29 + 18 us on 64 big tiles x 4 splits and the reduce pass, 24 us on 256 mid tiles; 4096^3, where 256 big
+  // tiles fill the chip, 127 against 158 us)
+  const bool mid = policy == kTileMid || (policy == kTileAuto && big < 192 && K / BS <= 64);
   return {mid, splits_for(mid ? midt : big, M, N, K)};
 }
 
