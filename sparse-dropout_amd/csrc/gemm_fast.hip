@@ -578,19 +578,33 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
 // A wave owns up to two WHOLE kept tiles (tile t of the group goes to wave t%8, so the two waves of a
 // SIMD always carry equal work +-1): 2x2 MFMAs per 16-wide step from 2 + 2 fragments, accumulators
 // statically indexed by the wave's slot, operand tiles addressed dynamically.
-constexpr int GW = 6;                      // column blocks with kept tiles per group
-constexpr int G_BOFF = R * TILE;           // dY tiles first, then W tiles
-constexpr int G_STAGE = (R + GW) * TILE;   // 80 KB
-constexpr int G_SMEM = 2 * G_STAGE;        // all of the 160 KB; everything else lives in registers
-constexpr int G_MAX_CB = 32768;            // per-column flags share the first stage before the loads start
+// SddBig   4 row blocks x groups of at most 6 active column blocks and 16 kept tiles, two tile slots per wave:
+//           two 80 KB stages, all of the LDS
+// SddMid   2 row blocks x at most 4 active column blocks and 8 kept tiles, one slot per wave: twice as many
+//           workgroups with half the loads per step each, for outputs that give the big shape too few
+template <int R_, int GW_, int SLOTS_>
+struct SddShape {
+  static constexpr int R = R_;           // row blocks per workgroup
+  static constexpr int GW = GW_;         // column blocks with kept tiles per group
+  static constexpr int SLOTS = SLOTS_;   // whole tiles a wave can own
+  static constexpr int MAXT = 8 * SLOTS; // kept tiles per group
+  static constexpr int BOFF = R * TILE;  // dY tiles first, then W tiles
+  static constexpr int STAGE = (R + GW) * TILE;
+  static constexpr int SMEM = 2 * STAGE;
+  static constexpr int MINCOLS = GW < MAXT / R ? GW : MAXT / R;  // column blocks a group is sure to cover
+};
+using SddBig = SddShape<4, 6, 2>;
+using SddMid = SddShape<2, 4, 1>;
+constexpr int G_MAX_CB = 8192;             // per-column flags share the first stage (of either shape) before the loads start
 
 // EDGE = the output width or the reduction length is not a multiple of 64 (both multiples of 8): the
 // overhanging 16-byte chunks / rows of the last column block / reduction block are fetched from inside the
 // matrix instead, as in the DSD kernel, the fragments of the last reduction block are zeroed past the end,
 // and nothing is stored past the last column.  (A ragged M costs nothing worth a separate instance.)
-template <typename T, bool EDGE>
+template <typename T, bool EDGE, typename G>
 __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tiles_m, int gmax, int Mb,
                                                             int Cb) {
+  constexpr int R = G::R, GW = G::GW, SLOTS = G::SLOTS, G_BOFF = G::BOFF, G_STAGE = G::STAGE;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   uint32_t* flags = reinterpret_cast<uint32_t*>(smem);  // bit r: tile (row block rb0 + r, column block c) kept
   int* rec = reinterpret_cast<int*>(smem + 4 * ((Cb + 3) & ~3));  // c_lo, c_hi, ncols, kept bits, cols[GW]
@@ -604,7 +618,7 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
 
   // ---- per-column keep flags of this row quad -------------------------------------------------------
   {
-    const uint32_t all = (rb0 + R <= Mb) ? 0xfu : ((1u << (Mb - rb0)) - 1u);
+    const uint32_t all = (rb0 + R <= Mb) ? ((1u << R) - 1u) : ((1u << (Mb - rb0)) - 1u);
     const uint32_t init = g.row_ptr ? 0u : all;
     for (int i = tid; i < Cb; i += THREADS) flags[i] = init;
     if (tid < 16) rec[tid] = 0;
@@ -629,7 +643,7 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
         const uint32_t f = (uint32_t)__builtin_amdgcn_readlane((int)fv, i);
         if (f == 0) continue;
         const int a = __builtin_popcount(f);
-        if (width == GW || cnt + a > 16) {  // the group ends in front of this column block
+        if (width == GW || cnt + a > G::MAXT) {  // the group ends in front of this column block
           if (grp == gi) {
             lo = start;
             hi = base + i;
@@ -677,10 +691,10 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
   const int ntiles = __builtin_popcount(kept);
 
   // this wave's tiles: tile t of the group (set bits of `kept` in order) belongs to wave t % 8
-  int my_r[2], my_j[2], my_c[2];
-  bool act[2];
+  int my_r[SLOTS], my_j[SLOTS], my_c[SLOTS];
+  bool act[SLOTS];
 #pragma unroll
-  for (int k = 0; k < 2; ++k) {
+  for (int k = 0; k < SLOTS; ++k) {
     const int t = wave + 8 * k;
     act[k] = t < ntiles;
     uint32_t m = kept;
@@ -793,9 +807,9 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
   // the two waves of a SIMD (w and w + 4) issue their loads half a step apart
   const bool late = wave >= 4;
 
-  f32x16 acc[2][2][2];  // [slot][32-row half][32-column half]
+  f32x16 acc[SLOTS][2][2];  // [slot][32-row half][32-column half]
 #pragma unroll
-  for (int k = 0; k < 2; ++k)
+  for (int k = 0; k < SLOTS; ++k)
 #pragma unroll
     for (int a = 0; a < 2; ++a)
 #pragma unroll
@@ -847,19 +861,21 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
       read_unit(0);
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        read_unit(u + 1);
+        if (u + 1 < 4 * SLOTS) read_unit(u + 1);
         __builtin_amdgcn_sched_barrier(0);
         mfma_unit(std::integral_constant<int, 0>{}, u);
         __builtin_amdgcn_sched_barrier(0);
         if (u == 1 && mid) issue_loads(step + 1, stage ^ 1);
       }
-      if (act[1]) {
+      if constexpr (SLOTS == 2) {
+        if (act[1]) {
 #pragma unroll
-        for (int u = 4; u < 8; ++u) {
-          if (u + 1 < 8) read_unit(u + 1);
-          __builtin_amdgcn_sched_barrier(0);
-          mfma_unit(std::integral_constant<int, 1>{}, u);
-          __builtin_amdgcn_sched_barrier(0);
+          for (int u = 4; u < 8; ++u) {
+            if (u + 1 < 8) read_unit(u + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_unit(std::integral_constant<int, 1>{}, u);
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
       }
     }
@@ -869,7 +885,7 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
 
   // ---- epilogue ---------------------------------------------------------------------------------------
 #pragma unroll
-  for (int k = 0; k < 2; ++k) {
+  for (int k = 0; k < SLOTS; ++k) {
     if (!act[k]) continue;
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
@@ -960,15 +976,26 @@ DsdPlan plan_dsd(int64_t M, int64_t N, int64_t K) {
   return {mid, splits_for(mid ? midt : big, M, N, K)};
 }
 
+template <typename T, bool EDGE, typename G>
+int launch_sdd_shape(const GemmArgs& g, hipStream_t stream) {
+  static bool configured[kMaxDevices] = {};
+  if (int rc = allow_big_lds(reinterpret_cast<const void*>(&sdd_group_kernel<T, EDGE, G>), G::SMEM, configured)) return rc;
+  const int Mb = (int)((g.M + BS - 1) / BS), Cb = (int)((g.N + BS - 1) / BS);
+  // the grid provides for the most groups a row of the block grid can split into
+  const int tiles_m = (Mb + G::R - 1) / G::R, gmax = (Cb + G::MINCOLS - 1) / G::MINCOLS;
+  hipLaunchKernelGGL((sdd_group_kernel<T, EDGE, G>), dim3((unsigned)(tiles_m * gmax)), dim3(THREADS), G::SMEM, stream,
+                     g, tiles_m, gmax, Mb, Cb);
+  return check_launch("sdd_group_kernel");
+}
+
+// the big shape when its grid (at p = 0: a workgroup per 4 x 4 tiles) gives three quarters of the CUs a workgroup
 template <typename T, bool EDGE>
 int launch_sdd_group(const GemmArgs& g, hipStream_t stream) {
-  static bool configured[kMaxDevices] = {};
-  if (int rc = allow_big_lds(reinterpret_cast<const void*>(&sdd_group_kernel<T, EDGE>), G_SMEM, configured)) return rc;
-  const int Mb = (int)((g.M + BS - 1) / BS), Cb = (int)((g.N + BS - 1) / BS);
-  const int tiles_m = (Mb + R - 1) / R, gmax = (Cb + R - 1) / R;
-  hipLaunchKernelGGL((sdd_group_kernel<T, EDGE>), dim3((unsigned)(tiles_m * gmax)), dim3(THREADS), G_SMEM, stream, g,
-                     tiles_m, gmax, Mb, Cb);
-  return check_launch("sdd_group_kernel");
+  const int64_t Mb = (g.M + BS - 1) / BS, Cb = (g.N + BS - 1) / BS;
+  const int64_t big = ((Mb + 3) / 4) * ((Cb + 3) / 4);
+  const int policy = tile_policy.load(std::memory_order_relaxed);
+  const bool mid = policy == kTileMid || (policy == kTileAuto && big < 192);
+  return mid ? launch_sdd_shape<T, EDGE, SddMid>(g, stream) : launch_sdd_shape<T, EDGE, SddBig>(g, stream);
 }
 
 int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
@@ -979,7 +1006,7 @@ int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
                         g.b.sc % 8 == 0 && g.c_sr % 8 == 0 && g.a.sr < (1 << 22) &&
                         g.b.sc < (1 << 22);  // per-lane byte offsets are 32-bit
   const int64_t Cb = (g.N + BS - 1) / BS;
-  const int64_t tiles = (((g.M + BS - 1) / BS + R - 1) / R) * ((Cb + R - 1) / R);
+  const int64_t tiles = (((g.M + BS - 1) / BS + 1) / 2) * ((Cb + 3) / 4);  // the larger of the two shapes' grids
   if (!layout_ok || !shape_ok || !align_ok || tiles > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
   if (Cb > G_MAX_CB) return SD_ERR_UNSUPPORTED;
   const bool edge = g.N % BS != 0 || g.K % BS != 0;
