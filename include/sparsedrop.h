@@ -66,8 +66,8 @@ const char* sd_last_error(void);
 const char* sd_last_kernel(void);
 
 /* Workgroup shape of the specialised DSD / dense kernels: SD_TILE_AUTO picks from the shape (256 x 256
- * output tiles when they give three quarters of the CUs a workgroup or the reduction is longer than 4096, split
- * over workgroups then; 128 x 128 otherwise), the other two
+ * output tiles when there are more than 128 of them, 128 x 128 otherwise; the SDD kernel's group shape follows the
+ * same rule), the other two
  * force one shape for every later call of the process.  Returns the previous setting, -1 for an unknown
  * value.  A tuning and test hook; results do not depend on it beyond fp32 summation order.  No
  * counterpart in the reference (its tile is a compile-time GemmConfig, gemm_configs/gemm_config.cuh:19-100). */

@@ -968,11 +968,12 @@ DsdPlan plan_dsd(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0) return {false, 1};
   const int policy = tile_policy.load(std::memory_order_relaxed);
   const int64_t big = dsd_tiles<DsdBig>(M, N), midt = dsd_tiles<DsdMid>(M, N);
-  // the 256 x 256 shape when it gives three quarters of the CUs a workgroup, and for long reductions, which it
-  // splits over workgroups (measured: 1024^3 forward 29 us on 16 big tiles, 13 us on 64 mid tiles; 2048^3
-  // 29 + 18 us on 64 big tiles x 4 splits and the reduce pass, 24 us on 256 mid tiles; 4096^3, where 256 big
-  // tiles fill the chip, 127 against 158 us)
-  const bool mid = policy == kTileMid || (policy == kTileAuto && big < 192 && K / BS <= 64);
+  // the 256 x 256 shape when it gives more than half of the CUs a workgroup (measured: 1024^3 forward 29 us on
+  // 16 big tiles, 13 us on 64 mid tiles; 2048^3 29 + 18 us on 64 big tiles x 4 splits and the reduce pass,
+  // 24 us on 256 mid tiles; 8192 x 1024 x 1024, 128 big tiles, 30 against 22 us; 3072^3, 144 big tiles, 79
+  // against 94 us; 4096^3, 256 big tiles, 127 against 158 us; weight gradients over 16384 to 131072 rows
+  // 15-30 % faster on mid tiles x fewer splits)
+  const bool mid = policy == kTileMid || (policy == kTileAuto && big <= 128);
   return {mid, splits_for(mid ? midt : big, M, N, K)};
 }
 
@@ -988,13 +989,13 @@ int launch_sdd_shape(const GemmArgs& g, hipStream_t stream) {
   return check_launch("sdd_group_kernel");
 }
 
-// the big shape when its grid (at p = 0: a workgroup per 4 x 4 tiles) gives three quarters of the CUs a workgroup
+// the big shape when its grid (at p = 0: a workgroup per 4 x 4 tiles) gives more than half of the CUs a workgroup
 template <typename T, bool EDGE>
 int launch_sdd_group(const GemmArgs& g, hipStream_t stream) {
   const int64_t Mb = (g.M + BS - 1) / BS, Cb = (g.N + BS - 1) / BS;
   const int64_t big = ((Mb + 3) / 4) * ((Cb + 3) / 4);
   const int policy = tile_policy.load(std::memory_order_relaxed);
-  const bool mid = policy == kTileMid || (policy == kTileAuto && big < 192);
+  const bool mid = policy == kTileMid || (policy == kTileAuto && big <= 128);
   return mid ? launch_sdd_shape<T, EDGE, SddMid>(g, stream) : launch_sdd_shape<T, EDGE, SddBig>(g, stream);
 }
 
