@@ -255,6 +255,7 @@ int sd_col2im(const void* cols, int64_t cols_ld, void* dx, int64_t dx_stride_n,
  * 256, C*R*S a multiple of 8, R*S <= 30, and the input rows of 256 output positions (all channels) plus a
  * column table fitting in LDS (C * (256/Q + R - 1) * W * 2 + ceil(C*R*S/64)*256 <= about 55 KB).
  * Anything else returns SD_ERR_UNSUPPORTED with nothing launched: use sd_im2col + sd_gemm_dsd_lists.
+ * NULL lists = every block kept: the dense convolution (block_size is then ignored, scale still applied).
  * ------------------------------------------------------------------------------------------- */
 int sd_conv2d_dsd_lists(const void* x, int64_t x_stride_n, int64_t x_stride_c, int64_t x_stride_h,
                         int64_t x_stride_w, const void* weight, int64_t weight_ld,

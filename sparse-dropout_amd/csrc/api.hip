@@ -325,11 +325,17 @@ int sd_conv2d_dsd_lists(const void* x, int64_t sn, int64_t sc, int64_t sh, int64
                         int64_t stride_w, int64_t dil_h, int64_t dil_w, const int32_t* row_ptr,
                         const int32_t* col_idx, int64_t bs, float scale, int dtype, void* stream) {
   SD_REQUIRE(dtype == SD_F16 || dtype == SD_BF16, "dtype must be SD_F16 or SD_BF16 (got %d)", dtype);
-  SD_REQUIRE(x && weight && y && row_ptr && col_idx, "null pointer argument");
+  SD_REQUIRE(x && weight && y, "null pointer argument");
+  SD_REQUIRE((row_ptr == nullptr) == (col_idx == nullptr), "row_ptr and col_idx must both be given or both be null");
   SD_REQUIRE(n > 0 && c > 0 && h > 0 && w > 0 && k_out > 0 && r > 0 && s > 0, "sizes must be positive");
   SD_REQUIRE(stride_h > 0 && stride_w > 0 && dil_h > 0 && dil_w > 0 && pad_h >= 0 && pad_w >= 0,
              "strides and dilations must be positive, paddings non-negative");
-  if (int rc = check_sparse(bs, scale)) return rc;
+  if (row_ptr) {
+    if (int rc = check_sparse(bs, scale)) return rc;
+  } else {
+    SD_REQUIRE(scale == scale, "scale is NaN");
+    bs = 64;
+  }
   const int64_t P = (h + 2 * pad_h - dil_h * (r - 1) - 1) / stride_h + 1;
   const int64_t Q = (w + 2 * pad_w - dil_w * (s - 1) - 1) / stride_w + 1;
   SD_REQUIRE(P > 0 && Q > 0, "the kernel does not fit the padded input");

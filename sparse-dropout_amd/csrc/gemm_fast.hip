@@ -1031,7 +1031,7 @@ int launch_conv_t(const GemmArgs& g, const ImplicitConv& cg, int smem, hipStream
 
 int launch_conv_implicit(const GemmArgs& g, const ImplicitConv& cg, int64_t P, int64_t stride_h, int64_t stride_w,
                          int64_t dil_h, int64_t dil_w, int64_t R, int64_t x_sw, int dtype, hipStream_t stream) {
-  if (g.bs != BS || g.row_ptr == nullptr) return SD_ERR_UNSUPPORTED;
+  if (g.row_ptr != nullptr && g.bs != BS) return SD_ERR_UNSUPPORTED;
   const bool geom_ok = stride_h == 1 && stride_w == 1 && dil_h == 1 && dil_w == 1 && x_sw == 1 && cg.Q > 0 &&
                        cg.Q <= BS && BS % cg.Q == 0 && (P * cg.Q) % (BS * DsdConv::R) == 0 && cg.W % 8 == 0 &&
                        cg.pad_h >= 0 && cg.pad_w >= 0 && cg.pad_w <= 8 && cg.S - 1 - cg.pad_w <= 8 && R * cg.S == cg.RS &&

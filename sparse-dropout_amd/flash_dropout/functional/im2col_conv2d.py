@@ -62,9 +62,13 @@ class _Im2colConv2d(torch.autograd.Function):
                                   lists.col_ptr, lists.row_idx)
             ctx.list_shape = lists.shape
         else:
-            cols = ext.im2col(input, (r, s), padding, stride, dilation)
-            y2 = ext.gemm(cols, w2)
-            ctx.save_for_backward(cols, w2)
+            y2 = ext.conv2d_dsd_lists(input, w2, None, 0, 1.0, (r, s), padding, stride,
+                                      dilation) if IMPLICIT_FORWARD else None
+            ctx.implicit = y2 is not None
+            if y2 is None:
+                cols = ext.im2col(input, (r, s), padding, stride, dilation)
+                y2 = ext.gemm(cols, w2)
+            ctx.save_for_backward(input if ctx.implicit else cols, w2)
         ctx.geom = (tuple(input.shape), tuple(kernel.shape), padding, stride, dilation, block_size, kernel_bs, p,
                     input.is_contiguous(memory_format=torch.channels_last) and not input.is_contiguous())
         return y2.view(n, po * qo, k).permute(0, 2, 1).view(n, k, po, qo)
@@ -96,6 +100,8 @@ class _Im2colConv2d(torch.autograd.Function):
                 dcols = ext.gemm(dy2, w2.t())
                 dx = ext.col2im(dcols, x_shape, (r, s), padding, stride, dilation, channels_last=ch_last)
             if ctx.needs_input_grad[1]:
+                if ctx.implicit:
+                    cols = ext.im2col(cols, (r, s), padding, stride, dilation)
                 dk = ext.gemm(cols.t(), dy2.t(), transposed_out=True).t().reshape(k_shape)
         return dx, dk, None, None, None, None, None, None, None
 

@@ -432,11 +432,13 @@ class GEMM:
                        self._stream(x))
         return cols
 
-    def conv2d_dsd_lists(self, x: torch.Tensor, weight2d: torch.Tensor, lists: KeptLists, block_size, scale: float,
-                         kernel_size, padding=(0, 0), stride=(1, 1), dilation=(1, 1)) -> torch.Tensor | None:
+    def conv2d_dsd_lists(self, x: torch.Tensor, weight2d: torch.Tensor, lists: KeptLists | None, block_size,
+                         scale: float, kernel_size, padding=(0, 0), stride=(1, 1),
+                         dilation=(1, 1)) -> torch.Tensor | None:
         """Implicit-GEMM forward of the block-dropout convolution: the [N*P*Q, K] product of the patch matrix
-        (never materialised) with ``weight2d`` [K, C*R*S] over the kept blocks of ``lists``.  Returns None
-        when the library does not take the geometry (the caller then goes through :meth:`im2col`)."""
+        (never materialised) with ``weight2d`` [K, C*R*S] over the kept blocks of ``lists`` (None: all of them,
+        the dense convolution).  Returns None when the library does not take the geometry (the caller then
+        goes through :meth:`im2col`)."""
         if x.dim() != 4 or not x.is_cuda or x.dtype not in _DTYPES:
             raise ValueError("x must be a 4D float16/bfloat16 tensor on the GPU")
         n, c, h, w = x.shape
@@ -447,17 +449,20 @@ class GEMM:
         if (weight2d.dim() != 2 or weight2d.shape[1] != c * r * s or weight2d.dtype != x.dtype
                 or weight2d.device != x.device or weight2d.stride(1) != 1):
             raise ValueError(f"weight2d must be a [K, {c * r * s}] {x.dtype} matrix on {x.device} with unit column stride")
-        bs = _block_size(block_size)
-        want = (ceil(n * p * q / bs), ceil(c * r * s / bs))
-        if tuple(lists.shape) != want:
-            raise ValueError(f"lists are for a {lists.shape} mask, patch matrix needs {want}")
+        bs, rp, ci = 0, None, None
+        if lists is not None:
+            bs = _block_size(block_size)
+            want = (ceil(n * p * q / bs), ceil(c * r * s / bs))
+            if tuple(lists.shape) != want:
+                raise ValueError(f"lists are for a {lists.shape} mask, patch matrix needs {want}")
+            rp, ci = lists.row_ptr.data_ptr(), lists.col_idx.data_ptr()
         k = weight2d.shape[0]
         y = torch.empty((n * p * q, k), dtype=x.dtype, device=x.device)
         with _guard(x.device):
             rc = self.lib.sd_conv2d_dsd_lists(x.data_ptr(), *x.stride(), weight2d.data_ptr(), weight2d.stride(0),
                                               y.data_ptr(), y.stride(0), n, c, h, w, k, r, s, *padding, *stride,
-                                              *dilation, lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(), bs,
-                                              float(scale), _DTYPES[x.dtype], self._stream(x))
+                                              *dilation, rp, ci, bs, float(scale), _DTYPES[x.dtype],
+                                              self._stream(x))
         if rc == 2:  # geometry not taken: nothing was launched
             return None
         if rc != 0:

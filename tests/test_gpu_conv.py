@@ -169,6 +169,23 @@ def test_implicit_gemm_conv_forward(cfg, taken, p, dtype):
     assert rel_fro(y, ry2) <= REL_FRO_TOL
 
 
+@pytest.mark.parametrize("cfg,taken", [g for g in IMPLICIT_GEOMS if g[1]][:5])
+def test_implicit_gemm_conv_dense(cfg, taken):
+    """No lists = every block kept: the dense convolution, against torch's conv2d in fp32."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(2)
+    x = torch.randn(cfg["n"], cfg["c"], cfg["h"], cfg["w"], generator=gen).half()
+    fan_in = cfg["c"] * cfg["r"] * cfg["s"]
+    k = ((torch.rand(cfg["k"], cfg["c"], cfg["r"], cfg["s"], generator=gen) * 2 - 1) * fan_in ** -0.5).half()
+    y = ext.conv2d_dsd_lists(x.cuda(), k.cuda().reshape(cfg["k"], fan_in), None, 0, 1.0, (cfg["r"], cfg["s"]), **_geo(cfg))
+    assert y is not None
+    ref = torch.nn.functional.conv2d(x.float(), k.float(), padding=cfg["padding"])
+    n, kk, p_, q_ = ref.shape
+    assert rel_fro(y, ref.permute(0, 2, 3, 1).reshape(n * p_ * q_, kk).numpy()) <= REL_FRO_TOL
+
+
 def test_implicit_and_explicit_conv_routes_agree():
     """The autograd function with the implicit forward (input kept, kept patch blocks re-gathered for the weight
     gradient) and with the explicit one (patch matrix kept) give the same three results."""
