@@ -109,6 +109,38 @@ GemmArgs make_args(const void* A, int64_t asr, int64_t asc, const void* B, int64
 
 using namespace sd;
 
+// Geometry of an implicit-GEMM launch whose LDS copy of the input covers `blocks` 64-position row blocks.
+static ImplicitConv conv_geometry(const void* x, int64_t sn, int64_t sc, int64_t sh, int64_t c, int64_t h, int64_t w,
+                                  int64_t P, int64_t Q, int64_t r, int64_t s, int64_t pad_h, int64_t pad_w,
+                                  int64_t blocks) {
+  ImplicitConv cg;
+  cg.x = static_cast<const uint16_t*>(x);
+  cg.sn = sn;
+  cg.sc = sc;
+  cg.sh = sh;
+  cg.C = (int)c;
+  cg.H = (int)h;
+  cg.W = (int)w;
+  cg.Q = (int)Q;
+  cg.RS = (int)(r * s);
+  cg.S = (int)s;
+  cg.pad_h = (int)pad_h;
+  cg.pad_w = (int)pad_w;
+  cg.rpb = (int)(64 / Q);
+  cg.blocks_per_img = (int)(P * Q / 64);
+  cg.PR = (int)(blocks * (64 / Q) + r - 1);
+  cg.PW = (int)(w + 8);
+  cg.patch_stride = 0;
+  cg.K = (int)(c * r * s);
+  auto magic = [](int64_t d) { return d <= 1 ? 0u : (uint32_t)(((1ull << 32) + (uint64_t)d - 1) / (uint64_t)d); };
+  cg.m_spc = magic(cg.PR * (w / 8));
+  cg.m_spr = magic(w / 8);
+  cg.m_RS = magic(r * s);
+  cg.m_S = magic(s);
+  cg.m_Q = magic(Q);
+  return cg;
+}
+
 extern "C" {
 
 int sd_version(void) { return 100; }
@@ -342,33 +374,41 @@ int sd_conv2d_dsd_lists(const void* x, int64_t sn, int64_t sc, int64_t sh, int64
   SD_REQUIRE(wld >= c * r * s && yld >= k_out, "leading dimensions too small");
   if (bs != 64 || Q > 64 || 64 % Q != 0 || c * r * s > (1 << 16) || h > (1 << 20) || w > (1 << 12) || r > 64 || s > 64)
     return SD_ERR_UNSUPPORTED;
-  ImplicitConv cg;
-  cg.x = static_cast<const uint16_t*>(x);
-  cg.sn = sn;
-  cg.sc = sc;
-  cg.sh = sh;
-  cg.C = (int)c;
-  cg.H = (int)h;
-  cg.W = (int)w;
-  cg.Q = (int)Q;
-  cg.RS = (int)(r * s);
-  cg.S = (int)s;
-  cg.pad_h = (int)pad_h;
-  cg.pad_w = (int)pad_w;
-  cg.rpb = (int)(64 / Q);
-  cg.blocks_per_img = (int)(P * Q / 64);
-  cg.PR = (int)(4 * (64 / Q) + r - 1);
-  cg.PW = (int)(w + 8);
-  cg.K = (int)(c * r * s);
-  auto magic = [](int64_t d) { return d <= 1 ? 0u : (uint32_t)(((1ull << 32) + (uint64_t)d - 1) / (uint64_t)d); };
-  cg.m_spc = magic(cg.PR * (w / 8));
-  cg.m_spr = magic(w / 8);
-  cg.m_RS = magic(r * s);
-  cg.m_S = magic(s);
-  cg.m_Q = magic(Q);
+  ImplicitConv cg = conv_geometry(x, sn, sc, sh, c, h, w, P, Q, r, s, pad_h, pad_w, /*blocks=*/4);
   GemmArgs g = make_args(nullptr, 0, 0, weight, wld, 1, y, yld, 1, n * P * Q, k_out, c * r * s, bs, scale, row_ptr,
                          col_idx);
   const int rc = launch_conv_implicit(g, cg, P, stride_h, stride_w, dil_h, dil_w, r, sw, dtype, (hipStream_t)stream);
+  if (rc == SD_OK) last_kernel = "specialised";
+  return rc;
+}
+
+int sd_conv2d_dw_lists(const void* x, int64_t sn, int64_t sc, int64_t sh, int64_t sw, const void* dy, int64_t dyld,
+                       void* dw, int64_t dwld, int64_t n, int64_t c, int64_t h, int64_t w, int64_t k_out, int64_t r,
+                       int64_t s, int64_t pad_h, int64_t pad_w, int64_t stride_h, int64_t stride_w, int64_t dil_h,
+                       int64_t dil_w, const int32_t* col_ptr, const int32_t* row_idx, int64_t bs, float scale,
+                       int dtype, void* workspace, int64_t workspace_bytes, void* stream) {
+  SD_REQUIRE(dtype == SD_F16 || dtype == SD_BF16, "dtype must be SD_F16 or SD_BF16 (got %d)", dtype);
+  SD_REQUIRE(x && dy && dw, "null pointer argument");
+  SD_REQUIRE((col_ptr == nullptr) == (row_idx == nullptr), "col_ptr and row_idx must both be given or both be null");
+  SD_REQUIRE(n > 0 && c > 0 && h > 0 && w > 0 && k_out > 0 && r > 0 && s > 0, "sizes must be positive");
+  SD_REQUIRE(stride_h > 0 && stride_w > 0 && dil_h > 0 && dil_w > 0 && pad_h >= 0 && pad_w >= 0,
+             "strides and dilations must be positive, paddings non-negative");
+  if (col_ptr) {
+    if (int rc = check_sparse(bs, scale)) return rc;
+  } else {
+    SD_REQUIRE(scale == scale, "scale is NaN");
+    bs = 64;
+  }
+  const int64_t P = (h + 2 * pad_h - dil_h * (r - 1) - 1) / stride_h + 1;
+  const int64_t Q = (w + 2 * pad_w - dil_w * (s - 1) - 1) / stride_w + 1;
+  SD_REQUIRE(P > 0 && Q > 0, "the kernel does not fit the padded input");
+  SD_REQUIRE(dyld >= k_out && dwld >= c * r * s, "leading dimensions too small");
+  if (bs != 64 || Q > 64 || 64 % Q != 0 || c * r * s > (1 << 16) || h > (1 << 20) || w > (1 << 12) || r > 64 || s > 64)
+    return SD_ERR_UNSUPPORTED;
+  ImplicitConv cg = conv_geometry(x, sn, sc, sh, c, h, w, P, Q, r, s, pad_h, pad_w, /*blocks=*/1);
+  GemmArgs g = make_args(nullptr, 1, c * r * s, dy, 1, dyld, dw, 1, dwld, c * r * s, k_out, n * P * Q, bs, scale,
+                         col_ptr, row_idx, workspace, workspace_bytes);
+  const int rc = launch_conv_implicit_dw(g, cg, P, stride_h, stride_w, dil_h, dil_w, r, sw, dtype, (hipStream_t)stream);
   if (rc == SD_OK) last_kernel = "specialised";
   return rc;
 }

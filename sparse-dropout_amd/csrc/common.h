@@ -121,6 +121,7 @@ struct ImplicitConv {
   int blocks_per_img;  // P * Q / 64
   int PR;              // input rows a workgroup's 4 row blocks touch: 4 * rpb + R - 1
   int PW;              // halfs per row of the LDS copy: 8 zeros, then the W of the image
+  int patch_stride;    // weight gradient: halfs between the two alternating copies (set by the launcher)
   int K;               // C * R * S
   // ceil(2^32 / d) for the divisors the kernel needs (0 for d = 1): x / d == umulhi(x, m) while x * d < 2^32
   uint32_t m_spc, m_spr, m_RS, m_S, m_Q;  // d = PR * W / 8, W / 8, R * S, S, Q
@@ -144,6 +145,10 @@ int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream);
 // SD_ERR_UNSUPPORTED (without an error message) for geometries it does not take.
 int launch_conv_implicit(const GemmArgs& g, const ImplicitConv& cg, int64_t P, int64_t stride_h, int64_t stride_w,
                          int64_t dil_h, int64_t dil_w, int64_t R, int64_t x_sw, int dtype, hipStream_t stream);
+// weight gradient of the same convolution without the patch matrix: g.M = C*R*S, g.N = K_out, g.K = N*P*Q, g.b =
+// dY^T, g.c column-major, the lists those of the transposed mask; cg.PR = rows one 64-position block touches.
+int launch_conv_implicit_dw(const GemmArgs& g, ImplicitConv cg, int64_t P, int64_t stride_h, int64_t stride_w,
+                            int64_t dil_h, int64_t dil_w, int64_t R, int64_t x_sw, int dtype, hipStream_t stream);
 // which workgroup shape the DSD kernel runs in: chosen from the shape, or forced (tuning and tests);
 // returns the previous policy, -1 for an unknown one
 enum { kTileAuto = 0, kTileBig = 1, kTileMid = 2 };

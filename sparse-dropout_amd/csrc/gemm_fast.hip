@@ -82,6 +82,7 @@ using DsdMid = DsdShape<2, 4, 1, 1>;
 // fit in LDS next to the stages
 using DsdConv = DsdShape<2, 4, 1>;
 constexpr int CONV_PATCH_MAX = 163840 - DsdConv::SMEM_BYTES - 16;  // bytes left for patch + column table
+constexpr int CONV_T_PATCH_MAX = 24 * 1024;  // weight gradient: bytes of one step's copy of its input rows
 __device__ inline int step_block(uint32_t e) { return (int)(e & 0xffffu); }
 __device__ inline uint32_t step_flags(uint32_t e) { return e >> 16; }
 __device__ inline uint32_t uniform(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane(v); }
@@ -154,7 +155,7 @@ __device__ inline u32x2 lds_read_tr(const char* p) {
 template <typename T, bool TRANS, bool CM, bool RAGGED, typename S, bool IMPLICIT = false>
 __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m, int tiles_n,
                                                          int Mb, int Kb_all, ImplicitConv cg) {
-  static_assert(!IMPLICIT || (!TRANS && S::R == 4 && S::THREADS == 512), "the gather assumes 512 threads x 4 row blocks");
+  static_assert(!IMPLICIT || (S::R == 4 && S::THREADS == 512), "the gather assumes 512 threads x 4 row blocks");
   constexpr int R = S::R, BN = S::BN, THREADS = S::THREADS, NT = S::NT, STAGE = S::STAGE, A_OFF = S::A_OFF;
   constexpr int BL = S::BL, AL = S::AL, RW = S::RW;
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -223,8 +224,8 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   uint16_t* ktab = nullptr;
   uint32_t gat_base[4];  // byte offset of (this thread's tile row, tap 0) in the patch, per row block
   const int gat_row = tid / 8, gat_pc = tid % 8;  // the tile row and physical 16-byte chunk this thread builds
-  if constexpr (IMPLICIT) {
-    auto div = [](int x, uint32_t magic) { return magic ? (int)__umulhi((uint32_t)x, magic) : x; };
+  [[maybe_unused]] auto div = [](int x, uint32_t magic) { return magic ? (int)__umulhi((uint32_t)x, magic) : x; };
+  if constexpr (IMPLICIT && !TRANS) {
     const int img = rb0 / cg.blocks_per_img;
     const int p0 = (rb0 - img * cg.blocks_per_img) * cg.rpb;  // first output row of the workgroup
     const int h0 = p0 - cg.pad_h;                              // input row of patch row 0
@@ -263,6 +264,78 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
       if (dst[j] >= 0) *reinterpret_cast<u32x4*>(patch + dst[j]) = v[j];
     __syncthreads();
   }
+  // Weight gradient (reduction-strided instance): the reduction runs over output positions, so every step
+  // has its own 64 positions (rpb output rows of one image) and its own copy of the input rows they touch --
+  // only the channels of the workgroup's 256 patch-matrix columns, PR = rpb + R - 1 rows each.  Two copies
+  // alternate: the one for step s+2 is fetched into registers at the top of step s and written to LDS at
+  // its end, the tiles of step s+1 are built from the other while step s computes.  The tile a row block
+  // keeps is [64 positions][its 64 columns], rows of 128 bytes, in the swizzle of the transposing reads.
+  constexpr int TSEG = IMPLICIT && TRANS ? (CONV_T_PATCH_MAX / 16 + THREADS - 1) / THREADS : 1;
+  [[maybe_unused]] u32x4 tp_v[TSEG];      // a step's input rows on their way to LDS
+  [[maybe_unused]] int tp_dst[TSEG];      // where this thread's segments go in a copy (halfs), -1 = none
+  [[maybe_unused]] int64_t tp_src[TSEG];  // and where they come from, relative to (image, input row h0)
+  [[maybe_unused]] int tp_row[TSEG];      // their row in the copy
+  [[maybe_unused]] uint16_t* patch1 = nullptr;
+  if constexpr (IMPLICIT && TRANS) {
+    const int k_lo = rb0 * BS;
+    const int k_hi = k_lo + R * BS < cg.K ? k_lo + R * BS : cg.K;
+    const int c_lo = div(k_lo, cg.m_RS), nch = div(k_hi - 1, cg.m_RS) - c_lo + 1;
+    const int spr = cg.W / 8, spc = cg.PR * spr;
+    const int total = nch * spc, rows = nch * cg.PR;
+    patch1 = patch + cg.patch_stride;
+    ktab = patch1 + cg.patch_stride;
+#pragma unroll
+    for (int j = 0; j < TSEG; ++j) {
+      const int seg = tid + j * THREADS;
+      const int c = div(seg, cg.m_spc), rem = seg - c * spc;
+      const int row = div(rem, cg.m_spr), w8 = rem - row * spr;
+      tp_dst[j] = seg < total ? (c * cg.PR + row) * cg.PW + 8 + w8 * 8 : -1;
+      tp_src[j] = (int64_t)(c_lo + c) * cg.sc + (int64_t)row * cg.sh + w8 * 8;
+      tp_row[j] = row;
+    }
+    for (int m = tid; m <= rows; m += THREADS) {  // the halo groups of both copies; the steps never write them
+      *reinterpret_cast<u32x4*>(patch + m * cg.PW) = u32x4{0u, 0u, 0u, 0u};
+      *reinterpret_cast<u32x4*>(patch1 + m * cg.PW) = u32x4{0u, 0u, 0u, 0u};
+    }
+    for (int kl = tid; kl < R * BS; kl += THREADS) {
+      const int k = k_lo + kl;
+      const int c = div(k, cg.m_RS), tap = k - c * cg.RS;
+      const int rr = div(tap, cg.m_S), ss = tap - rr * cg.S;
+      // columns past the last one belong to rows of the result that are not stored
+      ktab[kl] = k < cg.K ? (uint16_t)((((c - c_lo) * cg.PR + rr) * cg.PW + ss) * 2) : (uint16_t)0;
+    }
+    const int prow = div(gat_row, cg.m_Q), q = gat_row - prow * cg.Q;
+    gat_base[0] = (uint32_t)((prow * cg.PW + 8 + q - cg.pad_w) * 2);
+  }
+  // fetches the input rows of the step with table word `entry` (its reduction block is a block of 64 positions)
+  [[maybe_unused]] auto tpatch_load = [&](uint32_t entry) {
+    const int mb = step_block(entry);
+    const int img = mb / cg.blocks_per_img;
+    const int h0 = (mb - img * cg.blocks_per_img) * cg.rpb - cg.pad_h;
+    const uint16_t* src = cg.x + (int64_t)img * cg.sn + (int64_t)h0 * cg.sh;
+#pragma unroll
+    for (int j = 0; j < TSEG; ++j) {
+      const int h = h0 + tp_row[j];
+      tp_v[j] = u32x4{0u, 0u, 0u, 0u};
+      if (tp_dst[j] >= 0 && h >= 0 && h < cg.H) tp_v[j] = *reinterpret_cast<const u32x4*>(src + tp_src[j]);
+    }
+  };
+  [[maybe_unused]] auto tpatch_store = [&](uint16_t* copy) {
+#pragma unroll
+    for (int j = 0; j < TSEG; ++j)
+      if (tp_dst[j] >= 0) *reinterpret_cast<u32x4*>(copy + tp_dst[j]) = tp_v[j];
+  };
+  // this thread's 16 bytes of the tile [64 positions][64 columns of row block r] from a step's copy
+  [[maybe_unused]] auto gather_tile_t = [&](int r, const uint16_t* copy, char* tile) {
+    const int lc = gat_pc ^ (((gat_row >> 1) & 1) << 2);  // logical chunk: columns r*64 + lc*8 .. +7 of the workgroup
+    const u16x8 off = *reinterpret_cast<const u16x8*>(ktab + r * BS + lc * 8);
+    const char* pb = reinterpret_cast<const char*>(copy) + gat_base[0];
+    uint32_t v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = *reinterpret_cast<const uint16_t*>(pb + off[e]);
+    *reinterpret_cast<u32x4*>(tile + gat_row * 128 + gat_pc * 16) =
+        u32x4{v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16)};
+  };
   // builds this thread's 16 bytes of the patch-matrix tile (row block r of the workgroup, reduction block kb)
   auto gather_tile = [&](int r, int kb, char* tile) {
     const int lc = gat_pc ^ ((gat_row >> 1) & 7);  // logical chunk: columns kb*64 + lc*8 .. +7
@@ -387,6 +460,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   }
   const int64_t b_red_stride = TRANS ? (int64_t)BS * g.b.sc * 2 : (int64_t)BS * 2;
 
+  [[maybe_unused]] const uint16_t* tcopy = patch;  // implicit weight gradient: the copy the next tiles are built from
   auto issue_loads = [&](uint32_t entry, int stage) {  // entry: wave-uniform step table word
     const int kb = step_block(entry);
     const uint32_t fl = step_flags(entry);
@@ -404,8 +478,12 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
 #pragma unroll
     for (int r = 0; r < R; ++r)
       if (fl & (1u << r)) {
-        if constexpr (IMPLICIT) {
+        if constexpr (IMPLICIT && !TRANS) {
           gather_tile(r, kb, st + A_OFF + r * TILE);
+          continue;
+        }
+        if constexpr (IMPLICIT && TRANS) {
+          gather_tile_t(r, tcopy, st + A_OFF + r * TILE);
           continue;
         }
 #pragma unroll
@@ -509,6 +587,17 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   // long returned: a read-and-wait at the top of a step would put an LDS round trip in front of its MFMAs.
   const bool late = __builtin_amdgcn_readfirstlane(rh) != 0;
   uint32_t e_cur = uniform(step_e[0]), e_next = uniform(step_e[1]);
+  if constexpr (IMPLICIT && TRANS) {
+    if (nsteps > 0) {
+      tpatch_load(e_cur);
+      tpatch_store(patch);
+    }
+    if (nsteps > 1) {
+      tpatch_load(e_next);
+      tpatch_store(patch1);
+    }
+    __syncthreads();  // the copies, their halo groups and the column table
+  }
   if (nsteps > 0) issue_loads(e_cur, 0);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
@@ -517,6 +606,10 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
     const int stage = step & 1;
     const uint32_t e_after = step_e[step + 2];
     const bool more = step + 1 < nsteps;
+    if constexpr (IMPLICIT && TRANS) {
+      if (step + 2 < nsteps) tpatch_load(uniform(step_e[step + 2]));
+      tcopy = ((step + 1) & 1) ? patch1 : patch;  // holds the rows of step + 1
+    }
     const uint32_t mine = (step_flags(e_cur) >> (RW * rh)) & ((1u << RW) - 1u);
     const bool mid = late && more && mine != 0u;
     if (more && !mid) issue_loads(e_next, stage ^ 1);
@@ -528,6 +621,9 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
       else if (mine == 2u) compute(std::integral_constant<int, 2>{}, st, mid, e_next, stage ^ 1, red_tail);
     } else {
       if (mine) compute(std::integral_constant<int, 1>{}, st, mid, e_next, stage ^ 1, red_tail);
+    }
+    if constexpr (IMPLICIT && TRANS) {
+      if (step + 2 < nsteps) tpatch_store((step & 1) ? patch1 : patch);  // last read for this step's tiles, a step ago
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -1027,7 +1123,57 @@ int launch_conv_t(const GemmArgs& g, const ImplicitConv& cg, int smem, hipStream
   return check_launch("dsd_kernel (implicit conv)");
 }
 
+template <typename T, bool RAGGED>
+int launch_conv_dw_t(const GemmArgs& g, const ImplicitConv& cg, int smem, int splits, hipStream_t stream) {
+  static bool configured[kMaxDevices] = {};
+  auto* kernel = &dsd_kernel<T, true, true, RAGGED, DsdConv, true>;
+  if (int rc = allow_big_lds(reinterpret_cast<const void*>(kernel), 163840, configured)) return rc;
+  const int Mb = (int)((g.M + BS - 1) / BS), Kb = (int)(g.K / BS);
+  const int tiles_m = (Mb + DsdConv::R - 1) / DsdConv::R, tiles_n = (int)((g.N + DsdConv::BN - 1) / DsdConv::BN);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits), dim3(DsdConv::THREADS), smem, stream,
+                     g, tiles_m, tiles_n, Mb, Kb, cg);
+  if (int rc = check_launch("dsd_kernel (implicit conv weight gradient)")) return rc;
+  if (splits > 1) return launch_splitk_reduce(g, splits, true, T::id, stream);
+  return SD_OK;
+}
+
 }  // namespace
+
+// g: M = C*R*S (rows of the result), N = K_out, K = N*P*Q (the reduction); b = dY^T (b.sr == 1), c column-major
+// (c_sr == 1); lists = the CSC lists of the patch matrix's mask (kept row blocks per column block).
+int launch_conv_implicit_dw(const GemmArgs& g, ImplicitConv cg, int64_t P, int64_t stride_h, int64_t stride_w,
+                            int64_t dil_h, int64_t dil_w, int64_t R, int64_t x_sw, int dtype, hipStream_t stream) {
+  if (g.row_ptr != nullptr && g.bs != BS) return SD_ERR_UNSUPPORTED;
+  const bool geom_ok = stride_h == 1 && stride_w == 1 && dil_h == 1 && dil_w == 1 && x_sw == 1 && cg.Q > 0 &&
+                       cg.Q <= BS && BS % cg.Q == 0 && (P * cg.Q) % BS == 0 && cg.W % 8 == 0 && cg.pad_h >= 0 &&
+                       cg.pad_w >= 0 && cg.pad_w <= 8 && cg.S - 1 - cg.pad_w <= 8 && R * cg.S == cg.RS &&
+                       cg.PW == cg.W + 8 && cg.PR == cg.rpb + R - 1;
+  if (!geom_ok) return SD_ERR_UNSUPPORTED;
+  const int64_t nch_max = (DsdConv::R * BS - 1) / cg.RS + 2;  // channels 256 consecutive columns can touch
+  const int64_t copy_elems = ((nch_max < cg.C ? nch_max : cg.C) * cg.PR * cg.PW + 8 + 7) & ~7LL;
+  if (copy_elems * 2 > CONV_T_PATCH_MAX) return SD_ERR_UNSUPPORTED;
+  cg.patch_stride = (int)copy_elems;
+  const int64_t extra = 2 * copy_elems * 2 + DsdConv::R * BS * 2;
+  const int smem = ((DsdConv::SMEM_BYTES + 15) & ~15) + (int)extra;
+  if (smem > 163840) return SD_ERR_UNSUPPORTED;
+  const bool align_ok = aligned16(cg.x) && cg.sn % 8 == 0 && cg.sc % 8 == 0 && cg.sh % 8 == 0 && aligned16(g.b.ptr) &&
+                        g.b.sr == 1 && g.b.sc % 8 == 0 && g.b.sc < (1 << 22) && g.c_sr == 1 && g.M % 8 == 0 &&
+                        g.N % 8 == 0 && g.K % BS == 0 && g.K / BS < 65536;
+  if (!align_ok) return SD_ERR_UNSUPPORTED;
+  // the reduction over positions is long and the result small: split it over workgroups as the explicit kernel does
+  const int64_t tiles = dsd_tiles<DsdConv>(g.M, g.N);
+  int splits = splits_for(tiles, g.M, g.N, g.K);
+  const int64_t part_bytes = g.M * g.N * 4;
+  if (splits > 1 && (g.ws == nullptr || g.ws_bytes < part_bytes * splits)) splits = g.ws ? (int)(g.ws_bytes / part_bytes) : 1;
+  if (splits < 1) splits = 1;
+  if ((g.K / BS + splits - 1) / splits > MAX_STEPS) return SD_ERR_UNSUPPORTED;
+  const bool ragged = g.M % BS != 0 || g.N % BS != 0;
+  if (dtype == SD_BF16)
+    return ragged ? launch_conv_dw_t<BF16, true>(g, cg, smem, splits, stream)
+                  : launch_conv_dw_t<BF16, false>(g, cg, smem, splits, stream);
+  return ragged ? launch_conv_dw_t<F16, true>(g, cg, smem, splits, stream)
+                : launch_conv_dw_t<F16, false>(g, cg, smem, splits, stream);
+}
 
 int launch_conv_implicit(const GemmArgs& g, const ImplicitConv& cg, int64_t P, int64_t stride_h, int64_t stride_w,
                          int64_t dil_h, int64_t dil_w, int64_t R, int64_t x_sw, int dtype, hipStream_t stream) {

@@ -91,18 +91,26 @@ class _Im2colConv2d(torch.autograd.Function):
                 dcols = ext.gemm_sdd_lists(dy2, w2.t(), lists, kernel_bs, scale, kept_only=True)
                 dx = ext.col2im(dcols, x_shape, (r, s), padding, stride, dilation, mask, block_size, ch_last)
             if ctx.needs_input_grad[1]:
-                if ctx.implicit:  # the forward kept the input, not the patch matrix: gather the kept blocks now
-                    cols = ext.im2col(cols, (r, s), padding, stride, dilation, lists, kernel_bs)
-                dk = ext.gemm_dsd_lists(cols.t(), dy2.t(), lists.transposed(), kernel_bs, scale,
-                                        transposed_out=True).t().reshape(k_shape)
+                if ctx.implicit:  # the forward kept the input, not the patch matrix
+                    dk = ext.conv2d_dw_lists(cols, dy2, lists, kernel_bs, scale, (r, s), padding, stride, dilation)
+                    if dk is None:  # gather the kept blocks now
+                        cols = ext.im2col(cols, (r, s), padding, stride, dilation, lists, kernel_bs)
+                if dk is None:
+                    dk = ext.gemm_dsd_lists(cols.t(), dy2.t(), lists.transposed(), kernel_bs, scale,
+                                            transposed_out=True).t()
+                dk = dk.reshape(k_shape)
         else:
             if ctx.needs_input_grad[0]:
                 dcols = ext.gemm(dy2, w2.t())
                 dx = ext.col2im(dcols, x_shape, (r, s), padding, stride, dilation, channels_last=ch_last)
             if ctx.needs_input_grad[1]:
                 if ctx.implicit:
-                    cols = ext.im2col(cols, (r, s), padding, stride, dilation)
-                dk = ext.gemm(cols.t(), dy2.t(), transposed_out=True).t().reshape(k_shape)
+                    dk = ext.conv2d_dw_lists(cols, dy2, None, 0, 1.0, (r, s), padding, stride, dilation)
+                    if dk is None:
+                        cols = ext.im2col(cols, (r, s), padding, stride, dilation)
+                if dk is None:
+                    dk = ext.gemm(cols.t(), dy2.t(), transposed_out=True).t()
+                dk = dk.reshape(k_shape)
         return dx, dk, None, None, None, None, None, None, None
 
 

@@ -47,6 +47,10 @@ SIGNATURES = {
                                     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                     c_void_p, c_void_p, c_int64, c_float, c_int, c_void_p]),
+    "sd_conv2d_dw_lists": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64,
+                                   c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                   c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                   c_void_p, c_void_p, c_int64, c_float, c_int, c_void_p, c_int64, c_void_p]),
     "sd_im2col": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64,
                           *([c_int64] * 12), c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "sd_col2im": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64,

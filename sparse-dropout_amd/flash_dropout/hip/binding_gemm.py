@@ -470,6 +470,46 @@ class GEMM:
             raise {1: ValueError}.get(rc, SparseDropError)(f"sd_conv2d_dsd_lists: {msg}")
         return y
 
+    def conv2d_dw_lists(self, x: torch.Tensor, dy2d: torch.Tensor, lists: KeptLists | None, block_size,
+                        scale: float, kernel_size, padding=(0, 0), stride=(1, 1),
+                        dilation=(1, 1)) -> torch.Tensor | None:
+        """Implicit-GEMM weight gradient of the block-dropout convolution: [K, C*R*S] from the input ``x`` and
+        the output gradient ``dy2d`` [N*P*Q, K], over the kept blocks of ``lists`` (the lists of the patch
+        matrix's mask; None = dense), without the patch matrix.  Returns None when the library does not take
+        the geometry."""
+        if x.dim() != 4 or not x.is_cuda or x.dtype not in _DTYPES:
+            raise ValueError("x must be a 4D float16/bfloat16 tensor on the GPU")
+        n, c, h, w = x.shape
+        r, s = kernel_size
+        p, q = self.conv_out_hw(h, w, r, s, padding, stride, dilation)
+        if p <= 0 or q <= 0:
+            raise ValueError("kernel does not fit the padded image")
+        if (dy2d.dim() != 2 or dy2d.shape[0] != n * p * q or dy2d.dtype != x.dtype or dy2d.device != x.device
+                or dy2d.stride(1) != 1):
+            raise ValueError(f"dy2d must be a [{n * p * q}, K] {x.dtype} matrix on {x.device} with unit column stride")
+        bs, cp, ri = 0, None, None
+        if lists is not None:
+            bs = _block_size(block_size)
+            want = (ceil(n * p * q / bs), ceil(c * r * s / bs))
+            if tuple(lists.shape) != want:
+                raise ValueError(f"lists are for a {lists.shape} mask, patch matrix needs {want}")
+            cp, ri = lists.col_ptr.data_ptr(), lists.row_idx.data_ptr()
+        k = dy2d.shape[1]
+        dw = torch.empty((k, c * r * s), dtype=x.dtype, device=x.device)
+        nbytes = self.lib.sd_splitk_workspace_bytes(c * r * s, k, n * p * q, 64, 1)
+        ws = torch.empty(nbytes // 4, dtype=torch.float32, device=x.device) if nbytes > 0 else None
+        with _guard(x.device):
+            rc = self.lib.sd_conv2d_dw_lists(x.data_ptr(), *x.stride(), dy2d.data_ptr(), dy2d.stride(0),
+                                             dw.data_ptr(), dw.stride(0), n, c, h, w, k, r, s, *padding, *stride,
+                                             *dilation, cp, ri, bs, float(scale), _DTYPES[x.dtype],
+                                             ws.data_ptr() if ws is not None else None, nbytes, self._stream(x))
+        if rc == 2:  # geometry not taken: nothing was launched
+            return None
+        if rc != 0:
+            msg = self.lib.sd_last_error().decode(errors="replace")
+            raise {1: ValueError}.get(rc, SparseDropError)(f"sd_conv2d_dw_lists: {msg}")
+        return dw
+
     def col2im(self, cols: torch.Tensor, x_shape, kernel_size, padding=(0, 0), stride=(1, 1),
                dilation=(1, 1), mask: torch.Tensor | None = None, block_size=None,
                channels_last: bool = False) -> torch.Tensor:

@@ -186,6 +186,40 @@ def test_implicit_gemm_conv_dense(cfg, taken):
     assert rel_fro(y, ref.permute(0, 2, 3, 1).reshape(n * p_ * q_, kk).numpy()) <= REL_FRO_TOL
 
 
+@pytest.mark.parametrize("cfg,fwd_taken", IMPLICIT_GEOMS)
+@pytest.mark.parametrize("p", [0.0, 0.5])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_implicit_gemm_conv_weight_gradient(cfg, fwd_taken, p, dtype):
+    """sd_conv2d_dw_lists (no patch matrix) against the oracle and against im2col + DSD on the transposed
+    operands; it takes every geometry the forward takes (and some more: P*Q only has to be a multiple of 64)."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(cfg["c"] * 3 + cfg["k"])
+    x = torch.randn(cfg["n"], cfg["c"], cfg["h"], cfg["w"], generator=gen).to(dtype)
+    fan_in = cfg["c"] * cfg["r"] * cfg["s"]
+    p_, q_ = O.conv_out_hw(cfg["h"], cfg["w"], cfg["r"], cfg["s"], **_geo(cfg))
+    rows = cfg["n"] * p_ * q_
+    dy2 = torch.randn(rows, cfg["k"], generator=gen).to(dtype)
+    mask = cpu_mask(O.mask_shape(rows, fan_in, 64), p, gen)
+    lists = ext.build_lists(mask.cuda())
+    s = 1 / (1 - p)
+    xg, dyg = x.cuda(), dy2.cuda()
+    dw = ext.conv2d_dw_lists(xg, dyg, lists, 64, s, (cfg["r"], cfg["s"]), **_geo(cfg))
+    if dw is None:
+        assert not fwd_taken
+        return
+    assert tuple(dw.shape) == (cfg["k"], fan_in)
+    cols = ext.im2col(xg, (cfg["r"], cfg["s"]), **_geo(cfg))
+    explicit = ext.gemm_dsd_lists(cols.t(), dyg.t(), lists.transposed(), 64, s, transposed_out=True).t()
+    assert rel_fro(dw, to_np(explicit)) <= 2e-3
+    ref = O.dsd_dw(to_np(dy2), O.im2col(to_np(x), cfg["r"], cfg["s"], **_geo(cfg)), mask.numpy(), 64, p, np.float32)
+    assert rel_fro(dw, ref) <= REL_FRO_TOL
+    if p == 0.0:  # and without lists: the dense weight gradient
+        dense = ext.conv2d_dw_lists(xg, dyg, None, 0, 1.0, (cfg["r"], cfg["s"]), **_geo(cfg))
+        assert dense is not None and rel_fro(dense, ref) <= REL_FRO_TOL
+
+
 def test_implicit_and_explicit_conv_routes_agree():
     """The autograd function with the implicit forward (input kept, kept patch blocks re-gathered for the weight
     gradient) and with the explicit one (patch matrix kept) give the same three results."""
