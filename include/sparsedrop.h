@@ -272,10 +272,11 @@ int sd_conv2d_dsd_lists(const void* x, int64_t x_stride_n, int64_t x_stride_c, i
  * (dw_ld); col_ptr / row_idx are the CSC lists of the patch matrix's mask (kept row blocks per column block; NULL,
  * NULL = dense).  The reduction runs over output positions: every step copies the input rows of its 64 positions
  * (the channels of the workgroup's 256 columns only) into LDS and builds the kept tiles from them; it is split over
- * workgroups when `workspace` (sd_splitk_workspace_bytes(C*R*S, k_out, N*P*Q, 64, dtype) bytes, may be NULL) allows.
+ * workgroups when `workspace` (sd_conv2d_dw_workspace_bytes bytes, 16-byte aligned; may be NULL) allows.
  * Taken: stride 1, dilation 1, unit w stride of x, W a multiple of 8, Q a divisor of 64, P*Q a multiple of 64,
  * C*R*S and k_out multiples of 8, one step's copy <= 24 KB.  Anything else returns SD_ERR_UNSUPPORTED with
  * nothing launched.  No counterpart in the reference. */
+int64_t sd_conv2d_dw_workspace_bytes(int64_t n, int64_t c, int64_t k_out, int64_t r, int64_t s, int64_t p, int64_t q);
 int sd_conv2d_dw_lists(const void* x, int64_t x_stride_n, int64_t x_stride_c, int64_t x_stride_h,
                        int64_t x_stride_w, const void* dy, int64_t dy_ld, void* dw, int64_t dw_ld,
                        int64_t n, int64_t c, int64_t h, int64_t w, int64_t k_out, int64_t r, int64_t s,

@@ -382,6 +382,13 @@ int sd_conv2d_dsd_lists(const void* x, int64_t sn, int64_t sc, int64_t sh, int64
   return rc;
 }
 
+int64_t sd_conv2d_dw_workspace_bytes(int64_t n, int64_t c, int64_t k_out, int64_t r, int64_t s, int64_t p, int64_t q) {
+  if (n <= 0 || c <= 0 || k_out <= 0 || r <= 0 || s <= 0 || p <= 0 || q <= 0) return 0;
+  const int64_t rows = c * r * s;
+  const int splits = conv_dw_splits(rows, k_out, n * p * q);
+  return splits > 1 ? (int64_t)splits * rows * k_out * 4 : 0;
+}
+
 int sd_conv2d_dw_lists(const void* x, int64_t sn, int64_t sc, int64_t sh, int64_t sw, const void* dy, int64_t dyld,
                        void* dw, int64_t dwld, int64_t n, int64_t c, int64_t h, int64_t w, int64_t k_out, int64_t r,
                        int64_t s, int64_t pad_h, int64_t pad_w, int64_t stride_h, int64_t stride_w, int64_t dil_h,

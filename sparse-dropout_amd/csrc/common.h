@@ -149,6 +149,8 @@ int launch_conv_implicit(const GemmArgs& g, const ImplicitConv& cg, int64_t P, i
 // dY^T, g.c column-major, the lists those of the transposed mask; cg.PR = rows one 64-position block touches.
 int launch_conv_implicit_dw(const GemmArgs& g, ImplicitConv cg, int64_t P, int64_t stride_h, int64_t stride_w,
                             int64_t dil_h, int64_t dil_w, int64_t R, int64_t x_sw, int dtype, hipStream_t stream);
+// reduction splits that launch would like for a [M x N] result over a reduction of K (1 = none)
+int conv_dw_splits(int64_t M, int64_t N, int64_t K);
 // which workgroup shape the DSD kernel runs in: chosen from the shape, or forced (tuning and tests);
 // returns the previous policy, -1 for an unknown one
 enum { kTileAuto = 0, kTileBig = 1, kTileMid = 2 };

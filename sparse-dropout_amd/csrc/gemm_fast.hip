@@ -1175,6 +1175,11 @@ int launch_conv_implicit_dw(const GemmArgs& g, ImplicitConv cg, int64_t P, int64
                 : launch_conv_dw_t<F16, false>(g, cg, smem, splits, stream);
 }
 
+int conv_dw_splits(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 1;
+  return splits_for(dsd_tiles<DsdConv>(M, N), M, N, K);
+}
+
 int launch_conv_implicit(const GemmArgs& g, const ImplicitConv& cg, int64_t P, int64_t stride_h, int64_t stride_w,
                          int64_t dil_h, int64_t dil_w, int64_t R, int64_t x_sw, int dtype, hipStream_t stream) {
   if (g.row_ptr != nullptr && g.bs != BS) return SD_ERR_UNSUPPORTED;

@@ -496,7 +496,7 @@ class GEMM:
             cp, ri = lists.col_ptr.data_ptr(), lists.row_idx.data_ptr()
         k = dy2d.shape[1]
         dw = torch.empty((k, c * r * s), dtype=x.dtype, device=x.device)
-        nbytes = self.lib.sd_splitk_workspace_bytes(c * r * s, k, n * p * q, 64, 1)
+        nbytes = self.lib.sd_conv2d_dw_workspace_bytes(n, c, k, r, s, p, q)
         ws = torch.empty(nbytes // 4, dtype=torch.float32, device=x.device) if nbytes > 0 else None
         with _guard(x.device):
             rc = self.lib.sd_conv2d_dw_lists(x.data_ptr(), *x.stride(), dy2d.data_ptr(), dy2d.stride(0),
