@@ -276,6 +276,22 @@ int sd_conv2d_dsd_lists(const void* x, int64_t x_stride_n, int64_t x_stride_c, i
  * Taken: stride 1, dilation 1, unit w stride of x, W a multiple of 8, Q a divisor of 64, P*Q a multiple of 64,
  * C*R*S and k_out multiples of 8, one step's copy <= 24 KB.  Anything else returns SD_ERR_UNSUPPORTED with
  * nothing launched.  No counterpart in the reference. */
+/* Input gradient of the same convolution in one launch: sd_gemm_sdd_lists_kept + sd_col2im without the gradient
+ * of the patch matrix in memory.  dy is [N*P*Q, k_out] row-major, weight [k_out, C*R*S] row-major, dx [N, C, H, W]
+ * addressed by element strides, fully overwritten.  mask: one byte per 64 x 64 block of the patch
+ * matrix (non-zero = dropped, strides in bytes), NULL = dense.  A workgroup keeps the dY tiles of the output rows
+ * that reach its band of input rows in LDS, forms the kept tiles of dY . W per 64-column block and folds them
+ * (deterministically: every dx element has one owner and a fixed summation order).  Taken: stride 1, dilation 1,
+ * block_size 64, k_out 64 or 128, Q a divisor of 64, P*Q a multiple of 64, C*R*S a multiple of 8 and at most 4096,
+ * R*S <= 64, small kernels relative to the row block (R - 1 <= 64/Q + 1); anything else returns SD_ERR_UNSUPPORTED
+ * with nothing launched.  No counterpart in the reference. */
+int sd_conv2d_dx(const void* dy, int64_t dy_ld, const void* weight, int64_t weight_ld,
+                 void* dx, int64_t dx_stride_n, int64_t dx_stride_c, int64_t dx_stride_h, int64_t dx_stride_w,
+                 const uint8_t* mask, int64_t mask_stride_r, int64_t mask_stride_c,
+                 int64_t n, int64_t c, int64_t h, int64_t w, int64_t k_out, int64_t r, int64_t s,
+                 int64_t pad_h, int64_t pad_w, int64_t stride_h, int64_t stride_w, int64_t dil_h, int64_t dil_w,
+                 int64_t block_size, float scale, int dtype, void* stream);
+
 int64_t sd_conv2d_dw_workspace_bytes(int64_t n, int64_t c, int64_t k_out, int64_t r, int64_t s, int64_t p, int64_t q);
 int sd_conv2d_dw_lists(const void* x, int64_t x_stride_n, int64_t x_stride_c, int64_t x_stride_h,
                        int64_t x_stride_w, const void* dy, int64_t dy_ld, void* dw, int64_t dw_ld,

@@ -382,6 +382,25 @@ int sd_conv2d_dsd_lists(const void* x, int64_t sn, int64_t sc, int64_t sh, int64
   return rc;
 }
 
+int sd_conv2d_dx(const void* dy, int64_t dy_ld, const void* weight, int64_t weight_ld, void* dx, int64_t sn,
+                 int64_t sc, int64_t sh, int64_t sw, const uint8_t* mask, int64_t msr, int64_t msc, int64_t n,
+                 int64_t c, int64_t h, int64_t w, int64_t k_out, int64_t r, int64_t s, int64_t pad_h, int64_t pad_w,
+                 int64_t stride_h, int64_t stride_w, int64_t dil_h, int64_t dil_w, int64_t bs, float scale, int dtype,
+                 void* stream) {
+  SD_REQUIRE(dtype == SD_F16 || dtype == SD_BF16, "dtype must be SD_F16 or SD_BF16 (got %d)", dtype);
+  SD_REQUIRE(dy && weight && dx, "null pointer argument");
+  SD_REQUIRE(n > 0 && c > 0 && h > 0 && w > 0 && k_out > 0 && r > 0 && s > 0, "sizes must be positive");
+  SD_REQUIRE(stride_h > 0 && stride_w > 0 && dil_h > 0 && dil_w > 0 && pad_h >= 0 && pad_w >= 0,
+             "strides and dilations must be positive, paddings non-negative");
+  SD_REQUIRE(scale == scale, "scale is NaN");
+  if (mask != nullptr && bs != 64) return SD_ERR_UNSUPPORTED;
+  if (h > (1 << 20) || w > (1 << 12) || c * r * s > (1 << 16)) return SD_ERR_UNSUPPORTED;
+  const int rc = launch_conv_dx(dy, dy_ld, weight, weight_ld, dx, sn, sc, sh, sw, mask, msr, msc, n, c, h, w, k_out, r,
+                                s, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, scale, dtype, (hipStream_t)stream);
+  if (rc == SD_OK) last_kernel = "specialised";
+  return rc;
+}
+
 int64_t sd_conv2d_dw_workspace_bytes(int64_t n, int64_t c, int64_t k_out, int64_t r, int64_t s, int64_t p, int64_t q) {
   if (n <= 0 || c <= 0 || k_out <= 0 || r <= 0 || s <= 0 || p <= 0 || q <= 0) return 0;
   const int64_t rows = c * r * s;

@@ -151,6 +151,13 @@ int launch_conv_implicit_dw(const GemmArgs& g, ImplicitConv cg, int64_t P, int64
                             int64_t dil_h, int64_t dil_w, int64_t R, int64_t x_sw, int dtype, hipStream_t stream);
 // reduction splits that launch would like for a [M x N] result over a reduction of K (1 = none)
 int conv_dw_splits(int64_t M, int64_t N, int64_t K);
+// input gradient of the stride-1 convolution straight from dY and the weights (kept 64 x 64 tiles of the patch
+// matrix's gradient are formed and folded in LDS); SD_ERR_UNSUPPORTED without a message for what it does not take
+int launch_conv_dx(const void* dy, int64_t dy_ld, const void* w, int64_t w_ld, void* dx, int64_t sn, int64_t sc,
+                   int64_t sh, int64_t sw, const uint8_t* mask, int64_t msr, int64_t msc, int64_t n, int64_t c,
+                   int64_t h, int64_t wd, int64_t k_out, int64_t r, int64_t s, int64_t pad_h, int64_t pad_w,
+                   int64_t stride_h, int64_t stride_w, int64_t dil_h, int64_t dil_w, float scale, int dtype,
+                   hipStream_t stream);
 // which workgroup shape the DSD kernel runs in: chosen from the shape, or forced (tuning and tests);
 // returns the previous policy, -1 for an unknown one
 enum { kTileAuto = 0, kTileBig = 1, kTileMid = 2 };

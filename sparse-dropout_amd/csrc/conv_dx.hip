@@ -1,0 +1,334 @@
+// Input gradient of the (block-dropout) convolution in one launch, without the gradient of the patch
+// matrix ever reaching memory:
+//
+//   dx[n, c, h, w] = scale * sum over taps (r, s) of keep[m / 64, k / 64] * (dY . W)[m, k]
+//   with m = (n, h - r + pad_h, w - s + pad_w) the output position the tap reads from and k = (c, r, s)
+//
+// i.e. the SDD product dY . W restricted to kept 64 x 64 tiles followed by col2im (the adjoint of the
+// F.unfold gather of flash_dropout/functional/im2col_conv2d.py:17-20), for stride 1 and dilation 1.
+//
+// A workgroup owns HB = 2 * (64 / Q) input rows of one image, all channels.  The output rows whose taps
+// reach them lie in at most four consecutive 64-position row blocks of dY; their dY tiles (all of the
+// reduction, K_out <= 128) stay in LDS for the whole kernel.  Then, for every 64-column block of the patch
+// matrix in turn: the W tile of the block arrives by direct loads (double buffered), every wave multiplies
+// one 32-row half of one dY tile with it (MFMA, fp32) if the mask keeps that tile and writes the scaled
+// result, rounded once as the two-kernel route rounds it, to an LDS staging area; after a barrier each
+// thread, owner of a fixed (input row, w) and of a few of the block's channels, adds up the taps of its
+// elements that fall in this block from the staging area.  A channel's R*S columns span at most two
+// consecutive blocks, so its sums are carried in a small fp32 ring in LDS and written out once, when its last
+// column has been seen.  Every sum has one owner and a fixed order: the result is deterministic.
+#include "common.h"
+
+namespace sd {
+namespace {
+
+constexpr int BS = 64;
+constexpr int TILE = BS * BS * 2;
+constexpr int THREADS = 512;
+constexpr int NB = 4;           // row blocks of dY per workgroup
+constexpr int KS_MAX = 2;       // 64-wide reduction steps: K_out <= 128
+constexpr int STAGE_LD = 68;    // halfs per staged row: 64 + 4 so that the two half-waves of a store hit different banks
+constexpr int OFF_W = NB * KS_MAX * TILE;                 // 64 KB of dY tiles, then
+constexpr int OFF_STAGE = OFF_W + 2 * KS_MAX * TILE;      // two W tiles of 16 KB, then
+constexpr int OFF_ACC = OFF_STAGE + NB * BS * STAGE_LD * 2;  // the staging area, then the ring
+constexpr int DYN_LDS_MAX = 163840 - 256;  // the kernel also has a few bytes of static LDS
+constexpr int ACC_MAX = DYN_LDS_MAX - OFF_ACC;  // bytes left for the ring of open channel sums
+
+typedef __attribute__((address_space(3))) void lds_void;
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+
+// wave-wide 1 KB direct global->LDS load (lane i's 16 bytes land at lds_dst + 16*i); issued as assembly so
+// that the compiler keeps counting LDS reads precisely, waited for with an explicit vmcnt(0)
+__device__ inline void load16_to_lds(const void* g, char* lds_dst) {
+  const uint32_t a = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_void*)lds_dst);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(a) : "memory");
+}
+__device__ inline u32x2 lds_read_tr(const char* p) {
+  s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p);
+  return __builtin_bit_cast(u32x2, v);
+}
+
+struct DxArgs {
+  const uint16_t* dy;  // [N*P*Q, K_out], row-major
+  int64_t dy_ld;
+  const uint16_t* w;   // [K_out, C*R*S], row-major
+  int64_t w_ld;
+  uint16_t* dx;        // [N, C, H, W] by element strides
+  int64_t sn, sc, sh, sw;
+  const uint8_t* mask;  // [N*P*Q/64, ceil(C*R*S/64)] bytes, non-zero = dropped; null = keep everything
+  int64_t msr, msc;
+  int C, H, W, P, Q, R, S, pad_h, pad_w;
+  int rpb_shift;        // log2(64 / Q): output rows per row block
+  int HB, bands;        // input rows per workgroup, workgroups per image
+  int blocks_per_img;   // P * Q / 64
+  int K, Kb, KS;        // C*R*S, its 64-blocks, K_out / 64
+  int ring_n;           // channels whose sums can be open at once: those of one block column plus the carried ones
+  float scale;
+};
+
+// RT, ST: the kernel size at compile time (the tap loops unroll and the per-tap address terms become per-thread
+// constants), or 0, 0 for any size.
+template <typename T, int RT, int ST>
+__global__ __launch_bounds__(THREADS) void conv_dx_kernel(DxArgs g) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  char* dyt = smem;
+  char* wt = smem + OFF_W;
+  uint16_t* stage = reinterpret_cast<uint16_t*>(smem + OFF_STAGE);
+  float* ring = reinterpret_cast<float*>(smem + OFF_ACC);
+
+  const int tid = threadIdx.x, lane = tid % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  const int img = blockIdx.x / g.bands, band = blockIdx.x - img * g.bands;
+  const int h0 = band * g.HB;
+  const int RS = RT > 0 ? RT * ST : g.R * g.S;
+  const int rpb = 1 << g.rpb_shift;
+  // output rows the taps of input rows [h0, h0 + HB) read: p = h - r + pad_h
+  const int p_lo = h0 - (g.R - 1) + g.pad_h;
+  const int pb0 = p_lo >> g.rpb_shift;  // arithmetic shift: floor, also below zero
+  const int pbn = g.P >> g.rpb_shift;   // row blocks per image
+
+  // ---- keep flags of the four row blocks: bit j = block column j kept ----------------------------------
+  __shared__ uint64_t keep[NB];  // in LDS: indexed by run-time row blocks below
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    const int pb = pb0 + b;
+    const bool valid = pb >= 0 && pb < pbn;
+    bool k = valid && lane < g.Kb;
+    if (k && g.mask) k = g.mask[((int64_t)img * g.blocks_per_img + pb) * g.msr + lane * g.msc] == 0;
+    const uint64_t bits = __ballot(k);
+    if (tid == 0) keep[b] = bits;
+  }
+  __syncthreads();
+
+  // ---- dY tiles, the first W tile, the ring -------------------------------------------------------------
+  const int ld_row = wave * 8 + lane / 8, ld_pch = lane % 8;
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    if (keep[b] == 0) continue;  // outside the image, or nothing kept
+    const int64_t m = ((int64_t)img * g.blocks_per_img + pb0 + b) * BS + ld_row;
+    for (int ks = 0; ks < g.KS; ++ks)
+      load16_to_lds(g.dy + m * g.dy_ld + ks * BS + (ld_pch ^ ((ld_row >> 1) & 7)) * 8,
+                    dyt + (b * KS_MAX + ks) * TILE + wave * 1024);
+  }
+  // W tile of block column j, reduction step ks: rows = reduction index, 64 columns = 128 bytes each
+  auto load_w = [&](int j, int buf) {
+    int chunk = ld_pch ^ (((ld_row >> 1) & 1) << 2);
+    if (j * BS + chunk * 8 >= g.K) chunk = 0;  // past the last column: never gathered, only kept readable
+    for (int ks = 0; ks < g.KS; ++ks)
+      load16_to_lds(g.w + (int64_t)(ks * BS + ld_row) * g.w_ld + j * BS + chunk * 8,
+                    wt + (buf * KS_MAX + ks) * TILE + wave * 1024);
+  };
+  load_w(0, 0);
+  const int hw_n = g.HB * g.W;  // elements per channel in the band
+  for (int i = tid; i < g.ring_n * hw_n; i += THREADS) ring[i] = 0.f;
+
+  // ---- per-lane fragment offsets (the tile layouts of the GEMM kernels) ----------------------------------
+  const int t_blk = wave >> 1, half = wave & 1;  // this wave's dY tile and its 32-row half
+  int a_off[4], b_off[4];
+  {
+    const int fr_sw = (lane >> 1) & 7;
+    const int b4 = lane / 16, e = (lane % 16) / 4, j4 = lane % 4;
+    const int row = 8 * (b4 / 2) + e;
+    const int b_ch = (2 * (b4 % 2) + j4 / 2) ^ (((e >> 1) & 1) << 2);
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      a_off[kk] = (half * 32 + lane % 32) * 128 + ((2 * kk + lane / 32) ^ fr_sw) * 16;
+      b_off[kk] = (16 * kk + row) * 128 + b_ch * 16 + (j4 % 2) * 8;  // ^ 64 for the second 32 columns
+    }
+  }
+  // ---- this thread's fixed (input row, w) and channel phase for the gather ------------------------------
+  const int groups = THREADS / hw_n;            // channels handled per pass over the block's channels (>= 1)
+  const int cgrp = tid / hw_n;                  // >= groups: idle in the gather
+  const int hw = tid - cgrp * hw_n;
+  const int hl = hw / g.W, wq = hw - hl * g.W;
+  const int h = h0 + hl;
+
+  // known kernel size: per tap row the staged row it reads and the keep word of its row block, per tap column
+  // the position inside that row (-1: the tap falls outside the output)
+  constexpr int RN = RT > 0 ? RT : 1, SN = ST > 0 ? ST : 1;
+  [[maybe_unused]] uint64_t tap_keep[RN];
+  [[maybe_unused]] int tap_row[RN], tap_col[SN];
+  if constexpr (RT > 0) {
+#pragma unroll
+    for (int rr = 0; rr < RT; ++rr) {
+      const int p = h - rr + g.pad_h;
+      const bool ok = p >= 0 && p < g.P && h < g.H;
+      const int b = ok ? (p >> g.rpb_shift) - pb0 : 0;
+      tap_keep[rr] = ok ? keep[b] : 0ull;
+      tap_row[rr] = (b * BS + (p - (pb0 + b) * rpb) * g.Q) * STAGE_LD;
+    }
+#pragma unroll
+    for (int ss = 0; ss < ST; ++ss) {
+      const int q = wq - ss + g.pad_w;
+      tap_col[ss] = (q >= 0 && q < g.Q) ? q * STAGE_LD : -1;
+    }
+  }
+
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  for (int j = 0; j < g.Kb; ++j) {
+    if (j + 1 < g.Kb) load_w(j + 1, (j + 1) & 1);
+    // ---- kept tiles of this block column: MFMA, scale, round, stage ------------------------------------
+    if ((keep[t_blk] >> j) & 1ull) {
+      f32x16 acc[2];
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[nt][v] = 0.f;
+      for (int ks = 0; ks < g.KS; ++ks) {
+        const char* at = dyt + (t_blk * KS_MAX + ks) * TILE;
+        const char* bt = wt + ((j & 1) * KS_MAX + ks) * TILE;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          const u32x4 af = *reinterpret_cast<const u32x4*>(at + a_off[kk]);
+#pragma unroll
+          for (int nt = 0; nt < 2; ++nt) {
+            const char* p = bt + (b_off[kk] ^ (nt * 64));
+            const u32x2 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * 128);
+            acc[nt] = T::mfma32(af, u32x4{lo.x, lo.y, hi.x, hi.y}, acc[nt]);
+          }
+        }
+      }
+      uint16_t* st = stage + (t_blk * BS + half * 32) * STAGE_LD;
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int row = 8 * (v / 4) + 4 * (lane / 32) + (v % 4);
+          st[row * STAGE_LD + nt * 32 + lane % 32] = T::from_float(acc[nt][v] * g.scale);
+        }
+    }
+    __syncthreads();
+    // ---- the taps of this block column, summed into the owners' ring entries ----------------------------
+    {
+      const int k_lo = j * BS, k_hi = (k_lo + BS < g.K ? k_lo + BS : g.K) - 1;
+      const int c_lo = k_lo / RS, c_hi = k_hi / RS;
+      if (cgrp < groups && h < g.H) {
+        int slot = (c_lo + cgrp) % g.ring_n;
+        for (int c = c_lo + cgrp; c <= c_hi; c += groups) {
+          float sum = 0.f;
+          int k = c * RS - k_lo;  // column of tap (0, 0) inside the block (may be negative)
+          if constexpr (RT > 0) {
+#pragma unroll
+            for (int rr = 0; rr < RT; ++rr) {
+              const bool row_ok = (tap_keep[rr] >> j) & 1ull;
+#pragma unroll
+              for (int ss = 0; ss < ST; ++ss, ++k)
+                if (row_ok && tap_col[ss] >= 0 && (unsigned)k < (unsigned)BS)
+                  sum += T::to_float(stage[tap_row[rr] + tap_col[ss] + k]);
+            }
+          } else {
+            for (int rr = 0; rr < g.R; ++rr) {
+              const int p = h - rr + g.pad_h;
+              const int b = (p >> g.rpb_shift) - pb0;
+              const bool row_ok = p >= 0 && p < g.P && ((keep[b & (NB - 1)] >> j) & 1ull);
+              const uint16_t* srow = stage + ((b & (NB - 1)) * BS + (p - (pb0 + b) * rpb) * g.Q) * STAGE_LD;
+              for (int ss = 0; ss < g.S; ++ss, ++k) {
+                const int q = wq - ss + g.pad_w;
+                if (row_ok && k >= 0 && k < BS && q >= 0 && q < g.Q) sum += T::to_float(srow[q * STAGE_LD + k]);
+              }
+            }
+          }
+          float* r = ring + (slot * hw_n + hw);
+          slot += groups;
+          if (slot >= g.ring_n) slot -= g.ring_n;
+          const float total = *r + sum;
+          if (c * RS + RS - 1 <= k_hi) {  // the channel's last column is in this block: done
+            g.dx[(int64_t)img * g.sn + (int64_t)c * g.sc + (int64_t)h * g.sh + (int64_t)wq * g.sw] = T::from_float(total);
+            *r = 0.f;
+          } else {
+            *r = total;
+          }
+        }
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+}
+
+template <typename T, int RT, int ST>
+int launch_t(const DxArgs& g, int64_t wgs, int smem, hipStream_t stream) {
+  static bool configured[16] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16)
+    return fail(SD_ERR_RUNTIME, "hipGetDevice failed or device index out of range");
+  if (!configured[dev]) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_dx_kernel<T, RT, ST>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, DYN_LDS_MAX);
+    if (e != hipSuccess) return fail(SD_ERR_RUNTIME, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured[dev] = true;
+  }
+  hipLaunchKernelGGL((conv_dx_kernel<T, RT, ST>), dim3((unsigned)wgs), dim3(THREADS), smem, stream, g);
+  return check_launch("conv_dx_kernel");
+}
+
+}  // namespace
+
+// Returns SD_ERR_UNSUPPORTED (no message, nothing launched) for geometries the kernel does not take.
+int launch_conv_dx(const void* dy, int64_t dy_ld, const void* w, int64_t w_ld, void* dx, int64_t sn, int64_t sc,
+                   int64_t sh, int64_t sw, const uint8_t* mask, int64_t msr, int64_t msc, int64_t n, int64_t c,
+                   int64_t h, int64_t wd, int64_t k_out, int64_t r, int64_t s, int64_t pad_h, int64_t pad_w,
+                   int64_t stride_h, int64_t stride_w, int64_t dil_h, int64_t dil_w, float scale, int dtype,
+                   hipStream_t stream) {
+  if (stride_h != 1 || stride_w != 1 || dil_h != 1 || dil_w != 1) return SD_ERR_UNSUPPORTED;
+  const int64_t P = h + 2 * pad_h - r + 1, Q = wd + 2 * pad_w - s + 1;
+  if (P <= 0 || Q <= 0 || Q > BS || BS % Q != 0 || (P * Q) % BS != 0) return SD_ERR_UNSUPPORTED;
+  if (k_out % BS != 0 || k_out > BS * KS_MAX) return SD_ERR_UNSUPPORTED;
+  const int64_t K = c * r * s, Kb = (K + BS - 1) / BS;
+  if (Kb > 64 || K % 8 != 0 || r * s > BS) return SD_ERR_UNSUPPORTED;  // keep flags are one 64-bit word per row block
+  const int64_t rpb = BS / Q, HB = 2 * rpb;
+  // the output rows one band's taps read must fit the four row blocks held in LDS
+  // (first row p_lo = h0 - (R-1) + pad_h lies up to rpb-1 rows into its block)
+  if ((rpb - 1) + HB + (r - 1) > NB * rpb) return SD_ERR_UNSUPPORTED;
+  const int64_t hw_n = HB * wd;
+  // a channel's columns span at most two blocks; the ring holds every channel a block column can touch
+  const int64_t ring_n = (BS + r * s - 1) / (r * s) + 2;
+  if (hw_n > THREADS || ring_n * hw_n * 4 > ACC_MAX) return SD_ERR_UNSUPPORTED;
+  const bool align_ok = reinterpret_cast<uintptr_t>(dy) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
+                        dy_ld % 8 == 0 && w_ld % 8 == 0 && dy_ld >= k_out && w_ld >= K;
+  if (!align_ok) return SD_ERR_UNSUPPORTED;
+  const int64_t bands = (h + HB - 1) / HB;
+  const int64_t wgs = n * bands;
+  if (wgs > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
+  DxArgs g;
+  g.dy = static_cast<const uint16_t*>(dy);
+  g.dy_ld = dy_ld;
+  g.w = static_cast<const uint16_t*>(w);
+  g.w_ld = w_ld;
+  g.dx = static_cast<uint16_t*>(dx);
+  g.sn = sn;
+  g.sc = sc;
+  g.sh = sh;
+  g.sw = sw;
+  g.mask = mask;
+  g.msr = msr;
+  g.msc = msc;
+  g.C = (int)c;
+  g.H = (int)h;
+  g.W = (int)wd;
+  g.P = (int)P;
+  g.Q = (int)Q;
+  g.R = (int)r;
+  g.S = (int)s;
+  g.pad_h = (int)pad_h;
+  g.pad_w = (int)pad_w;
+  g.rpb_shift = 0;
+  while ((1 << g.rpb_shift) < rpb) ++g.rpb_shift;
+  g.HB = (int)HB;
+  g.bands = (int)bands;
+  g.blocks_per_img = (int)(P * Q / BS);
+  g.K = (int)K;
+  g.Kb = (int)Kb;
+  g.KS = (int)(k_out / BS);
+  g.scale = scale;
+  g.ring_n = (int)ring_n;
+  const int smem = OFF_ACC + (int)(ring_n * hw_n * 4);
+  if (r == 3 && s == 3)
+    return dtype == SD_BF16 ? launch_t<BF16, 3, 3>(g, wgs, smem, stream) : launch_t<F16, 3, 3>(g, wgs, smem, stream);
+  return dtype == SD_BF16 ? launch_t<BF16, 0, 0>(g, wgs, smem, stream) : launch_t<F16, 0, 0>(g, wgs, smem, stream);
+}
+
+}  // namespace sd

@@ -23,6 +23,8 @@ from ..hip.binding_gemm import GEMM, KeptLists, _block_size
 # Use the implicit-GEMM forward (sd_conv2d_dsd_lists) where the library takes the geometry.  Module-level
 # switch so that tests and benchmarks can compare both routes.
 IMPLICIT_FORWARD = True
+# Use the one-launch input gradient (sd_conv2d_dx) where the library takes the geometry.
+FUSED_INPUT_GRADIENT = True
 
 
 def _pair(v) -> tuple[int, int]:
@@ -87,9 +89,13 @@ class _Im2colConv2d(torch.autograd.Function):
             lists = KeptLists(saved[3], saved[4], saved[5], saved[6], ctx.list_shape)
             scale = 1.0 / (1.0 - p)
             if ctx.needs_input_grad[0]:
-                # col2im skips the dropped blocks, so the SDD need not zero them
-                dcols = ext.gemm_sdd_lists(dy2, w2.t(), lists, kernel_bs, scale, kept_only=True)
-                dx = ext.col2im(dcols, x_shape, (r, s), padding, stride, dilation, mask, block_size, ch_last)
+                if FUSED_INPUT_GRADIENT and block_size == 64:
+                    dx = ext.conv2d_dx(dy2, w2, x_shape, (r, s), padding, stride, dilation, mask, block_size, scale,
+                                       ch_last)
+                if dx is None:
+                    # col2im skips the dropped blocks, so the SDD need not zero them
+                    dcols = ext.gemm_sdd_lists(dy2, w2.t(), lists, kernel_bs, scale, kept_only=True)
+                    dx = ext.col2im(dcols, x_shape, (r, s), padding, stride, dilation, mask, block_size, ch_last)
             if ctx.needs_input_grad[1]:
                 if ctx.implicit:  # the forward kept the input, not the patch matrix
                     dk = ext.conv2d_dw_lists(cols, dy2, lists, kernel_bs, scale, (r, s), padding, stride, dilation)
@@ -101,8 +107,11 @@ class _Im2colConv2d(torch.autograd.Function):
                 dk = dk.reshape(k_shape)
         else:
             if ctx.needs_input_grad[0]:
-                dcols = ext.gemm(dy2, w2.t())
-                dx = ext.col2im(dcols, x_shape, (r, s), padding, stride, dilation, channels_last=ch_last)
+                if FUSED_INPUT_GRADIENT:
+                    dx = ext.conv2d_dx(dy2, w2, x_shape, (r, s), padding, stride, dilation, channels_last=ch_last)
+                if dx is None:
+                    dcols = ext.gemm(dy2, w2.t())
+                    dx = ext.col2im(dcols, x_shape, (r, s), padding, stride, dilation, channels_last=ch_last)
             if ctx.needs_input_grad[1]:
                 if ctx.implicit:
                     dk = ext.conv2d_dw_lists(cols, dy2, None, 0, 1.0, (r, s), padding, stride, dilation)

@@ -47,6 +47,11 @@ SIGNATURES = {
                                     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                     c_void_p, c_void_p, c_int64, c_float, c_int, c_void_p]),
+    "sd_conv2d_dx": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                             c_void_p, c_int64, c_int64,
+                             c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                             c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                             c_int64, c_float, c_int, c_void_p]),
     "sd_conv2d_dw_workspace_bytes": (c_int64, [c_int64] * 7),
     "sd_conv2d_dw_lists": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64,
                                    c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,

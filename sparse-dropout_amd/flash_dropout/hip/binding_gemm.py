@@ -510,6 +510,42 @@ class GEMM:
             raise {1: ValueError}.get(rc, SparseDropError)(f"sd_conv2d_dw_lists: {msg}")
         return dw
 
+    def conv2d_dx(self, dy2d: torch.Tensor, weight2d: torch.Tensor, x_shape, kernel_size, padding=(0, 0),
+                  stride=(1, 1), dilation=(1, 1), mask: torch.Tensor | None = None, block_size=None,
+                  scale: float = 1.0, channels_last: bool = False) -> torch.Tensor | None:
+        """Input gradient of the (block-dropout) convolution in one launch: ``dy2d`` [N*P*Q, K] and
+        ``weight2d`` [K, C*R*S] -> [N, C, H, W], the patch matrix's gradient never in memory.  ``mask`` is the
+        block mask of the patch matrix (True = dropped).  Returns None when the library does not take the
+        geometry (the caller then goes through :meth:`gemm_sdd_lists` and :meth:`col2im`)."""
+        n, c, h, w = x_shape
+        r, s = kernel_size
+        p, q = self.conv_out_hw(h, w, r, s, padding, stride, dilation)
+        if (dy2d.dim() != 2 or not dy2d.is_cuda or dy2d.dtype not in _DTYPES or dy2d.stride(1) != 1
+                or dy2d.shape[0] != n * p * q):
+            raise ValueError(f"dy2d must be a row-major [{n * p * q}, K] float16/bfloat16 matrix on the GPU")
+        k = dy2d.shape[1]
+        if (tuple(weight2d.shape) != (k, c * r * s) or weight2d.dtype != dy2d.dtype or weight2d.device != dy2d.device
+                or weight2d.stride(1) != 1):
+            raise ValueError(f"weight2d must be a [{k}, {c * r * s}] {dy2d.dtype} matrix with unit column stride")
+        mp, msr, msc, bs = None, 0, 0, 64
+        if mask is not None:
+            bs = _block_size(block_size)
+            mask = _check_mask(mask, (ceil(n * p * q / bs), ceil(c * r * s / bs)), dy2d)
+            mp = mask.data_ptr()
+            msr, msc = _mask_strides(mask)
+        fmt = torch.channels_last if channels_last else torch.contiguous_format
+        dx = torch.empty((n, c, h, w), dtype=dy2d.dtype, device=dy2d.device, memory_format=fmt)
+        with _guard(dy2d.device):
+            rc = self.lib.sd_conv2d_dx(dy2d.data_ptr(), dy2d.stride(0), weight2d.data_ptr(), weight2d.stride(0),
+                                       dx.data_ptr(), *dx.stride(), mp, msr, msc, n, c, h, w, k, r, s, *padding,
+                                       *stride, *dilation, bs, float(scale), _DTYPES[dy2d.dtype], self._stream(dy2d))
+        if rc == 2:  # geometry not taken: nothing was launched
+            return None
+        if rc != 0:
+            msg = self.lib.sd_last_error().decode(errors="replace")
+            raise {1: ValueError}.get(rc, SparseDropError)(f"sd_conv2d_dx: {msg}")
+        return dx
+
     def col2im(self, cols: torch.Tensor, x_shape, kernel_size, padding=(0, 0), stride=(1, 1),
                dilation=(1, 1), mask: torch.Tensor | None = None, block_size=None,
                channels_last: bool = False) -> torch.Tensor:

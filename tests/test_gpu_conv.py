@@ -220,6 +220,63 @@ def test_implicit_gemm_conv_weight_gradient(cfg, fwd_taken, p, dtype):
         assert dense is not None and rel_fro(dense, ref) <= REL_FRO_TOL
 
 
+DX_GEOMS = [
+    (dict(n=4, c=64, h=32, w=32, k=128, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),   # the conv configuration's layer
+    (dict(n=2, c=16, h=16, w=16, k=64, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),    # 144 columns: ragged last block
+    (dict(n=2, c=16, h=33, w=33, k=128, r=2, s=2, padding=(0, 0), stride=(1, 1), dilation=(1, 1)), True),   # 2x2 on a 33 x 33 image: one block column, 18 open channels
+    (dict(n=2, c=64, h=32, w=32, k=128, r=1, s=1, padding=(0, 0), stride=(1, 1), dilation=(1, 1)), False),  # 1x1: 64 channels per block column do not fit the ring
+    (dict(n=2, c=32, h=16, w=64, k=64, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),    # one output row per block
+    (dict(n=3, c=24, h=32, w=8, k=128, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),    # 8 output rows per block
+    (dict(n=2, c=16, h=34, w=32, k=64, r=3, s=1, padding=(0, 0), stride=(1, 1), dilation=(1, 1)), True),    # no padding, H not a multiple of the band
+    (dict(n=2, c=8, h=16, w=16, k=64, r=5, s=5, padding=(2, 2), stride=(1, 1), dilation=(1, 1)), True),     # 25 taps, 4 output rows per block
+    (dict(n=2, c=40, h=32, w=32, k=128, r=2, s=2, padding=(0, 0), stride=(1, 1), dilation=(1, 1)), False),  # Q = 31
+    (dict(n=3, c=8, h=32, w=32, k=64, r=5, s=5, padding=(2, 2), stride=(1, 1), dilation=(1, 1)), False),    # 5 taps high on 2-row blocks
+    (dict(n=2, c=16, h=16, w=16, k=40, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), False),   # K_out = 40
+    (dict(n=2, c=8, h=32, w=32, k=64, r=3, s=3, padding=(1, 1), stride=(2, 2), dilation=(1, 1)), False),    # stride
+]
+
+
+@pytest.mark.parametrize("cfg,taken", DX_GEOMS)
+@pytest.mark.parametrize("p", [0.0, 0.5])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("channels_last", [False, True])
+def test_fused_conv_input_gradient(cfg, taken, p, dtype, channels_last):
+    """sd_conv2d_dx (kept tiles of dY.W formed and folded in LDS) against the oracle's dx and against the
+    two-kernel route; run twice, the result must be bitwise the same (one owner and one order per sum)."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(cfg["c"] * 5 + cfg["k"])
+    shape = (cfg["n"], cfg["c"], cfg["h"], cfg["w"])
+    fan_in = cfg["c"] * cfg["r"] * cfg["s"]
+    kern = ((torch.rand(cfg["k"], cfg["c"], cfg["r"], cfg["s"], generator=gen) * 2 - 1) * fan_in ** -0.5).to(dtype)
+    p_, q_ = O.conv_out_hw(cfg["h"], cfg["w"], cfg["r"], cfg["s"], **_geo(cfg))
+    rows = cfg["n"] * p_ * q_
+    dy2 = torch.randn(rows, cfg["k"], generator=gen).to(dtype)
+    mask = cpu_mask(O.mask_shape(rows, fan_in, 64), p, gen)
+    s = 1 / (1 - p)
+    w2 = kern.cuda().reshape(cfg["k"], fan_in)
+    dx = ext.conv2d_dx(dy2.cuda(), w2, shape, (cfg["r"], cfg["s"]), mask=mask.cuda(), block_size=64, scale=s,
+                       channels_last=channels_last, **_geo(cfg))
+    if not taken:
+        assert dx is None
+        return
+    assert dx is not None and tuple(dx.shape) == shape
+    again = ext.conv2d_dx(dy2.cuda(), w2, shape, (cfg["r"], cfg["s"]), mask=mask.cuda(), block_size=64, scale=s,
+                          channels_last=channels_last, **_geo(cfg))
+    assert torch.equal(dx, again)
+    lists = ext.build_lists(mask.cuda())
+    dcols = ext.gemm_sdd_lists(dy2.cuda(), w2.t(), lists, 64, s)
+    two_step = ext.col2im(dcols, shape, (cfg["r"], cfg["s"]), mask=mask.cuda(), block_size=64, **_geo(cfg))
+    assert rel_fro(dx, to_np(two_step)) <= 2e-3
+    ref = O.col2im(O.sdd_dx(to_np(dy2), to_np(w2.cpu()), mask.numpy(), 64, p, np.float32), shape, cfg["r"], cfg["s"],
+                   **_geo(cfg))
+    assert rel_fro(dx, ref) <= REL_FRO_TOL
+    if p == 0.0:  # no mask: the dense input gradient
+        dense = ext.conv2d_dx(dy2.cuda(), w2, shape, (cfg["r"], cfg["s"]), **_geo(cfg))
+        assert dense is not None and rel_fro(dense, ref) <= REL_FRO_TOL
+
+
 def test_implicit_and_explicit_conv_routes_agree():
     """The autograd function with the implicit forward (input kept, kept patch blocks re-gathered for the weight
     gradient) and with the explicit one (patch matrix kept) give the same three results."""
@@ -236,6 +293,7 @@ def test_implicit_and_explicit_conv_routes_agree():
     out = {}
     for implicit in (True, False):
         prev, mod.IMPLICIT_FORWARD = mod.IMPLICIT_FORWARD, implicit
+        prev_dx, mod.FUSED_INPUT_GRADIENT = mod.FUSED_INPUT_GRADIENT, implicit
         try:
             xg, kg = x.clone().requires_grad_(), k.clone().requires_grad_()
             y = F.blockwise_dropout_conv2d_mask(xg, mask, 64, 0.5, kg, padding=(1, 1))
@@ -243,6 +301,7 @@ def test_implicit_and_explicit_conv_routes_agree():
             out[implicit] = (y.detach(), xg.grad, kg.grad)
         finally:
             mod.IMPLICIT_FORWARD = prev
+            mod.FUSED_INPUT_GRADIENT = prev_dx
     for a, b, what in zip(out[True], out[False], ("y", "dx", "dk")):
         assert rel_fro(a, to_np(b)) <= 1e-3, what
 
