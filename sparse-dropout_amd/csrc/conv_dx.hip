@@ -8,8 +8,9 @@
 // F.unfold gather of flash_dropout/functional/im2col_conv2d.py:17-20), for stride 1 and dilation 1.
 //
 // A workgroup owns HB = 2 * (64 / Q) input rows of one image, all channels.  The output rows whose taps
-// reach them lie in at most four consecutive 64-position row blocks of dY; their dY tiles (all of the
-// reduction, K_out <= 128) stay in LDS for the whole kernel.  Then, for every 64-column block of the patch
+// reach them lie in at most four consecutive 64-position row blocks of dY; each of the eight waves keeps 32
+// rows of them (all of the reduction, K_out <= 128) in registers as MFMA operands for the whole kernel, so
+// that two workgroups fit a CU and one folds while the other multiplies.  Then, for every 64-column block of the patch
 // matrix in turn: the W tile of the block arrives by direct loads (double buffered), every wave multiplies
 // one 32-row half of one dY tile with it (MFMA, fp32) if the mask keeps that tile and writes the scaled
 // result, rounded once as the two-kernel route rounds it, to an LDS staging area; after a barrier each
@@ -28,10 +29,9 @@ constexpr int THREADS = 512;
 constexpr int NB = 4;           // row blocks of dY per workgroup
 constexpr int KS_MAX = 2;       // 64-wide reduction steps: K_out <= 128
 constexpr int STAGE_LD = 68;    // halfs per staged row: 64 + 4 so that the two half-waves of a store hit different banks
-constexpr int OFF_W = NB * KS_MAX * TILE;                 // 64 KB of dY tiles, then
-constexpr int OFF_STAGE = OFF_W + 2 * KS_MAX * TILE;      // two W tiles of 16 KB, then
+constexpr int OFF_STAGE = 2 * KS_MAX * TILE;              // two W tiles of 16 KB, then
 constexpr int OFF_ACC = OFF_STAGE + NB * BS * STAGE_LD * 2;  // the staging area, then the ring
-constexpr int DYN_LDS_MAX = 163840 - 256;  // the kernel also has a few bytes of static LDS
+constexpr int DYN_LDS_MAX = 81920 - 256;   // half a CU's LDS (two workgroups per CU); a few bytes are static
 constexpr int ACC_MAX = DYN_LDS_MAX - OFF_ACC;  // bytes left for the ring of open channel sums
 
 typedef __attribute__((address_space(3))) void lds_void;
@@ -72,8 +72,7 @@ struct DxArgs {
 template <typename T, int RT, int ST>
 __global__ __launch_bounds__(THREADS) void conv_dx_kernel(DxArgs g) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  char* dyt = smem;
-  char* wt = smem + OFF_W;
+  char* wt = smem;
   uint16_t* stage = reinterpret_cast<uint16_t*>(smem + OFF_STAGE);
   float* ring = reinterpret_cast<float*>(smem + OFF_ACC);
 
@@ -101,15 +100,24 @@ __global__ __launch_bounds__(THREADS) void conv_dx_kernel(DxArgs g) {
   }
   __syncthreads();
 
-  // ---- dY tiles, the first W tile, the ring -------------------------------------------------------------
+  // ---- this wave's 32 rows of dY as MFMA fragments (lane: row lane % 32, 8 reduction indices per 16), the
+  //      first W tile, the ring ----------------------------------------------------------------------------
+  const int t_blk = wave >> 1, half = wave & 1;  // this wave's dY row block and its 32-row half
   const int ld_row = wave * 8 + lane / 8, ld_pch = lane % 8;
+  u32x4 af[KS_MAX][4];
 #pragma unroll
-  for (int b = 0; b < NB; ++b) {
-    if (keep[b] == 0) continue;  // outside the image, or nothing kept
-    const int64_t m = ((int64_t)img * g.blocks_per_img + pb0 + b) * BS + ld_row;
-    for (int ks = 0; ks < g.KS; ++ks)
-      load16_to_lds(g.dy + m * g.dy_ld + ks * BS + (ld_pch ^ ((ld_row >> 1) & 7)) * 8,
-                    dyt + (b * KS_MAX + ks) * TILE + wave * 1024);
+  for (int ks = 0; ks < KS_MAX; ++ks)
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) af[ks][kk] = u32x4{0u, 0u, 0u, 0u};
+  if (keep[t_blk] != 0) {  // inside the image and something kept
+    const int64_t m = ((int64_t)img * g.blocks_per_img + pb0 + t_blk) * BS + half * 32 + lane % 32;
+    const uint16_t* src = g.dy + m * g.dy_ld + (lane / 32) * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS_MAX; ++ks)
+      if (ks < g.KS) {
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) af[ks][kk] = *reinterpret_cast<const u32x4*>(src + ks * BS + kk * 16);
+      }
   }
   // W tile of block column j, reduction step ks: rows = reduction index, 64 columns = 128 bytes each
   auto load_w = [&](int j, int buf) {
@@ -124,16 +132,13 @@ __global__ __launch_bounds__(THREADS) void conv_dx_kernel(DxArgs g) {
   for (int i = tid; i < g.ring_n * hw_n; i += THREADS) ring[i] = 0.f;
 
   // ---- per-lane fragment offsets (the tile layouts of the GEMM kernels) ----------------------------------
-  const int t_blk = wave >> 1, half = wave & 1;  // this wave's dY tile and its 32-row half
-  int a_off[4], b_off[4];
+  int b_off[4];
   {
-    const int fr_sw = (lane >> 1) & 7;
     const int b4 = lane / 16, e = (lane % 16) / 4, j4 = lane % 4;
     const int row = 8 * (b4 / 2) + e;
     const int b_ch = (2 * (b4 % 2) + j4 / 2) ^ (((e >> 1) & 1) << 2);
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
-      a_off[kk] = (half * 32 + lane % 32) * 128 + ((2 * kk + lane / 32) ^ fr_sw) * 16;
       b_off[kk] = (16 * kk + row) * 128 + b_ch * 16 + (j4 % 2) * 8;  // ^ 64 for the second 32 columns
     }
   }
@@ -177,17 +182,17 @@ __global__ __launch_bounds__(THREADS) void conv_dx_kernel(DxArgs g) {
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[nt][v] = 0.f;
-      for (int ks = 0; ks < g.KS; ++ks) {
-        const char* at = dyt + (t_blk * KS_MAX + ks) * TILE;
+#pragma unroll
+      for (int ks = 0; ks < KS_MAX; ++ks) {
+        if (ks >= g.KS) break;
         const char* bt = wt + ((j & 1) * KS_MAX + ks) * TILE;
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
-          const u32x4 af = *reinterpret_cast<const u32x4*>(at + a_off[kk]);
 #pragma unroll
           for (int nt = 0; nt < 2; ++nt) {
             const char* p = bt + (b_off[kk] ^ (nt * 64));
             const u32x2 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * 128);
-            acc[nt] = T::mfma32(af, u32x4{lo.x, lo.y, hi.x, hi.y}, acc[nt]);
+            acc[nt] = T::mfma32(af[ks][kk], u32x4{lo.x, lo.y, hi.x, hi.y}, acc[nt]);
           }
         }
       }
@@ -200,6 +205,8 @@ __global__ __launch_bounds__(THREADS) void conv_dx_kernel(DxArgs g) {
           st[row * STAGE_LD + nt * 32 + lane % 32] = T::from_float(acc[nt][v] * g.scale);
         }
     }
+    // the next W tile has had the products to arrive; so have the stores of the previous block's sums
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     // ---- the taps of this block column, summed into the owners' ring entries ----------------------------
     {
@@ -244,8 +251,7 @@ __global__ __launch_bounds__(THREADS) void conv_dx_kernel(DxArgs g) {
         }
       }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+    __syncthreads();  // the staging area and this block's W buffer are free again
   }
 }
 
