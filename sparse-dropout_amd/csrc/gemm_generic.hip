@@ -248,18 +248,48 @@ __global__ __launch_bounds__(THREADS) void gemm_generic_kernel(GemmArgs g, int t
   }
 }
 
-// C = scale * sum over splits of the fp32 partial tiles; one thread per element, lanes along C's
-// contiguous index (the workspace is laid out the same way).
+// C = scale * sum over splits of the fp32 partial tiles.  A workgroup owns 256 consecutive elements of C's
+// contiguous order (the workspace is laid out the same way): lane l of every wave takes elements 4l .. 4l+3 as
+// one 16-byte load per split, the four waves share out the splits and their partial sums meet in LDS.
 template <typename T>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs g, int splits, bool trans) {
+  __shared__ float part[3][256];
   const int64_t total = g.M * g.N;
-  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (e >= total) return;
-  float acc = 0.f;
-  for (int s = 0; s < splits; ++s) acc += g.ws[(int64_t)s * total + e];
-  const int64_t m = trans ? e % g.M : e / g.N;
-  const int64_t n = trans ? e / g.M : e % g.N;
-  g.c[m * g.c_sr + n * g.c_sc] = T::from_float(acc * g.scale);
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int64_t e0 = (int64_t)blockIdx.x * 256 + lane * 4;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  if (e0 + 3 < total && total % 4 == 0) {
+    const float* src = g.ws + e0;
+    int s = wave;
+#pragma unroll 4
+    for (; s < splits; s += 4) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(src + (int64_t)s * total);
+      acc[0] += v[0];
+      acc[1] += v[1];
+      acc[2] += v[2];
+      acc[3] += v[3];
+    }
+  } else {
+    for (int s = wave; s < splits; s += 4)
+#pragma unroll
+      for (int v = 0; v < 4; ++v)
+        if (e0 + v < total) acc[v] += g.ws[(int64_t)s * total + e0 + v];
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) part[wave - 1][lane * 4 + v] = acc[v];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    const int64_t e = e0 + v;
+    if (e >= total) break;
+    const float sum = ((acc[v] + part[0][lane * 4 + v]) + part[1][lane * 4 + v]) + part[2][lane * 4 + v];
+    const int64_t m = trans ? e % g.M : e / g.N;
+    const int64_t n = trans ? e / g.M : e % g.N;
+    g.c[m * g.c_sr + n * g.c_sc] = T::from_float(sum * g.scale);
+  }
 }
 
 template <typename T, int MODE>
