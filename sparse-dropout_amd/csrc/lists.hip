@@ -71,6 +71,15 @@ struct MaskSrc {
     // 24 random bits -> [0, 1) in steps of 2^-24, exact in fp32; True (dropped) with probability p
     return (float)(c[e & 3] >> 8) * 0x1p-24f < p;
   }
+  // One generator call yields the draws of four consecutive entries: bit v = entry 4 * grp + v is dropped.
+  __device__ inline uint32_t dropped4(uint64_t grp) const {
+    uint32_t c[4] = {(uint32_t)grp, (uint32_t)(grp >> 32), off_lo, off_hi};
+    Philox{seed_lo, seed_hi}(c);
+    uint32_t bits = 0;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) bits |= ((float)(c[v] >> 8) * 0x1p-24f < p ? 1u : 0u) << v;
+    return bits;
+  }
   __device__ inline bool dropped(int32_t i, int32_t j) const {
     return split == 1 ? dropped_entry(i, j) : dropped_entry(i / split, j / split);
   }
@@ -139,6 +148,13 @@ __device__ inline void block_scan_inplace(int32_t* ptr, int64_t n, int32_t* lds 
 __device__ inline void write_mask(const MaskSrc& src, int64_t mb, uint8_t* out, int64_t first,
                                   int64_t stride) {
   const int64_t total = mb * src.kb;
+  if (src.mask == nullptr) {  // drawn: four entries per generator call
+    for (int64_t grp = first; grp * 4 < total; grp += stride) {
+      const uint32_t bits = src.dropped4((uint64_t)grp);
+      for (int v = 0; v < 4 && grp * 4 + v < total; ++v) out[grp * 4 + v] = (bits >> v) & 1u;
+    }
+    return;
+  }
   for (int64_t e = first; e < total; e += stride)
     out[e] = src.dropped_entry((int32_t)(e / src.kb), (int32_t)(e % src.kb)) ? 1 : 0;
 }
@@ -212,10 +228,31 @@ __global__ __launch_bounds__(kFlatThreads) void build_lists_flat(ListJob job0, L
   const int f0 = b * kFlatChunk;
 
   // kept entries in front of this block's chunk
+  // a mask drawn at the listed granularity: entry index = row-major position, four entries share a generator call
+  const bool drawn4 = job.src.mask == nullptr && job.src.split == 1 && job.src.kb == (job.by_col ? (int)job.nlines : len);
   int cnt = 0;
-  for (int f = tid; f < f0; f += kFlatThreads) {
-    const int line = f / len;
-    cnt += job.kept(line, f - line * len) ? 1 : 0;
+  if (drawn4 && !job.by_col) {
+    for (int grp = tid; grp * 4 < f0; grp += kFlatThreads) cnt += __popc(~job.src.dropped4((uint64_t)grp) & 0xFu);
+  } else if (drawn4) {
+    // lines are columns: in front of (col0, row0) lies every entry of an earlier column and the rows above in col0
+    const int kb = job.src.kb;
+    const int col0 = f0 / len, row0 = f0 - col0 * len;
+    for (int grp = tid; grp * 4 < total_entries; grp += kFlatThreads) {
+      uint32_t kept = ~job.src.dropped4((uint64_t)grp) & 0xFu;
+      int row = (grp * 4) / kb, col = grp * 4 - row * kb;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const bool front = grp * 4 + v < total_entries && (col < col0 || (col == col0 && row < row0));
+        if (!front) kept &= ~(1u << v);
+        if (++col == kb) { col = 0; ++row; }
+      }
+      cnt += __popc(kept);
+    }
+  } else {
+    for (int f = tid; f < f0; f += kFlatThreads) {
+      const int line = f / len;
+      cnt += job.kept(line, f - line * len) ? 1 : 0;
+    }
   }
   int base;
   block_exclusive_scan(cnt, lds, base);
@@ -224,7 +261,12 @@ __global__ __launch_bounds__(kFlatThreads) void build_lists_flat(ListJob job0, L
   const int mine = f0 + tid * kFlatPer;
   int line = mine / len, e = mine - line * len;
   uint32_t bits = 0;
-  {
+  if (drawn4 && !job.by_col) {  // mine is a multiple of four: one generator call
+    if (mine < total_entries) {
+      bits = ~job.src.dropped4((uint64_t)(mine / 4)) & 0xFu;
+      if (mine + 4 > total_entries) bits &= (1u << (total_entries - mine)) - 1u;
+    }
+  } else {
     int l = line, x = e;
 #pragma unroll
     for (int v = 0; v < kFlatPer; ++v) {
