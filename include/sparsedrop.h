@@ -68,7 +68,8 @@ const char* sd_last_kernel(void);
 /* Workgroup shape of the specialised DSD / dense kernels: SD_TILE_AUTO picks from the shape (256 x 256
  * output tiles when there are more than 128 of them, 128 x 128 otherwise; the SDD kernel's group shape follows the
  * same rule), the other two
- * force one shape for every later call of the process.  Returns the previous setting, -1 for an unknown
+ * force one shape for every later call of the process (SD_TILE_BIG also makes sd_conv2d_dsd_lists keep one
+ * LDS copy of all channels' input rows instead of a copy per step where both fit).  Returns the previous setting, -1 for an unknown
  * value.  A tuning and test hook; results do not depend on it beyond fp32 summation order.  No
  * counterpart in the reference (its tile is a compile-time GemmConfig, gemm_configs/gemm_config.cuh:19-100). */
 #define SD_TILE_AUTO 0

@@ -152,12 +152,15 @@ __device__ inline u32x2 lds_read_tr(const char* p) {
 // the patch matrix from that copy, in the layout the fragment reads expect, instead of loading them.  A
 // table in LDS maps a patch-matrix column (c, r, s) to its offset in the copy; whether
 // a tap falls outside the image never has to be asked: the copy carries a halo of zeros.
-template <typename T, bool TRANS, bool CM, bool RAGGED, typename S, bool IMPLICIT = false>
+// IMPLICIT = 2: the same with a copy per step that holds only the channels of the step's 64 columns (any number
+// of input channels fits); the reduction-strided instance (the weight gradient) always works that way.
+template <typename T, bool TRANS, bool CM, bool RAGGED, typename S, int IMPLICIT = 0>
 __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m, int tiles_n,
                                                          int Mb, int Kb_all, ImplicitConv cg) {
   static_assert(!IMPLICIT || (S::R == 4 && S::THREADS == 512), "the gather assumes 512 threads x 4 row blocks");
   constexpr int R = S::R, BN = S::BN, THREADS = S::THREADS, NT = S::NT, STAGE = S::STAGE, A_OFF = S::A_OFF;
   constexpr int BL = S::BL, AL = S::AL, RW = S::RW;
+  constexpr bool STEP_COPIES = IMPLICIT != 0 && (TRANS || IMPLICIT == 2);  // input rows copied per step
   extern __shared__ __attribute__((aligned(16))) char smem[];
   uint32_t* step_e = reinterpret_cast<uint32_t*>(smem + S::SMEM_STEPS);
   uint32_t* scratch = reinterpret_cast<uint32_t*>(smem + S::SMEM_SCRATCH);
@@ -225,7 +228,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   uint32_t gat_base[4];  // byte offset of (this thread's tile row, tap 0) in the patch, per row block
   const int gat_row = tid / 8, gat_pc = tid % 8;  // the tile row and physical 16-byte chunk this thread builds
   [[maybe_unused]] auto div = [](int x, uint32_t magic) { return magic ? (int)__umulhi((uint32_t)x, magic) : x; };
-  if constexpr (IMPLICIT && !TRANS) {
+  if constexpr (IMPLICIT == 1 && !TRANS) {
     const int img = rb0 / cg.blocks_per_img;
     const int p0 = (rb0 - img * cg.blocks_per_img) * cg.rpb;  // first output row of the workgroup
     const int h0 = p0 - cg.pad_h;                              // input row of patch row 0
@@ -270,12 +273,51 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   // alternate: the one for step s+2 is fetched into registers at the top of step s and written to LDS at
   // its end, the tiles of step s+1 are built from the other while step s computes.  The tile a row block
   // keeps is [64 positions][its 64 columns], rows of 128 bytes, in the swizzle of the transposing reads.
-  constexpr int TSEG = IMPLICIT && TRANS ? (CONV_T_PATCH_MAX / 16 + THREADS - 1) / THREADS : 1;
+  // The forward's per-step form (IMPLICIT == 2) does the same with the 256 positions of the workgroup fixed and
+  // the channels moving: a step's copy holds the <= 64 / (R*S) + 2 channels its 64 columns touch.
+  constexpr int TSEG = STEP_COPIES ? (CONV_T_PATCH_MAX / 16 + THREADS - 1) / THREADS : 1;
   [[maybe_unused]] u32x4 tp_v[TSEG];      // a step's input rows on their way to LDS
   [[maybe_unused]] int tp_dst[TSEG];      // where this thread's segments go in a copy (halfs), -1 = none
   [[maybe_unused]] int64_t tp_src[TSEG];  // and where they come from, relative to (image, input row h0)
   [[maybe_unused]] int tp_row[TSEG];      // their row in the copy
+  [[maybe_unused]] int tp_c[TSEG];        // forward: their channel, counted from the step's first
+  [[maybe_unused]] const uint16_t* fwd_x0 = nullptr;  // forward: (image, first input row) of the workgroup
+  [[maybe_unused]] int fwd_h0 = 0;
   [[maybe_unused]] uint16_t* patch1 = nullptr;
+  [[maybe_unused]] const uint16_t* tcopy = patch;  // the copy the next step's tiles are built from
+  if constexpr (IMPLICIT == 2 && !TRANS) {
+    const int img = rb0 / cg.blocks_per_img;
+    fwd_h0 = (rb0 - img * cg.blocks_per_img) * cg.rpb - cg.pad_h;
+    fwd_x0 = cg.x + (int64_t)img * cg.sn + (int64_t)fwd_h0 * cg.sh;
+    const int nch = (BS + cg.RS - 2) / cg.RS + 1;  // channels 64 consecutive columns can touch
+    const int spr = cg.W / 8, spc = cg.PR * spr;
+    const int total = nch * spc, rows = nch * cg.PR;
+    patch1 = patch + cg.patch_stride;
+    ktab = patch1 + cg.patch_stride;
+#pragma unroll
+    for (int j = 0; j < TSEG; ++j) {
+      const int seg = tid + j * THREADS;
+      const int c = div(seg, cg.m_spc), rem = seg - c * spc;
+      const int row = div(rem, cg.m_spr), w8 = rem - row * spr;
+      tp_dst[j] = seg < total ? (c * cg.PR + row) * cg.PW + 8 + w8 * 8 : -1;
+      tp_src[j] = (int64_t)c * cg.sc + (int64_t)row * cg.sh + w8 * 8;
+      tp_row[j] = row;
+      tp_c[j] = c;
+    }
+    for (int m = tid; m <= rows; m += THREADS) {  // the halo groups of both copies; the steps never write them
+      *reinterpret_cast<u32x4*>(patch + m * cg.PW) = u32x4{0u, 0u, 0u, 0u};
+      *reinterpret_cast<u32x4*>(patch1 + m * cg.PW) = u32x4{0u, 0u, 0u, 0u};
+    }
+    for (int k = tid; k < Kb_all * BS; k += THREADS) {
+      const int c = div(k, cg.m_RS), tap = k - c * cg.RS;
+      const int rr = div(tap, cg.m_S), ss = tap - rr * cg.S;
+      const int c_lo = div(k & ~(BS - 1), cg.m_RS);  // first channel of the column's block = of its step's copy
+      ktab[k] = k < cg.K ? (uint16_t)((((c - c_lo) * cg.PR + rr) * cg.PW + ss) * 2) : (uint16_t)0;
+    }
+    const int prow = div(gat_row, cg.m_Q), q = gat_row - prow * cg.Q;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) gat_base[r] = (uint32_t)(((r * cg.rpb + prow) * cg.PW + 8 + q - cg.pad_w) * 2);
+  }
   if constexpr (IMPLICIT && TRANS) {
     const int k_lo = rb0 * BS;
     const int k_hi = k_lo + R * BS < cg.K ? k_lo + R * BS : cg.K;
@@ -309,6 +351,18 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   }
   // fetches the input rows of the step with table word `entry` (its reduction block is a block of 64 positions)
   [[maybe_unused]] auto tpatch_load = [&](uint32_t entry) {
+    if constexpr (!TRANS) {  // forward: the step's reduction block is a block of 64 columns, i.e. a run of channels
+      const int c_lo = div(step_block(entry) * BS, cg.m_RS);
+      const uint16_t* src = fwd_x0 + (int64_t)c_lo * cg.sc;
+#pragma unroll
+      for (int j = 0; j < TSEG; ++j) {
+        const int h = fwd_h0 + tp_row[j];
+        tp_v[j] = u32x4{0u, 0u, 0u, 0u};
+        if (tp_dst[j] >= 0 && h >= 0 && h < cg.H && c_lo + tp_c[j] < cg.C)
+          tp_v[j] = *reinterpret_cast<const u32x4*>(src + tp_src[j]);
+      }
+      return;
+    }
     const int mb = step_block(entry);
     const int img = mb / cg.blocks_per_img;
     const int h0 = (mb - img * cg.blocks_per_img) * cg.rpb - cg.pad_h;
@@ -340,7 +394,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   auto gather_tile = [&](int r, int kb, char* tile) {
     const int lc = gat_pc ^ ((gat_row >> 1) & 7);  // logical chunk: columns kb*64 + lc*8 .. +7
     const u16x8 off = *reinterpret_cast<const u16x8*>(ktab + kb * BS + lc * 8);
-    const char* pb = reinterpret_cast<const char*>(patch) + gat_base[r];
+    const char* pb = reinterpret_cast<const char*>(IMPLICIT == 2 ? tcopy : patch) + gat_base[r];
     uint32_t v[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] = *reinterpret_cast<const uint16_t*>(pb + off[e]);
@@ -460,7 +514,6 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   }
   const int64_t b_red_stride = TRANS ? (int64_t)BS * g.b.sc * 2 : (int64_t)BS * 2;
 
-  [[maybe_unused]] const uint16_t* tcopy = patch;  // implicit weight gradient: the copy the next tiles are built from
   auto issue_loads = [&](uint32_t entry, int stage) {  // entry: wave-uniform step table word
     const int kb = step_block(entry);
     const uint32_t fl = step_flags(entry);
@@ -587,7 +640,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   // long returned: a read-and-wait at the top of a step would put an LDS round trip in front of its MFMAs.
   const bool late = __builtin_amdgcn_readfirstlane(rh) != 0;
   uint32_t e_cur = uniform(step_e[0]), e_next = uniform(step_e[1]);
-  if constexpr (IMPLICIT && TRANS) {
+  if constexpr (STEP_COPIES) {
     if (nsteps > 0) {
       tpatch_load(e_cur);
       tpatch_store(patch);
@@ -606,7 +659,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
     const int stage = step & 1;
     const uint32_t e_after = step_e[step + 2];
     const bool more = step + 1 < nsteps;
-    if constexpr (IMPLICIT && TRANS) {
+    if constexpr (STEP_COPIES) {
       if (step + 2 < nsteps) tpatch_load(uniform(step_e[step + 2]));
       tcopy = ((step + 1) & 1) ? patch1 : patch;  // holds the rows of step + 1
     }
@@ -622,7 +675,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
     } else {
       if (mine) compute(std::integral_constant<int, 1>{}, st, mid, e_next, stage ^ 1, red_tail);
     }
-    if constexpr (IMPLICIT && TRANS) {
+    if constexpr (STEP_COPIES) {
       if (step + 2 < nsteps) tpatch_store((step & 1) ? patch1 : patch);  // last read for this step's tiles, a step ago
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -1111,10 +1164,10 @@ int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
   return edge ? launch_sdd_group<F16, true>(g, stream) : launch_sdd_group<F16, false>(g, stream);
 }
 
-template <typename T, bool RAGGED>
+template <typename T, bool RAGGED, int FORM>
 int launch_conv_t(const GemmArgs& g, const ImplicitConv& cg, int smem, hipStream_t stream) {
   static bool configured[kMaxDevices] = {};
-  auto* kernel = &dsd_kernel<T, false, false, RAGGED, DsdConv, true>;
+  auto* kernel = &dsd_kernel<T, false, false, RAGGED, DsdConv, FORM>;
   if (int rc = allow_big_lds(reinterpret_cast<const void*>(kernel), 163840, configured)) return rc;
   const int Mb = (int)(g.M / BS), Kb = (int)((g.K + BS - 1) / BS);
   const int tiles_m = Mb / DsdConv::R, tiles_n = (int)((g.N + DsdConv::BN - 1) / DsdConv::BN);
@@ -1126,7 +1179,7 @@ int launch_conv_t(const GemmArgs& g, const ImplicitConv& cg, int smem, hipStream
 template <typename T, bool RAGGED>
 int launch_conv_dw_t(const GemmArgs& g, const ImplicitConv& cg, int smem, int splits, hipStream_t stream) {
   static bool configured[kMaxDevices] = {};
-  auto* kernel = &dsd_kernel<T, true, true, RAGGED, DsdConv, true>;
+  auto* kernel = &dsd_kernel<T, true, true, RAGGED, DsdConv, 1>;
   if (int rc = allow_big_lds(reinterpret_cast<const void*>(kernel), 163840, configured)) return rc;
   const int Mb = (int)((g.M + BS - 1) / BS), Kb = (int)(g.K / BS);
   const int tiles_m = (Mb + DsdConv::R - 1) / DsdConv::R, tiles_n = (int)((g.N + DsdConv::BN - 1) / DsdConv::BN);
@@ -1188,19 +1241,38 @@ int launch_conv_implicit(const GemmArgs& g, const ImplicitConv& cg, int64_t P, i
                        cg.pad_h >= 0 && cg.pad_w >= 0 && cg.pad_w <= 8 && cg.S - 1 - cg.pad_w <= 8 && R * cg.S == cg.RS &&
                        cg.PW == cg.W + 8;
   if (!geom_ok) return SD_ERR_UNSUPPORTED;
-  const int64_t patch_elems = (int64_t)cg.C * cg.PR * cg.PW + 8;  // rows with their halo groups, one more after the last
   const int64_t Kb = (g.K + BS - 1) / BS;
-  const int64_t extra = patch_elems * 2 + Kb * BS * 2;
-  if (extra > CONV_PATCH_MAX || Kb > MAX_STEPS) return SD_ERR_UNSUPPORTED;
+  if (Kb > MAX_STEPS) return SD_ERR_UNSUPPORTED;
   const bool align_ok = aligned16(cg.x) && cg.sn % 8 == 0 && cg.sc % 8 == 0 && cg.sh % 8 == 0 && aligned16(g.b.ptr) &&
                         g.b.sc == 1 && g.b.sr % 8 == 0 && g.b.sr < (1 << 22) && g.c_sc == 1 && g.K % 8 == 0 &&
                         g.M % (BS * DsdConv::R) == 0 && g.M / (BS * DsdConv::R) * ((g.N + 127) / 128) < 0x7fffffffLL;
   if (!align_ok) return SD_ERR_UNSUPPORTED;
-  const int smem = ((DsdConv::SMEM_BYTES + 15) & ~15) + (int)extra;
+  // two alternating copies of the channels one step's 64 columns touch (any number of channels; measured at least
+  // as fast as the other form wherever both fit) ...
+  const int64_t nch = (BS + cg.RS - 2) / cg.RS + 1;
+  const int64_t copy_elems = (nch * cg.PR * cg.PW + 8 + 7) & ~7LL;
+  const int64_t stepwise = 2 * copy_elems * 2 + Kb * BS * 2;
+  const bool step_ok = copy_elems * 2 <= CONV_T_PATCH_MAX && stepwise <= CONV_PATCH_MAX;
+  // ... or one copy of every channel's rows for the whole kernel if that fits next to the stages (many taps per
+  // 64 columns, e.g. 1 x 1 kernels, make a step's copy large; the large-tile policy prefers this form)
+  const int64_t patch_elems = (int64_t)cg.C * cg.PR * cg.PW + 8;  // rows with their halo groups, one more after the last
+  const int64_t whole = patch_elems * 2 + Kb * BS * 2;
+  const bool whole_ok = whole <= CONV_PATCH_MAX;
+  if (!step_ok && !whole_ok) return SD_ERR_UNSUPPORTED;
+  const bool use_steps = step_ok && !(whole_ok && tile_policy.load(std::memory_order_relaxed) == kTileBig);
   const bool ragged = g.N % BS != 0 || g.K % BS != 0;
+  if (use_steps) {
+    ImplicitConv cs = cg;
+    cs.patch_stride = (int)copy_elems;
+    const int smem = ((DsdConv::SMEM_BYTES + 15) & ~15) + (int)stepwise;
+    if (dtype == SD_BF16)
+      return ragged ? launch_conv_t<BF16, true, 2>(g, cs, smem, stream) : launch_conv_t<BF16, false, 2>(g, cs, smem, stream);
+    return ragged ? launch_conv_t<F16, true, 2>(g, cs, smem, stream) : launch_conv_t<F16, false, 2>(g, cs, smem, stream);
+  }
+  const int smem = ((DsdConv::SMEM_BYTES + 15) & ~15) + (int)whole;
   if (dtype == SD_BF16)
-    return ragged ? launch_conv_t<BF16, true>(g, cg, smem, stream) : launch_conv_t<BF16, false>(g, cg, smem, stream);
-  return ragged ? launch_conv_t<F16, true>(g, cg, smem, stream) : launch_conv_t<F16, false>(g, cg, smem, stream);
+    return ragged ? launch_conv_t<BF16, true, 1>(g, cg, smem, stream) : launch_conv_t<BF16, false, 1>(g, cg, smem, stream);
+  return ragged ? launch_conv_t<F16, true, 1>(g, cg, smem, stream) : launch_conv_t<F16, false, 1>(g, cg, smem, stream);
 }
 
 int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {

@@ -132,14 +132,27 @@ IMPLICIT_GEOMS = [
     (dict(n=2, c=16, h=16, w=16, k=64, r=3, s=3, padding=(2, 2), stride=(1, 1), dilation=(1, 1)), False),   # Q = 18
     (dict(n=2, c=8, h=32, w=32, k=64, r=3, s=3, padding=(1, 1), stride=(2, 2), dilation=(1, 1)), False),    # stride
     (dict(n=1, c=16, h=8, w=16, k=64, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), False),    # P*Q = 128
-    (dict(n=1, c=256, h=32, w=32, k=64, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), False),  # input rows do not fit in LDS
+    (dict(n=1, c=256, h=32, w=32, k=64, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),   # too many channels for one copy of the input rows: a copy per step
+    (dict(n=2, c=136, h=16, w=16, k=192, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),  # the same with 1224 columns (ragged), two column tiles
 ]
+
+
+@pytest.fixture(params=["auto", "big"])
+def copy_form(request):
+    """The implicit forward keeps a copy of the input rows per step, or one copy of all channels' rows for the
+    whole kernel where only that fits; the large-tile policy prefers the latter, so both run where both fit."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    prev = ext.set_tile_policy(request.param)
+    yield request.param
+    ext.set_tile_policy(prev)
 
 
 @pytest.mark.parametrize("cfg,taken", IMPLICIT_GEOMS)
 @pytest.mark.parametrize("p", [0.0, 0.5])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_implicit_gemm_conv_forward(cfg, taken, p, dtype):
+def test_implicit_gemm_conv_forward(cfg, taken, p, dtype, copy_form):
     """sd_conv2d_dsd_lists (no patch matrix) against the oracle and against im2col + DSD on the same lists;
     geometries it does not take must come back as None with nothing written."""
     from flash_dropout.hip import GEMM
@@ -169,8 +182,8 @@ def test_implicit_gemm_conv_forward(cfg, taken, p, dtype):
     assert rel_fro(y, ry2) <= REL_FRO_TOL
 
 
-@pytest.mark.parametrize("cfg,taken", [g for g in IMPLICIT_GEOMS if g[1]][:5])
-def test_implicit_gemm_conv_dense(cfg, taken):
+@pytest.mark.parametrize("cfg,taken", [g for g in IMPLICIT_GEOMS if g[1]][:5] + IMPLICIT_GEOMS[-2:])
+def test_implicit_gemm_conv_dense(cfg, taken, copy_form):
     """No lists = every block kept: the dense convolution, against torch's conv2d in fp32."""
     from flash_dropout.hip import GEMM
 
