@@ -9,8 +9,8 @@
 //
 // A workgroup owns HB = 2 * (64 / Q) input rows of one image, all channels.  The output rows whose taps
 // reach them lie in at most four consecutive 64-position row blocks of dY; each of the eight waves keeps 32
-// rows of them (all of the reduction, K_out <= 128) in registers as MFMA operands for the whole kernel, so
-// that two workgroups fit a CU and one folds while the other multiplies.  Then, for every 64-column block of the patch
+// rows of them (all of the reduction, K_out <= 256) in registers as MFMA operands for the whole kernel, so
+// that (for K_out <= 128) two workgroups fit a CU and one folds while the other multiplies.  Then, for every 64-column block of the patch
 // matrix in turn: the W tile of the block arrives by direct loads (double buffered), every wave multiplies
 // one 32-row half of one dY tile with it (MFMA, fp32) if the mask keeps that tile and writes the scaled
 // result, rounded once as the two-kernel route rounds it, to an LDS staging area; after a barrier each
@@ -27,12 +27,17 @@ constexpr int BS = 64;
 constexpr int TILE = BS * BS * 2;
 constexpr int THREADS = 512;
 constexpr int NB = 4;           // row blocks of dY per workgroup
-constexpr int KS_MAX = 2;       // 64-wide reduction steps: K_out <= 128
+constexpr int KS_LIMIT = 4;     // 64-wide reduction steps at most: K_out <= 256
 constexpr int STAGE_LD = 68;    // halfs per staged row: 64 + 4 so that the two half-waves of a store hit different banks
-constexpr int OFF_STAGE = 2 * KS_MAX * TILE;              // two W tiles of 16 KB, then
-constexpr int OFF_ACC = OFF_STAGE + NB * BS * STAGE_LD * 2;  // the staging area, then the ring
-constexpr int DYN_LDS_MAX = 81920 - 256;   // half a CU's LDS (two workgroups per CU); a few bytes are static
-constexpr int ACC_MAX = DYN_LDS_MAX - OFF_ACC;  // bytes left for the ring of open channel sums
+// LDS of an instance for K_out <= 64 * KS_MAX: two W tiles (one per buffer) of KS_MAX * 8 KB, the staging area, the ring
+template <int KS_MAX>
+struct DxLds {
+  static constexpr int OFF_STAGE = 2 * KS_MAX * TILE;
+  static constexpr int OFF_ACC = OFF_STAGE + NB * BS * STAGE_LD * 2;
+  // K_out <= 128: half a CU's LDS, so that two workgroups share a CU; beyond, all of it (a few bytes are static)
+  static constexpr int DYN_LDS_MAX = (KS_MAX <= 2 ? 81920 : 163840) - 256;
+  static constexpr int ACC_MAX = DYN_LDS_MAX - OFF_ACC;  // bytes left for the ring of open channel sums
+};
 
 typedef __attribute__((address_space(3))) void lds_void;
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -69,8 +74,9 @@ struct DxArgs {
 
 // RT, ST: the kernel size at compile time (the tap loops unroll and the per-tap address terms become per-thread
 // constants), or 0, 0 for any size.
-template <typename T, int RT, int ST>
+template <typename T, int RT, int ST, int KS_MAX>
 __global__ __launch_bounds__(THREADS) void conv_dx_kernel(DxArgs g) {
+  constexpr int OFF_STAGE = DxLds<KS_MAX>::OFF_STAGE, OFF_ACC = DxLds<KS_MAX>::OFF_ACC;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   char* wt = smem;
   uint16_t* stage = reinterpret_cast<uint16_t*>(smem + OFF_STAGE);
@@ -255,19 +261,21 @@ __global__ __launch_bounds__(THREADS) void conv_dx_kernel(DxArgs g) {
   }
 }
 
-template <typename T, int RT, int ST>
-int launch_t(const DxArgs& g, int64_t wgs, int smem, hipStream_t stream) {
+template <typename T, int RT, int ST, int KS_MAX>
+int launch_t(const DxArgs& g, int64_t wgs, hipStream_t stream) {
+  const int smem = DxLds<KS_MAX>::OFF_ACC + g.ring_n * g.HB * g.W * 4;
+  if (smem > DxLds<KS_MAX>::DYN_LDS_MAX) return SD_ERR_UNSUPPORTED;  // the ring of open channel sums does not fit
   static bool configured[16] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16)
     return fail(SD_ERR_RUNTIME, "hipGetDevice failed or device index out of range");
   if (!configured[dev]) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_dx_kernel<T, RT, ST>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, DYN_LDS_MAX);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_dx_kernel<T, RT, ST, KS_MAX>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, DxLds<KS_MAX>::DYN_LDS_MAX);
     if (e != hipSuccess) return fail(SD_ERR_RUNTIME, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     configured[dev] = true;
   }
-  hipLaunchKernelGGL((conv_dx_kernel<T, RT, ST>), dim3((unsigned)wgs), dim3(THREADS), smem, stream, g);
+  hipLaunchKernelGGL((conv_dx_kernel<T, RT, ST, KS_MAX>), dim3((unsigned)wgs), dim3(THREADS), smem, stream, g);
   return check_launch("conv_dx_kernel");
 }
 
@@ -282,7 +290,7 @@ int launch_conv_dx(const void* dy, int64_t dy_ld, const void* w, int64_t w_ld, v
   if (stride_h != 1 || stride_w != 1 || dil_h != 1 || dil_w != 1) return SD_ERR_UNSUPPORTED;
   const int64_t P = h + 2 * pad_h - r + 1, Q = wd + 2 * pad_w - s + 1;
   if (P <= 0 || Q <= 0 || Q > BS || BS % Q != 0 || (P * Q) % BS != 0) return SD_ERR_UNSUPPORTED;
-  if (k_out % BS != 0 || k_out > BS * KS_MAX) return SD_ERR_UNSUPPORTED;
+  if (k_out % BS != 0 || k_out > BS * KS_LIMIT) return SD_ERR_UNSUPPORTED;
   const int64_t K = c * r * s, Kb = (K + BS - 1) / BS;
   if (Kb > 64 || K % 8 != 0 || r * s > BS) return SD_ERR_UNSUPPORTED;  // keep flags are one 64-bit word per row block
   const int64_t rpb = BS / Q, HB = 2 * rpb;
@@ -292,7 +300,7 @@ int launch_conv_dx(const void* dy, int64_t dy_ld, const void* w, int64_t w_ld, v
   const int64_t hw_n = HB * wd;
   // a channel's columns span at most two blocks; the ring holds every channel a block column can touch
   const int64_t ring_n = (BS + r * s - 1) / (r * s) + 2;
-  if (hw_n > THREADS || ring_n * hw_n * 4 > ACC_MAX) return SD_ERR_UNSUPPORTED;
+  if (hw_n > THREADS) return SD_ERR_UNSUPPORTED;
   const bool align_ok = reinterpret_cast<uintptr_t>(dy) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
                         dy_ld % 8 == 0 && w_ld % 8 == 0 && dy_ld >= k_out && w_ld >= K;
   if (!align_ok) return SD_ERR_UNSUPPORTED;
@@ -331,10 +339,13 @@ int launch_conv_dx(const void* dy, int64_t dy_ld, const void* w, int64_t w_ld, v
   g.KS = (int)(k_out / BS);
   g.scale = scale;
   g.ring_n = (int)ring_n;
-  const int smem = OFF_ACC + (int)(ring_n * hw_n * 4);
-  if (r == 3 && s == 3)
-    return dtype == SD_BF16 ? launch_t<BF16, 3, 3>(g, wgs, smem, stream) : launch_t<F16, 3, 3>(g, wgs, smem, stream);
-  return dtype == SD_BF16 ? launch_t<BF16, 0, 0>(g, wgs, smem, stream) : launch_t<F16, 0, 0>(g, wgs, smem, stream);
+  const bool bf = dtype == SD_BF16, wide = k_out > 2 * BS;
+  if (r == 3 && s == 3) {
+    if (wide) return bf ? launch_t<BF16, 3, 3, 4>(g, wgs, stream) : launch_t<F16, 3, 3, 4>(g, wgs, stream);
+    return bf ? launch_t<BF16, 3, 3, 2>(g, wgs, stream) : launch_t<F16, 3, 3, 2>(g, wgs, stream);
+  }
+  if (wide) return bf ? launch_t<BF16, 0, 0, 4>(g, wgs, stream) : launch_t<F16, 0, 0, 4>(g, wgs, stream);
+  return bf ? launch_t<BF16, 0, 0, 2>(g, wgs, stream) : launch_t<F16, 0, 0, 2>(g, wgs, stream);
 }
 
 }  // namespace sd

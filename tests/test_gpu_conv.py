@@ -242,6 +242,10 @@ DX_GEOMS = [
     (dict(n=3, c=24, h=32, w=8, k=128, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),    # 8 output rows per block
     (dict(n=2, c=16, h=34, w=32, k=64, r=3, s=1, padding=(0, 0), stride=(1, 1), dilation=(1, 1)), True),    # no padding, H not a multiple of the band
     (dict(n=2, c=8, h=16, w=16, k=64, r=5, s=5, padding=(2, 2), stride=(1, 1), dilation=(1, 1)), True),     # 25 taps, 4 output rows per block
+    (dict(n=2, c=128, h=16, w=16, k=256, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),  # K_out = 256: the instance with the longer reduction
+    (dict(n=2, c=24, h=16, w=16, k=192, r=5, s=3, padding=(2, 1), stride=(1, 1), dilation=(1, 1)), True),   # K_out = 192, 15 taps
+    (dict(n=2, c=16, h=32, w=32, k=256, r=1, s=1, padding=(0, 0), stride=(1, 1), dilation=(1, 1)), True),   # 1x1 with K_out = 256: that instance's LDS holds the 66-slot ring
+    (dict(n=1, c=16, h=32, w=32, k=320, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), False),  # K_out = 320
     (dict(n=2, c=40, h=32, w=32, k=128, r=2, s=2, padding=(0, 0), stride=(1, 1), dilation=(1, 1)), False),  # Q = 31
     (dict(n=3, c=8, h=32, w=32, k=64, r=5, s=5, padding=(2, 2), stride=(1, 1), dilation=(1, 1)), False),    # 5 taps high on 2-row blocks
     (dict(n=2, c=16, h=16, w=16, k=40, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), False),   # K_out = 40
