@@ -131,6 +131,7 @@ static ImplicitConv conv_geometry(const void* x, int64_t sn, int64_t sc, int64_t
   cg.PR = (int)(blocks * (64 / Q) + r - 1);
   cg.PW = (int)(w + 8);
   cg.patch_stride = 0;
+  cg.units = 1;
   cg.K = (int)(c * r * s);
   auto magic = [](int64_t d) { return d <= 1 ? 0u : (uint32_t)(((1ull << 32) + (uint64_t)d - 1) / (uint64_t)d); };
   cg.m_spc = magic(cg.PR * (w / 8));
@@ -374,7 +375,11 @@ int sd_conv2d_dsd_lists(const void* x, int64_t sn, int64_t sc, int64_t sh, int64
   SD_REQUIRE(wld >= c * r * s && yld >= k_out, "leading dimensions too small");
   if (bs != 64 || Q > 64 || 64 % Q != 0 || c * r * s > (1 << 16) || h > (1 << 20) || w > (1 << 12) || r > 64 || s > 64)
     return SD_ERR_UNSUPPORTED;
-  ImplicitConv cg = conv_geometry(x, sn, sc, sh, c, h, w, P, Q, r, s, pad_h, pad_w, /*blocks=*/4);
+  // a workgroup's 256 output positions: 4 * 64 / Q consecutive rows of one image where P * Q allows, else four
+  // separate 64-position blocks
+  const bool one_run = (P * Q) % 256 == 0;
+  ImplicitConv cg = conv_geometry(x, sn, sc, sh, c, h, w, P, Q, r, s, pad_h, pad_w, /*blocks=*/one_run ? 4 : 1);
+  cg.units = one_run ? 1 : 4;
   GemmArgs g = make_args(nullptr, 0, 0, weight, wld, 1, y, yld, 1, n * P * Q, k_out, c * r * s, bs, scale, row_ptr,
                          col_idx);
   const int rc = launch_conv_implicit(g, cg, P, stride_h, stride_w, dil_h, dil_w, r, sw, dtype, (hipStream_t)stream);

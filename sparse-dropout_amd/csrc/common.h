@@ -119,7 +119,8 @@ struct ImplicitConv {
   int pad_h, pad_w;
   int rpb;             // output rows per 64-row block (64 / Q)
   int blocks_per_img;  // P * Q / 64
-  int PR;              // input rows a workgroup's 4 row blocks touch: 4 * rpb + R - 1
+  int PR;              // input rows a workgroup's 4 row blocks touch: 4 * rpb + R - 1 (units == 4: one block, rpb + R - 1)
+  int units;           // forward: 1 = the 4 row blocks share one run of input rows, 4 = each has its own (P*Q % 256 != 0)
   int PW;              // halfs per row of the LDS copy: 8 zeros, then the W of the image
   int patch_stride;    // weight gradient: halfs between the two alternating copies (set by the launcher)
   int K;               // C * R * S

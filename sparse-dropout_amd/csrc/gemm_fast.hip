@@ -279,29 +279,32 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   [[maybe_unused]] u32x4 tp_v[TSEG];      // a step's input rows on their way to LDS
   [[maybe_unused]] int tp_dst[TSEG];      // where this thread's segments go in a copy (halfs), -1 = none
   [[maybe_unused]] int64_t tp_src[TSEG];  // and where they come from, relative to (image, input row h0)
-  [[maybe_unused]] int tp_row[TSEG];      // their row in the copy
+  [[maybe_unused]] int tp_row[TSEG];      // their row in the copy (forward: their input row in the image)
   [[maybe_unused]] int tp_c[TSEG];        // forward: their channel, counted from the step's first
-  [[maybe_unused]] const uint16_t* fwd_x0 = nullptr;  // forward: (image, first input row) of the workgroup
-  [[maybe_unused]] int fwd_h0 = 0;
   [[maybe_unused]] uint16_t* patch1 = nullptr;
   [[maybe_unused]] const uint16_t* tcopy = patch;  // the copy the next step's tiles are built from
   if constexpr (IMPLICIT == 2 && !TRANS) {
-    const int img = rb0 / cg.blocks_per_img;
-    fwd_h0 = (rb0 - img * cg.blocks_per_img) * cg.rpb - cg.pad_h;
-    fwd_x0 = cg.x + (int64_t)img * cg.sn + (int64_t)fwd_h0 * cg.sh;
+    // cg.units == 1: the four row blocks are 4 * rpb consecutive output rows of one image and share one run of
+    // PR = 4 * rpb + R - 1 input rows per channel; cg.units == 4 (P * Q not a multiple of 256, e.g. 8 x 8 images):
+    // every row block has its own PR = rpb + R - 1 rows per channel, possibly from another image.
     const int nch = (BS + cg.RS - 2) / cg.RS + 1;  // channels 64 consecutive columns can touch
     const int spr = cg.W / 8, spc = cg.PR * spr;
-    const int total = nch * spc, rows = nch * cg.PR;
+    const int per_unit = nch * spc, total = cg.units * per_unit, rows = cg.units * nch * cg.PR;
     patch1 = patch + cg.patch_stride;
     ktab = patch1 + cg.patch_stride;
 #pragma unroll
     for (int j = 0; j < TSEG; ++j) {
       const int seg = tid + j * THREADS;
-      const int c = div(seg, cg.m_spc), rem = seg - c * spc;
+      const int u = (seg >= per_unit ? 1 : 0) + (seg >= 2 * per_unit ? 1 : 0) + (seg >= 3 * per_unit ? 1 : 0);
+      const int su = seg - u * per_unit;
+      const int c = div(su, cg.m_spc), rem = su - c * spc;
       const int row = div(rem, cg.m_spr), w8 = rem - row * spr;
-      tp_dst[j] = seg < total ? (c * cg.PR + row) * cg.PW + 8 + w8 * 8 : -1;
-      tp_src[j] = (int64_t)c * cg.sc + (int64_t)row * cg.sh + w8 * 8;
-      tp_row[j] = row;
+      const int rb = rb0 + u;
+      const int img = rb / cg.blocks_per_img;
+      const int h = (rb - img * cg.blocks_per_img) * cg.rpb - cg.pad_h + row;  // input row of the segment
+      tp_dst[j] = (seg < total && rb < Mb) ? ((u * nch + c) * cg.PR + row) * cg.PW + 8 + w8 * 8 : -1;
+      tp_src[j] = (int64_t)img * cg.sn + (int64_t)c * cg.sc + (int64_t)h * cg.sh + w8 * 8;
+      tp_row[j] = h;
       tp_c[j] = c;
     }
     for (int m = tid; m <= rows; m += THREADS) {  // the halo groups of both copies; the steps never write them
@@ -316,7 +319,10 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
     }
     const int prow = div(gat_row, cg.m_Q), q = gat_row - prow * cg.Q;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) gat_base[r] = (uint32_t)(((r * cg.rpb + prow) * cg.PW + 8 + q - cg.pad_w) * 2);
+    for (int r = 0; r < 4; ++r) {
+      const int first_row = cg.units == 1 ? r * cg.rpb : r * nch * cg.PR;  // of row block r in a copy
+      gat_base[r] = (uint32_t)(((first_row + prow) * cg.PW + 8 + q - cg.pad_w) * 2);
+    }
   }
   if constexpr (IMPLICIT && TRANS) {
     const int k_lo = rb0 * BS;
@@ -353,12 +359,11 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   [[maybe_unused]] auto tpatch_load = [&](uint32_t entry) {
     if constexpr (!TRANS) {  // forward: the step's reduction block is a block of 64 columns, i.e. a run of channels
       const int c_lo = div(step_block(entry) * BS, cg.m_RS);
-      const uint16_t* src = fwd_x0 + (int64_t)c_lo * cg.sc;
+      const uint16_t* src = cg.x + (int64_t)c_lo * cg.sc;
 #pragma unroll
       for (int j = 0; j < TSEG; ++j) {
-        const int h = fwd_h0 + tp_row[j];
         tp_v[j] = u32x4{0u, 0u, 0u, 0u};
-        if (tp_dst[j] >= 0 && h >= 0 && h < cg.H && c_lo + tp_c[j] < cg.C)
+        if (tp_dst[j] >= 0 && tp_row[j] >= 0 && tp_row[j] < cg.H && c_lo + tp_c[j] < cg.C)
           tp_v[j] = *reinterpret_cast<const u32x4*>(src + tp_src[j]);
       }
       return;
@@ -1170,7 +1175,7 @@ int launch_conv_t(const GemmArgs& g, const ImplicitConv& cg, int smem, hipStream
   auto* kernel = &dsd_kernel<T, false, false, RAGGED, DsdConv, FORM>;
   if (int rc = allow_big_lds(reinterpret_cast<const void*>(kernel), 163840, configured)) return rc;
   const int Mb = (int)(g.M / BS), Kb = (int)((g.K + BS - 1) / BS);
-  const int tiles_m = Mb / DsdConv::R, tiles_n = (int)((g.N + DsdConv::BN - 1) / DsdConv::BN);
+  const int tiles_m = (Mb + DsdConv::R - 1) / DsdConv::R, tiles_n = (int)((g.N + DsdConv::BN - 1) / DsdConv::BN);
   hipLaunchKernelGGL(kernel, dim3((unsigned)(tiles_m * tiles_n), 1u), dim3(DsdConv::THREADS), smem, stream, g,
                      tiles_m, tiles_n, Mb, Kb, cg);
   return check_launch("dsd_kernel (implicit conv)");
@@ -1236,8 +1241,12 @@ int conv_dw_splits(int64_t M, int64_t N, int64_t K) {
 int launch_conv_implicit(const GemmArgs& g, const ImplicitConv& cg, int64_t P, int64_t stride_h, int64_t stride_w,
                          int64_t dil_h, int64_t dil_w, int64_t R, int64_t x_sw, int dtype, hipStream_t stream) {
   if (g.row_ptr != nullptr && g.bs != BS) return SD_ERR_UNSUPPORTED;
+  // the four row blocks of a workgroup: consecutive output rows of one image sharing their input rows (units == 1,
+  // P * Q a multiple of 256), or each with its own input rows (units == 4, P * Q a multiple of 64)
+  const bool units_ok = (cg.units == 1 && (P * cg.Q) % (BS * DsdConv::R) == 0 && cg.PR == DsdConv::R * cg.rpb + R - 1) ||
+                        (cg.units == 4 && (P * cg.Q) % BS == 0 && cg.PR == cg.rpb + R - 1);
   const bool geom_ok = stride_h == 1 && stride_w == 1 && dil_h == 1 && dil_w == 1 && x_sw == 1 && cg.Q > 0 &&
-                       cg.Q <= BS && BS % cg.Q == 0 && (P * cg.Q) % (BS * DsdConv::R) == 0 && cg.W % 8 == 0 &&
+                       cg.Q <= BS && BS % cg.Q == 0 && units_ok && cg.W % 8 == 0 &&
                        cg.pad_h >= 0 && cg.pad_w >= 0 && cg.pad_w <= 8 && cg.S - 1 - cg.pad_w <= 8 && R * cg.S == cg.RS &&
                        cg.PW == cg.W + 8;
   if (!geom_ok) return SD_ERR_UNSUPPORTED;
@@ -1245,19 +1254,19 @@ int launch_conv_implicit(const GemmArgs& g, const ImplicitConv& cg, int64_t P, i
   if (Kb > MAX_STEPS) return SD_ERR_UNSUPPORTED;
   const bool align_ok = aligned16(cg.x) && cg.sn % 8 == 0 && cg.sc % 8 == 0 && cg.sh % 8 == 0 && aligned16(g.b.ptr) &&
                         g.b.sc == 1 && g.b.sr % 8 == 0 && g.b.sr < (1 << 22) && g.c_sc == 1 && g.K % 8 == 0 &&
-                        g.M % (BS * DsdConv::R) == 0 && g.M / (BS * DsdConv::R) * ((g.N + 127) / 128) < 0x7fffffffLL;
+                        g.M % BS == 0 && (g.M / (BS * DsdConv::R) + 1) * ((g.N + 127) / 128) < 0x7fffffffLL;
   if (!align_ok) return SD_ERR_UNSUPPORTED;
   // two alternating copies of the channels one step's 64 columns touch (any number of channels; measured at least
   // as fast as the other form wherever both fit) ...
   const int64_t nch = (BS + cg.RS - 2) / cg.RS + 1;
-  const int64_t copy_elems = (nch * cg.PR * cg.PW + 8 + 7) & ~7LL;
+  const int64_t copy_elems = (cg.units * nch * cg.PR * cg.PW + 8 + 7) & ~7LL;
   const int64_t stepwise = 2 * copy_elems * 2 + Kb * BS * 2;
   const bool step_ok = copy_elems * 2 <= CONV_T_PATCH_MAX && stepwise <= CONV_PATCH_MAX;
   // ... or one copy of every channel's rows for the whole kernel if that fits next to the stages (many taps per
   // 64 columns, e.g. 1 x 1 kernels, make a step's copy large; the large-tile policy prefers this form)
   const int64_t patch_elems = (int64_t)cg.C * cg.PR * cg.PW + 8;  // rows with their halo groups, one more after the last
   const int64_t whole = patch_elems * 2 + Kb * BS * 2;
-  const bool whole_ok = whole <= CONV_PATCH_MAX;
+  const bool whole_ok = whole <= CONV_PATCH_MAX && cg.units == 1;
   if (!step_ok && !whole_ok) return SD_ERR_UNSUPPORTED;
   const bool use_steps = step_ok && !(whole_ok && tile_policy.load(std::memory_order_relaxed) == kTileBig);
   const bool ragged = g.N % BS != 0 || g.K % BS != 0;
