@@ -253,8 +253,11 @@ int sd_col2im(const void* cols, int64_t cols_ld, void* dx, int64_t dx_stride_n,
  * no counterpart (its conv variants are stubs, layers/dropout_conv.py:86-99).
  *
  * Taken: stride 1, dilation 1, unit w stride of x, W a multiple of 8, Q a divisor of 64, P*Q a multiple of
- * 256, C*R*S a multiple of 8, R*S <= 30, and the input rows of 256 output positions (all channels) plus a
- * column table fitting in LDS (C * (256/Q + R - 1) * W * 2 + ceil(C*R*S/64)*256 <= about 55 KB).
+ * 64, C*R*S a multiple of 8 and at most 65536, pad_w <= 8 and S - 1 - pad_w <= 8, and one of two LDS budgets:
+ * the input rows that the <= 64 / (R*S) + 2 channels of one 64-column step touch within 24 KB (any number of
+ * channels; not 1 x 1 kernels with many channels), or the input rows of 256 output positions of ALL channels plus
+ * a column table within about 55 KB (C * (256/Q + R - 1) * (W + 8) * 2 + ceil(C*R*S/64) * 128; needs P*Q a
+ * multiple of 256).
  * Anything else returns SD_ERR_UNSUPPORTED with nothing launched: use sd_im2col + sd_gemm_dsd_lists.
  * NULL lists = every block kept: the dense convolution (block_size is then ignored, scale still applied).
  * ------------------------------------------------------------------------------------------- */
@@ -280,10 +283,10 @@ int sd_conv2d_dsd_lists(const void* x, int64_t x_stride_n, int64_t x_stride_c, i
 /* Input gradient of the same convolution in one launch: sd_gemm_sdd_lists_kept + sd_col2im without the gradient
  * of the patch matrix in memory.  dy is [N*P*Q, k_out] row-major, weight [k_out, C*R*S] row-major, dx [N, C, H, W]
  * addressed by element strides, fully overwritten.  mask: one byte per 64 x 64 block of the patch
- * matrix (non-zero = dropped, strides in bytes), NULL = dense.  A workgroup keeps the dY tiles of the output rows
- * that reach its band of input rows in LDS, forms the kept tiles of dY . W per 64-column block and folds them
+ * matrix (non-zero = dropped, strides in bytes), NULL = dense.  A workgroup keeps the dY rows of the output rows
+ * that reach its band of input rows in registers, forms the kept tiles of dY . W per 64-column block and folds them
  * (deterministically: every dx element has one owner and a fixed summation order).  Taken: stride 1, dilation 1,
- * block_size 64, k_out 64 or 128, Q a divisor of 64, P*Q a multiple of 64, C*R*S a multiple of 8 and at most 4096,
+ * block_size 64, k_out a multiple of 64 up to 256, Q a divisor of 64, P*Q a multiple of 64, C*R*S a multiple of 8 and at most 4096,
  * R*S <= 64, small kernels relative to the row block (R - 1 <= 64/Q + 1); anything else returns SD_ERR_UNSUPPORTED
  * with nothing launched.  No counterpart in the reference. */
 int sd_conv2d_dx(const void* dy, int64_t dy_ld, const void* weight, int64_t weight_ld,
