@@ -157,10 +157,28 @@ def cpu_baseline(size: int, bs: int, p: float, reps: int):
         naive_torch.forward_backward(x, w, dy, mask, bs, p)
         ts.append(time.perf_counter() - t0)
     t = statistics.median(ts)
+    # per-core figure: the same path on one thread at a size that keeps it to a few seconds
+    threads = torch.get_num_threads()
+    small = min(size, 2048)
+    xs, ws, dys = x[:small, :small].contiguous(), w[:small, :small].contiguous(), dy[:small, :small].contiguous()
+    ms_ = mask[: small // bs, : small // bs].contiguous()
+    torch.set_num_threads(1)
+    try:
+        naive_torch.forward_backward(xs, ws, dys, ms_, bs, p)
+        t1s = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            naive_torch.forward_backward(xs, ws, dys, ms_, bs, p)
+            t1s.append(time.perf_counter() - t0)
+    finally:
+        torch.set_num_threads(threads)
+    t1 = statistics.median(t1s)
     return {
+        "one_core": {"value": round(6.0 * small ** 3 / t1 / 1e12, 4), "unit": "TFLOP/s", "cores": 1,
+                     "sample": f"same path, torch.set_num_threads(1), M=N=K={small}, median of 3 reps ({t1 * 1e3:.1f} ms each)"},
         "value": round(6.0 * size ** 3 / t / 1e12, 4),
         "unit": "TFLOP/s",
-        "cores": torch.get_num_threads(),
+        "cores": threads,
         "kind": "port",
         "sample": f"oracle/naive_torch.py fwd+bwd fp32 at M=N=K={size}, bs={bs}, p={p}, median of {reps} reps "
                   f"({t * 1e3:.1f} ms each; host has {os.cpu_count()} logical cpus); dense-equivalent 6MNK/t",
