@@ -252,8 +252,8 @@ int sd_col2im(const void* cols, int64_t cols_ld, void* dx, int64_t dx_stride_n,
  * leading dimension y_ld.  This is what report.pdf section 5.3 proposes as future work; the reference has
  * no counterpart (its conv variants are stubs, layers/dropout_conv.py:86-99).
  *
- * Taken: stride 1, dilation 1, unit w stride of x, W a multiple of 8, Q a divisor of 64, P*Q a multiple of
- * 64, C*R*S a multiple of 8 and at most 65536, pad_w <= 8 and S - 1 - pad_w <= 8, and one of two LDS budgets:
+ * Taken: strides and dilations up to 8, unit w stride of x, W a multiple of 8, Q a divisor of 64, P*Q a multiple of
+ * 64, C*R*S a multiple of 8 and at most 65536, pad_w <= 8 and (S - 1) * dil_w - pad_w <= 8, and one of two LDS budgets:
  * the input rows that the <= 64 / (R*S) + 2 channels of one 64-column step touch within 24 KB (any number of
  * channels; not 1 x 1 kernels with many channels), or the input rows of 256 output positions of ALL channels plus
  * a column table within about 55 KB (C * (256/Q + R - 1) * (W + 8) * 2 + ceil(C*R*S/64) * 128; needs P*Q a
@@ -277,7 +277,7 @@ int sd_conv2d_dsd_lists(const void* x, int64_t x_stride_n, int64_t x_stride_c, i
  * NULL = dense).  The reduction runs over output positions: every step copies the input rows of its 64 positions
  * (the channels of the workgroup's 256 columns only) into LDS and builds the kept tiles from them; it is split over
  * workgroups when `workspace` (sd_conv2d_dw_workspace_bytes bytes, 16-byte aligned; may be NULL) allows.
- * Taken: stride 1, dilation 1, unit w stride of x, W a multiple of 8, Q a divisor of 64, P*Q a multiple of 64,
+ * Taken: strides and dilations up to 8, unit w stride of x, W a multiple of 8, Q a divisor of 64, P*Q a multiple of 64,
  * C*R*S and k_out multiples of 8, one step's copy <= 24 KB.  Anything else returns SD_ERR_UNSUPPORTED with
  * nothing launched.  No counterpart in the reference. */
 /* Input gradient of the same convolution in one launch: sd_gemm_sdd_lists_kept + sd_col2im without the gradient

@@ -112,7 +112,7 @@ using namespace sd;
 // Geometry of an implicit-GEMM launch whose LDS copy of the input covers `blocks` 64-position row blocks.
 static ImplicitConv conv_geometry(const void* x, int64_t sn, int64_t sc, int64_t sh, int64_t c, int64_t h, int64_t w,
                                   int64_t P, int64_t Q, int64_t r, int64_t s, int64_t pad_h, int64_t pad_w,
-                                  int64_t blocks) {
+                                  int64_t stride_h, int64_t stride_w, int64_t dil_h, int64_t dil_w, int64_t blocks) {
   ImplicitConv cg;
   cg.x = static_cast<const uint16_t*>(x);
   cg.sn = sn;
@@ -128,7 +128,11 @@ static ImplicitConv conv_geometry(const void* x, int64_t sn, int64_t sc, int64_t
   cg.pad_w = (int)pad_w;
   cg.rpb = (int)(64 / Q);
   cg.blocks_per_img = (int)(P * Q / 64);
-  cg.PR = (int)(blocks * (64 / Q) + r - 1);
+  cg.sth = (int)stride_h;
+  cg.stw = (int)stride_w;
+  cg.dlh = (int)dil_h;
+  cg.dlw = (int)dil_w;
+  cg.PR = (int)((blocks * (64 / Q) - 1) * stride_h + (r - 1) * dil_h + 1);
   cg.PW = (int)(w + 8);
   cg.patch_stride = 0;
   cg.units = 1;
@@ -373,12 +377,14 @@ int sd_conv2d_dsd_lists(const void* x, int64_t sn, int64_t sc, int64_t sh, int64
   const int64_t Q = (w + 2 * pad_w - dil_w * (s - 1) - 1) / stride_w + 1;
   SD_REQUIRE(P > 0 && Q > 0, "the kernel does not fit the padded input");
   SD_REQUIRE(wld >= c * r * s && yld >= k_out, "leading dimensions too small");
-  if (bs != 64 || Q > 64 || 64 % Q != 0 || c * r * s > (1 << 16) || h > (1 << 20) || w > (1 << 12) || r > 64 || s > 64)
+  if (bs != 64 || Q > 64 || 64 % Q != 0 || c * r * s > (1 << 16) || h > (1 << 20) || w > (1 << 12) || r > 64 || s > 64 ||
+      stride_h > 8 || stride_w > 8 || dil_h > 8 || dil_w > 8)
     return SD_ERR_UNSUPPORTED;
   // a workgroup's 256 output positions: 4 * 64 / Q consecutive rows of one image where P * Q allows, else four
   // separate 64-position blocks
   const bool one_run = (P * Q) % 256 == 0;
-  ImplicitConv cg = conv_geometry(x, sn, sc, sh, c, h, w, P, Q, r, s, pad_h, pad_w, /*blocks=*/one_run ? 4 : 1);
+  ImplicitConv cg = conv_geometry(x, sn, sc, sh, c, h, w, P, Q, r, s, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w,
+                                  /*blocks=*/one_run ? 4 : 1);
   cg.units = one_run ? 1 : 4;
   GemmArgs g = make_args(nullptr, 0, 0, weight, wld, 1, y, yld, 1, n * P * Q, k_out, c * r * s, bs, scale, row_ptr,
                          col_idx);
@@ -434,9 +440,11 @@ int sd_conv2d_dw_lists(const void* x, int64_t sn, int64_t sc, int64_t sh, int64_
   const int64_t Q = (w + 2 * pad_w - dil_w * (s - 1) - 1) / stride_w + 1;
   SD_REQUIRE(P > 0 && Q > 0, "the kernel does not fit the padded input");
   SD_REQUIRE(dyld >= k_out && dwld >= c * r * s, "leading dimensions too small");
-  if (bs != 64 || Q > 64 || 64 % Q != 0 || c * r * s > (1 << 16) || h > (1 << 20) || w > (1 << 12) || r > 64 || s > 64)
+  if (bs != 64 || Q > 64 || 64 % Q != 0 || c * r * s > (1 << 16) || h > (1 << 20) || w > (1 << 12) || r > 64 || s > 64 ||
+      stride_h > 8 || stride_w > 8 || dil_h > 8 || dil_w > 8)
     return SD_ERR_UNSUPPORTED;
-  ImplicitConv cg = conv_geometry(x, sn, sc, sh, c, h, w, P, Q, r, s, pad_h, pad_w, /*blocks=*/1);
+  ImplicitConv cg = conv_geometry(x, sn, sc, sh, c, h, w, P, Q, r, s, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w,
+                                  /*blocks=*/1);
   GemmArgs g = make_args(nullptr, 1, c * r * s, dy, 1, dyld, dw, 1, dwld, c * r * s, k_out, n * P * Q, bs, scale,
                          col_ptr, row_idx, workspace, workspace_bytes);
   const int rc = launch_conv_implicit_dw(g, cg, P, stride_h, stride_w, dil_h, dil_w, r, sw, dtype, (hipStream_t)stream);

@@ -109,17 +109,19 @@ struct GemmArgs {
   bool kept_only;    // SDD: dropped tiles of C are left untouched instead of being zeroed
 };
 
-// Geometry of a stride-1, dilation-1 convolution whose patch matrix the DSD kernel gathers itself
-// (implicit GEMM): x[n][c][h][w] with unit w stride, row block = 64 / Q whole output rows of one image.
+// Geometry of a convolution whose patch matrix the DSD kernel gathers itself (implicit GEMM):
+// x[n][c][h][w] with unit w stride, row block = 64 / Q whole output rows of one image.
 struct ImplicitConv {
   const uint16_t* x;
   int64_t sn, sc, sh;  // element strides of x
   int C, H, W, Q;      // channels, input height and width, output width
   int RS, S;           // taps per channel, kernel width
   int pad_h, pad_w;
+  int sth, stw, dlh, dlw;  // strides and dilations
   int rpb;             // output rows per 64-row block (64 / Q)
   int blocks_per_img;  // P * Q / 64
-  int PR;              // input rows a workgroup's 4 row blocks touch: 4 * rpb + R - 1 (units == 4: one block, rpb + R - 1)
+  int PR;              // input rows the output rows of a workgroup's 4 row blocks (units == 4: of one block) touch:
+                       // (output rows - 1) * stride + (R - 1) * dilation + 1
   int units;           // forward: 1 = the 4 row blocks share one run of input rows, 4 = each has its own (P*Q % 256 != 0)
   int PW;              // halfs per row of the LDS copy: 8 zeros, then the W of the image
   int patch_stride;    // weight gradient: halfs between the two alternating copies (set by the launcher)

@@ -231,7 +231,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   if constexpr (IMPLICIT == 1 && !TRANS) {
     const int img = rb0 / cg.blocks_per_img;
     const int p0 = (rb0 - img * cg.blocks_per_img) * cg.rpb;  // first output row of the workgroup
-    const int h0 = p0 - cg.pad_h;                              // input row of patch row 0
+    const int h0 = p0 * cg.sth - cg.pad_h;                     // input row of patch row 0
     const int spr = cg.W / 8, spc = cg.PR * spr;               // 16-byte segments per row, per channel
     const int total = cg.C * spc;
     const int rows = cg.C * cg.PR;
@@ -257,11 +257,12 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
       const int c = div(k, cg.m_RS), tap = k - c * cg.RS;
       const int rr = div(tap, cg.m_S), ss = tap - rr * cg.S;
       // columns past the last one read anything readable: their fragments are zeroed before the MFMAs
-      ktab[k] = k < cg.K ? (uint16_t)(((c * cg.PR + rr) * cg.PW + ss) * 2) : (uint16_t)0;
+      ktab[k] = k < cg.K ? (uint16_t)(((c * cg.PR + rr * cg.dlh) * cg.PW + ss * cg.dlw) * 2) : (uint16_t)0;
     }
     const int prow = div(gat_row, cg.m_Q), q = gat_row - prow * cg.Q;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) gat_base[r] = (uint32_t)(((r * cg.rpb + prow) * cg.PW + 8 + q - cg.pad_w) * 2);
+    for (int r = 0; r < 4; ++r)
+      gat_base[r] = (uint32_t)(((r * cg.rpb + prow) * cg.sth * cg.PW + 8 + q * cg.stw - cg.pad_w) * 2);
 #pragma unroll
     for (int j = 0; j < MAXSEG; ++j)
       if (dst[j] >= 0) *reinterpret_cast<u32x4*>(patch + dst[j]) = v[j];
@@ -301,7 +302,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
       const int row = div(rem, cg.m_spr), w8 = rem - row * spr;
       const int rb = rb0 + u;
       const int img = rb / cg.blocks_per_img;
-      const int h = (rb - img * cg.blocks_per_img) * cg.rpb - cg.pad_h + row;  // input row of the segment
+      const int h = (rb - img * cg.blocks_per_img) * cg.rpb * cg.sth - cg.pad_h + row;  // input row of the segment
       tp_dst[j] = (seg < total && rb < Mb) ? ((u * nch + c) * cg.PR + row) * cg.PW + 8 + w8 * 8 : -1;
       tp_src[j] = (int64_t)img * cg.sn + (int64_t)c * cg.sc + (int64_t)h * cg.sh + w8 * 8;
       tp_row[j] = h;
@@ -315,13 +316,13 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
       const int c = div(k, cg.m_RS), tap = k - c * cg.RS;
       const int rr = div(tap, cg.m_S), ss = tap - rr * cg.S;
       const int c_lo = div(k & ~(BS - 1), cg.m_RS);  // first channel of the column's block = of its step's copy
-      ktab[k] = k < cg.K ? (uint16_t)((((c - c_lo) * cg.PR + rr) * cg.PW + ss) * 2) : (uint16_t)0;
+      ktab[k] = k < cg.K ? (uint16_t)((((c - c_lo) * cg.PR + rr * cg.dlh) * cg.PW + ss * cg.dlw) * 2) : (uint16_t)0;
     }
     const int prow = div(gat_row, cg.m_Q), q = gat_row - prow * cg.Q;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int first_row = cg.units == 1 ? r * cg.rpb : r * nch * cg.PR;  // of row block r in a copy
-      gat_base[r] = (uint32_t)(((first_row + prow) * cg.PW + 8 + q - cg.pad_w) * 2);
+      const int first_row = cg.units == 1 ? r * cg.rpb * cg.sth : r * nch * cg.PR;  // of row block r in a copy
+      gat_base[r] = (uint32_t)(((first_row + prow * cg.sth) * cg.PW + 8 + q * cg.stw - cg.pad_w) * 2);
     }
   }
   if constexpr (IMPLICIT && TRANS) {
@@ -350,10 +351,10 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
       const int c = div(k, cg.m_RS), tap = k - c * cg.RS;
       const int rr = div(tap, cg.m_S), ss = tap - rr * cg.S;
       // columns past the last one belong to rows of the result that are not stored
-      ktab[kl] = k < cg.K ? (uint16_t)((((c - c_lo) * cg.PR + rr) * cg.PW + ss) * 2) : (uint16_t)0;
+      ktab[kl] = k < cg.K ? (uint16_t)((((c - c_lo) * cg.PR + rr * cg.dlh) * cg.PW + ss * cg.dlw) * 2) : (uint16_t)0;
     }
     const int prow = div(gat_row, cg.m_Q), q = gat_row - prow * cg.Q;
-    gat_base[0] = (uint32_t)((prow * cg.PW + 8 + q - cg.pad_w) * 2);
+    gat_base[0] = (uint32_t)((prow * cg.sth * cg.PW + 8 + q * cg.stw - cg.pad_w) * 2);
   }
   // fetches the input rows of the step with table word `entry` (its reduction block is a block of 64 positions)
   [[maybe_unused]] auto tpatch_load = [&](uint32_t entry) {
@@ -370,7 +371,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
     }
     const int mb = step_block(entry);
     const int img = mb / cg.blocks_per_img;
-    const int h0 = (mb - img * cg.blocks_per_img) * cg.rpb - cg.pad_h;
+    const int h0 = (mb - img * cg.blocks_per_img) * cg.rpb * cg.sth - cg.pad_h;
     const uint16_t* src = cg.x + (int64_t)img * cg.sn + (int64_t)h0 * cg.sh;
 #pragma unroll
     for (int j = 0; j < TSEG; ++j) {
@@ -1202,10 +1203,11 @@ int launch_conv_dw_t(const GemmArgs& g, const ImplicitConv& cg, int smem, int sp
 int launch_conv_implicit_dw(const GemmArgs& g, ImplicitConv cg, int64_t P, int64_t stride_h, int64_t stride_w,
                             int64_t dil_h, int64_t dil_w, int64_t R, int64_t x_sw, int dtype, hipStream_t stream) {
   if (g.row_ptr != nullptr && g.bs != BS) return SD_ERR_UNSUPPORTED;
-  const bool geom_ok = stride_h == 1 && stride_w == 1 && dil_h == 1 && dil_w == 1 && x_sw == 1 && cg.Q > 0 &&
-                       cg.Q <= BS && BS % cg.Q == 0 && (P * cg.Q) % BS == 0 && cg.W % 8 == 0 && cg.pad_h >= 0 &&
-                       cg.pad_w >= 0 && cg.pad_w <= 8 && cg.S - 1 - cg.pad_w <= 8 && R * cg.S == cg.RS &&
-                       cg.PW == cg.W + 8 && cg.PR == cg.rpb + R - 1;
+  const bool geom_ok = stride_h == cg.sth && stride_w == cg.stw && dil_h == cg.dlh && dil_w == cg.dlw && x_sw == 1 &&
+                       cg.Q > 0 && cg.Q <= BS && BS % cg.Q == 0 && (P * cg.Q) % BS == 0 && cg.W % 8 == 0 &&
+                       cg.pad_h >= 0 && cg.pad_w >= 0 && cg.pad_w <= 8 && (cg.S - 1) * dil_w - cg.pad_w <= 8 &&
+                       R * cg.S == cg.RS && cg.PW == cg.W + 8 &&
+                       cg.PR == (cg.rpb - 1) * stride_h + (R - 1) * dil_h + 1;
   if (!geom_ok) return SD_ERR_UNSUPPORTED;
   const int64_t nch_max = (DsdConv::R * BS - 1) / cg.RS + 2;  // channels 256 consecutive columns can touch
   const int64_t copy_elems = ((nch_max < cg.C ? nch_max : cg.C) * cg.PR * cg.PW + 8 + 7) & ~7LL;
@@ -1243,11 +1245,13 @@ int launch_conv_implicit(const GemmArgs& g, const ImplicitConv& cg, int64_t P, i
   if (g.row_ptr != nullptr && g.bs != BS) return SD_ERR_UNSUPPORTED;
   // the four row blocks of a workgroup: consecutive output rows of one image sharing their input rows (units == 1,
   // P * Q a multiple of 256), or each with its own input rows (units == 4, P * Q a multiple of 64)
-  const bool units_ok = (cg.units == 1 && (P * cg.Q) % (BS * DsdConv::R) == 0 && cg.PR == DsdConv::R * cg.rpb + R - 1) ||
-                        (cg.units == 4 && (P * cg.Q) % BS == 0 && cg.PR == cg.rpb + R - 1);
-  const bool geom_ok = stride_h == 1 && stride_w == 1 && dil_h == 1 && dil_w == 1 && x_sw == 1 && cg.Q > 0 &&
-                       cg.Q <= BS && BS % cg.Q == 0 && units_ok && cg.W % 8 == 0 &&
-                       cg.pad_h >= 0 && cg.pad_w >= 0 && cg.pad_w <= 8 && cg.S - 1 - cg.pad_w <= 8 && R * cg.S == cg.RS &&
+  const int64_t taps_h = (R - 1) * dil_h + 1;  // input rows under one output row
+  const bool units_ok =
+      (cg.units == 1 && (P * cg.Q) % (BS * DsdConv::R) == 0 && cg.PR == (DsdConv::R * cg.rpb - 1) * stride_h + taps_h) ||
+      (cg.units == 4 && (P * cg.Q) % BS == 0 && cg.PR == (cg.rpb - 1) * stride_h + taps_h);
+  const bool geom_ok = stride_h == cg.sth && stride_w == cg.stw && dil_h == cg.dlh && dil_w == cg.dlw && x_sw == 1 &&
+                       cg.Q > 0 && cg.Q <= BS && BS % cg.Q == 0 && units_ok && cg.W % 8 == 0 && cg.pad_h >= 0 &&
+                       cg.pad_w >= 0 && cg.pad_w <= 8 && (cg.S - 1) * dil_w - cg.pad_w <= 8 && R * cg.S == cg.RS &&
                        cg.PW == cg.W + 8;
   if (!geom_ok) return SD_ERR_UNSUPPORTED;
   const int64_t Kb = (g.K + BS - 1) / BS;

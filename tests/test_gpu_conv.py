@@ -130,7 +130,10 @@ IMPLICIT_GEOMS = [
     (dict(n=5, c=24, h=32, w=8, k=72, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),     # 8 output rows per block
     (dict(n=2, c=16, h=36, w=32, k=64, r=5, s=1, padding=(0, 0), stride=(1, 1), dilation=(1, 1)), True),    # no padding: P = 32 from H = 36
     (dict(n=2, c=16, h=16, w=16, k=64, r=3, s=3, padding=(2, 2), stride=(1, 1), dilation=(1, 1)), False),   # Q = 18
-    (dict(n=2, c=8, h=32, w=32, k=64, r=3, s=3, padding=(1, 1), stride=(2, 2), dilation=(1, 1)), False),    # stride
+    (dict(n=2, c=8, h=32, w=32, k=64, r=3, s=3, padding=(1, 1), stride=(2, 2), dilation=(1, 1)), True),     # stride 2: 16 x 16 outputs
+    (dict(n=2, c=24, h=32, w=32, k=64, r=3, s=3, padding=(2, 2), stride=(1, 1), dilation=(2, 2)), True),    # dilation 2
+    (dict(n=3, c=16, h=32, w=32, k=72, r=3, s=3, padding=(1, 1), stride=(2, 1), dilation=(1, 1)), True),    # stride 2 down, 1 across
+    (dict(n=2, c=40, h=64, w=16, k=64, r=5, s=3, padding=(4, 1), stride=(2, 2), dilation=(2, 1)), True),    # stride and dilation, Q = 8
     (dict(n=1, c=16, h=8, w=16, k=64, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),     # P*Q = 128: every 64-position block with its own input rows, half a workgroup
     (dict(n=5, c=32, h=8, w=8, k=64, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),      # 8 x 8 images: a workgroup's four blocks are four images, the last workgroup has one
     (dict(n=3, c=72, h=12, w=16, k=136, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),   # P*Q = 192: blocks of 4 rows, three per image, 648 columns
