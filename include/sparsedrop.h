@@ -285,9 +285,9 @@ int sd_conv2d_dsd_lists(const void* x, int64_t x_stride_n, int64_t x_stride_c, i
  * addressed by element strides, fully overwritten.  mask: one byte per 64 x 64 block of the patch
  * matrix (non-zero = dropped, strides in bytes), NULL = dense.  A workgroup keeps the dY rows of the output rows
  * that reach its band of input rows in registers, forms the kept tiles of dY . W per 64-column block and folds them
- * (deterministically: every dx element has one owner and a fixed summation order).  Taken: stride 1, dilation 1,
+ * (deterministically: every dx element has one owner and a fixed summation order).  Taken: strides and dilations up to 8,
  * block_size 64, k_out a multiple of 64 up to 256, Q a divisor of 64, P*Q a multiple of 64, C*R*S a multiple of 8 and at most 4096,
- * R*S <= 64, small kernels relative to the row block (R - 1 <= 64/Q + 1); anything else returns SD_ERR_UNSUPPORTED
+ * R*S <= 64, kernels whose taps from one input row reach at most three 64-position row blocks; anything else returns SD_ERR_UNSUPPORTED
  * with nothing launched.  No counterpart in the reference. */
 int sd_conv2d_dx(const void* dy, int64_t dy_ld, const void* weight, int64_t weight_ld,
                  void* dx, int64_t dx_stride_n, int64_t dx_stride_c, int64_t dx_stride_h, int64_t dx_stride_w,

@@ -2,12 +2,13 @@
 // matrix ever reaching memory:
 //
 //   dx[n, c, h, w] = scale * sum over taps (r, s) of keep[m / 64, k / 64] * (dY . W)[m, k]
-//   with m = (n, h - r + pad_h, w - s + pad_w) the output position the tap reads from and k = (c, r, s)
+//   with m = (n, (h + pad_h - r * dil_h) / stride_h, (w + pad_w - s * dil_w) / stride_w) the output position the
+//   tap reads from (taps whose quotients are not whole or fall outside the output contribute nothing), k = (c, r, s)
 //
 // i.e. the SDD product dY . W restricted to kept 64 x 64 tiles followed by col2im (the adjoint of the
-// F.unfold gather of flash_dropout/functional/im2col_conv2d.py:17-20), for stride 1 and dilation 1.
+// F.unfold gather of flash_dropout/functional/im2col_conv2d.py:17-20).
 //
-// A workgroup owns HB = 2 * (64 / Q) input rows of one image, all channels.  The output rows whose taps
+// A workgroup owns HB = 2 * (64 / Q) * stride_h input rows of one image, all channels.  The output rows whose taps
 // reach them lie in at most four consecutive 64-position row blocks of dY; each of the eight waves keeps 32
 // rows of them (all of the reduction, K_out <= 256) in registers as MFMA operands for the whole kernel, so
 // that (for K_out <= 128) two workgroups fit a CU and one folds while the other multiplies.  Then, for every 64-column block of the patch
@@ -64,6 +65,7 @@ struct DxArgs {
   const uint8_t* mask;  // [N*P*Q/64, ceil(C*R*S/64)] bytes, non-zero = dropped; null = keep everything
   int64_t msr, msc;
   int C, H, W, P, Q, R, S, pad_h, pad_w;
+  int sth, stw, dlh, dlw;  // strides and dilations
   int rpb_shift;        // log2(64 / Q): output rows per row block
   int HB, bands;        // input rows per workgroup, workgroups per image
   int blocks_per_img;   // P * Q / 64
@@ -88,8 +90,10 @@ __global__ __launch_bounds__(THREADS) void conv_dx_kernel(DxArgs g) {
   const int h0 = band * g.HB;
   const int RS = RT > 0 ? RT * ST : g.R * g.S;
   const int rpb = 1 << g.rpb_shift;
-  // output rows the taps of input rows [h0, h0 + HB) read: p = h - r + pad_h
-  const int p_lo = h0 - (g.R - 1) + g.pad_h;
+  // output rows the taps of input rows [h0, h0 + HB) read: p = (h + pad_h - r * dil) / stride where that divides;
+  // the first of them is the quotient rounded up (also below zero)
+  const int t_lo = h0 + g.pad_h - (g.R - 1) * g.dlh;
+  const int p_lo = t_lo >= 0 ? (t_lo + g.sth - 1) / g.sth : -((-t_lo) / g.sth);
   const int pb0 = p_lo >> g.rpb_shift;  // arithmetic shift: floor, also below zero
   const int pbn = g.P >> g.rpb_shift;   // row blocks per image
 
@@ -163,16 +167,18 @@ __global__ __launch_bounds__(THREADS) void conv_dx_kernel(DxArgs g) {
   if constexpr (RT > 0) {
 #pragma unroll
     for (int rr = 0; rr < RT; ++rr) {
-      const int p = h - rr + g.pad_h;
-      const bool ok = p >= 0 && p < g.P && h < g.H;
+      const int t = h + g.pad_h - rr * g.dlh;
+      const int p = t >= 0 ? t / g.sth : 0;
+      const bool ok = t >= 0 && p * g.sth == t && p < g.P && h < g.H;
       const int b = ok ? (p >> g.rpb_shift) - pb0 : 0;
       tap_keep[rr] = ok ? keep[b] : 0ull;
       tap_row[rr] = (b * BS + (p - (pb0 + b) * rpb) * g.Q) * STAGE_LD;
     }
 #pragma unroll
     for (int ss = 0; ss < ST; ++ss) {
-      const int q = wq - ss + g.pad_w;
-      tap_col[ss] = (q >= 0 && q < g.Q) ? q * STAGE_LD : -1;
+      const int u = wq + g.pad_w - ss * g.dlw;
+      const int q = u >= 0 ? u / g.stw : 0;
+      tap_col[ss] = (u >= 0 && q * g.stw == u && q < g.Q) ? q * STAGE_LD : -1;
     }
   }
 
@@ -234,13 +240,16 @@ __global__ __launch_bounds__(THREADS) void conv_dx_kernel(DxArgs g) {
             }
           } else {
             for (int rr = 0; rr < g.R; ++rr) {
-              const int p = h - rr + g.pad_h;
+              const int t = h + g.pad_h - rr * g.dlh;
+              const int p = t >= 0 ? t / g.sth : 0;
               const int b = (p >> g.rpb_shift) - pb0;
-              const bool row_ok = p >= 0 && p < g.P && ((keep[b & (NB - 1)] >> j) & 1ull);
+              const bool row_ok = t >= 0 && p * g.sth == t && p < g.P && ((keep[b & (NB - 1)] >> j) & 1ull);
               const uint16_t* srow = stage + ((b & (NB - 1)) * BS + (p - (pb0 + b) * rpb) * g.Q) * STAGE_LD;
               for (int ss = 0; ss < g.S; ++ss, ++k) {
-                const int q = wq - ss + g.pad_w;
-                if (row_ok && k >= 0 && k < BS && q >= 0 && q < g.Q) sum += T::to_float(srow[q * STAGE_LD + k]);
+                const int u = wq + g.pad_w - ss * g.dlw;
+                const int q = u >= 0 ? u / g.stw : 0;
+                if (row_ok && k >= 0 && k < BS && u >= 0 && q * g.stw == u && q < g.Q)
+                  sum += T::to_float(srow[q * STAGE_LD + k]);
               }
             }
           }
@@ -287,19 +296,27 @@ int launch_conv_dx(const void* dy, int64_t dy_ld, const void* w, int64_t w_ld, v
                    int64_t h, int64_t wd, int64_t k_out, int64_t r, int64_t s, int64_t pad_h, int64_t pad_w,
                    int64_t stride_h, int64_t stride_w, int64_t dil_h, int64_t dil_w, float scale, int dtype,
                    hipStream_t stream) {
-  if (stride_h != 1 || stride_w != 1 || dil_h != 1 || dil_w != 1) return SD_ERR_UNSUPPORTED;
-  const int64_t P = h + 2 * pad_h - r + 1, Q = wd + 2 * pad_w - s + 1;
+  if (stride_h < 1 || stride_w < 1 || dil_h < 1 || dil_w < 1 || stride_h > 8 || stride_w > 8 || dil_h > 8 || dil_w > 8)
+    return SD_ERR_UNSUPPORTED;
+  const int64_t P = (h + 2 * pad_h - dil_h * (r - 1) - 1) / stride_h + 1;
+  const int64_t Q = (wd + 2 * pad_w - dil_w * (s - 1) - 1) / stride_w + 1;
   if (P <= 0 || Q <= 0 || Q > BS || BS % Q != 0 || (P * Q) % BS != 0) return SD_ERR_UNSUPPORTED;
   if (k_out % BS != 0 || k_out > BS * KS_LIMIT) return SD_ERR_UNSUPPORTED;
   const int64_t K = c * r * s, Kb = (K + BS - 1) / BS;
   if (Kb > 64 || K % 8 != 0 || r * s > BS) return SD_ERR_UNSUPPORTED;  // keep flags are one 64-bit word per row block
-  const int64_t rpb = BS / Q, HB = 2 * rpb;
-  // the output rows one band's taps read must fit the four row blocks held in LDS
-  // (first row p_lo = h0 - (R-1) + pad_h lies up to rpb-1 rows into its block)
-  if ((rpb - 1) + HB + (r - 1) > NB * rpb) return SD_ERR_UNSUPPORTED;
-  const int64_t hw_n = HB * wd;
+  const int64_t rpb = BS / Q;
   // a channel's columns span at most two blocks; the ring holds every channel a block column can touch
   const int64_t ring_n = (BS + r * s - 1) / (r * s) + 2;
+  const int64_t ring_max = k_out > 2 * BS ? DxLds<4>::ACC_MAX : DxLds<2>::ACC_MAX;
+  // a band of HB input rows per workgroup: the input rows under two row blocks of output, fewer if a band's elements
+  // of one channel outnumber the threads or the ring of open channel sums would not fit
+  // and the output rows one band's taps read must fit the four row blocks the waves hold: at most
+  // (HB - 1 + (R - 1) * dil) / stride + 1 of them, the first up to rpb - 1 rows into its block
+  auto rows_fit = [&](int64_t hb) { return (rpb - 1) + (hb - 1 + (r - 1) * dil_h) / stride_h + 1 <= NB * rpb; };
+  int64_t HB = 2 * rpb * stride_h;
+  while (HB > 1 && (HB * wd > THREADS || ring_n * HB * wd * 4 > ring_max || !rows_fit(HB))) HB /= 2;
+  if (!rows_fit(HB)) return SD_ERR_UNSUPPORTED;
+  const int64_t hw_n = HB * wd;
   if (hw_n > THREADS) return SD_ERR_UNSUPPORTED;
   const bool align_ok = reinterpret_cast<uintptr_t>(dy) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
                         dy_ld % 8 == 0 && w_ld % 8 == 0 && dy_ld >= k_out && w_ld >= K;
@@ -329,6 +346,10 @@ int launch_conv_dx(const void* dy, int64_t dy_ld, const void* w, int64_t w_ld, v
   g.S = (int)s;
   g.pad_h = (int)pad_h;
   g.pad_w = (int)pad_w;
+  g.sth = (int)stride_h;
+  g.stw = (int)stride_w;
+  g.dlh = (int)dil_h;
+  g.dlw = (int)dil_w;
   g.rpb_shift = 0;
   while ((1 << g.rpb_shift) < rpb) ++g.rpb_shift;
   g.HB = (int)HB;

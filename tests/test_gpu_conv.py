@@ -242,7 +242,7 @@ DX_GEOMS = [
     (dict(n=4, c=64, h=32, w=32, k=128, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),   # the conv configuration's layer
     (dict(n=2, c=16, h=16, w=16, k=64, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),    # 144 columns: ragged last block
     (dict(n=2, c=16, h=33, w=33, k=128, r=2, s=2, padding=(0, 0), stride=(1, 1), dilation=(1, 1)), True),   # 2x2 on a 33 x 33 image: one block column, 18 open channels
-    (dict(n=2, c=64, h=32, w=32, k=128, r=1, s=1, padding=(0, 0), stride=(1, 1), dilation=(1, 1)), False),  # 1x1: 64 channels per block column do not fit the ring
+    (dict(n=2, c=64, h=32, w=32, k=128, r=1, s=1, padding=(0, 0), stride=(1, 1), dilation=(1, 1)), True),   # 1x1: 66 open channels per block column, so the band shrinks to one input row for the ring to fit
     (dict(n=2, c=32, h=16, w=64, k=64, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),    # one output row per block
     (dict(n=3, c=24, h=32, w=8, k=128, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), True),    # 8 output rows per block
     (dict(n=2, c=16, h=34, w=32, k=64, r=3, s=1, padding=(0, 0), stride=(1, 1), dilation=(1, 1)), True),    # no padding, H not a multiple of the band
@@ -252,9 +252,12 @@ DX_GEOMS = [
     (dict(n=2, c=16, h=32, w=32, k=256, r=1, s=1, padding=(0, 0), stride=(1, 1), dilation=(1, 1)), True),   # 1x1 with K_out = 256: that instance's LDS holds the 66-slot ring
     (dict(n=1, c=16, h=32, w=32, k=320, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), False),  # K_out = 320
     (dict(n=2, c=40, h=32, w=32, k=128, r=2, s=2, padding=(0, 0), stride=(1, 1), dilation=(1, 1)), False),  # Q = 31
-    (dict(n=3, c=8, h=32, w=32, k=64, r=5, s=5, padding=(2, 2), stride=(1, 1), dilation=(1, 1)), False),    # 5 taps high on 2-row blocks
+    (dict(n=3, c=8, h=32, w=32, k=64, r=5, s=5, padding=(2, 2), stride=(1, 1), dilation=(1, 1)), True),     # 5 taps high on 2-row blocks: the band shrinks to two input rows
     (dict(n=2, c=16, h=16, w=16, k=40, r=3, s=3, padding=(1, 1), stride=(1, 1), dilation=(1, 1)), False),   # K_out = 40
-    (dict(n=2, c=8, h=32, w=32, k=64, r=3, s=3, padding=(1, 1), stride=(2, 2), dilation=(1, 1)), False),    # stride
+    (dict(n=2, c=8, h=32, w=32, k=64, r=3, s=3, padding=(1, 1), stride=(2, 2), dilation=(1, 1)), True),     # stride 2: three of four taps fall between outputs
+    (dict(n=2, c=24, h=32, w=32, k=64, r=3, s=3, padding=(2, 2), stride=(1, 1), dilation=(2, 2)), True),    # dilation 2
+    (dict(n=3, c=16, h=32, w=32, k=128, r=3, s=3, padding=(1, 1), stride=(2, 1), dilation=(1, 1)), True),   # stride 2 down, 1 across
+    (dict(n=2, c=40, h=64, w=16, k=64, r=5, s=3, padding=(4, 1), stride=(2, 2), dilation=(2, 1)), True),    # stride and dilation, Q = 8
 ]
 
 
