@@ -302,9 +302,12 @@ def test_fused_conv_input_gradient(cfg, taken, p, dtype, channels_last):
         assert dense is not None and rel_fro(dense, ref) <= REL_FRO_TOL
 
 
-def test_implicit_and_explicit_conv_routes_agree():
+@pytest.mark.parametrize("stride,dilation,padding", [((1, 1), (1, 1), (1, 1)), ((2, 2), (1, 1), (1, 1)),
+                                                     ((1, 1), (2, 2), (2, 2))])
+def test_implicit_and_explicit_conv_routes_agree(stride, dilation, padding):
     """The autograd function with the implicit forward (input kept, kept patch blocks re-gathered for the weight
-    gradient) and with the explicit one (patch matrix kept) give the same three results."""
+    gradient, fused input gradient) and with the explicit one (patch matrix kept) give the same three results,
+    also for a strided and for a dilated convolution."""
     import sys
 
     import flash_dropout.functional as F
@@ -313,15 +316,17 @@ def test_implicit_and_explicit_conv_routes_agree():
     gen = torch.Generator().manual_seed(9)
     x = torch.randn(4, 64, 32, 32, generator=gen).half().cuda()
     k = (torch.randn(128, 64, 3, 3, generator=gen) * 0.04).half().cuda()
-    dy = torch.randn(4, 128, 32, 32, generator=gen).half().cuda()
-    mask = (torch.rand(64, 9, generator=gen) < 0.5).cuda()
+    p_, q_ = O.conv_out_hw(32, 32, 3, 3, padding=padding, stride=stride, dilation=dilation)
+    dy = torch.randn(4, 128, p_, q_, generator=gen).half().cuda()
+    mask = (torch.rand(4 * p_ * q_ // 64, 9, generator=gen) < 0.5).cuda()
     out = {}
     for implicit in (True, False):
         prev, mod.IMPLICIT_FORWARD = mod.IMPLICIT_FORWARD, implicit
         prev_dx, mod.FUSED_INPUT_GRADIENT = mod.FUSED_INPUT_GRADIENT, implicit
         try:
             xg, kg = x.clone().requires_grad_(), k.clone().requires_grad_()
-            y = F.blockwise_dropout_conv2d_mask(xg, mask, 64, 0.5, kg, padding=(1, 1))
+            y = F.blockwise_dropout_conv2d_mask(xg, mask, 64, 0.5, kg, padding=padding, stride=stride,
+                                                dilation=dilation)
             y.backward(dy)
             out[implicit] = (y.detach(), xg.grad, kg.grad)
         finally:
