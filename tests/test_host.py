@@ -75,6 +75,28 @@ def test_host_validation_rejects_bad_arguments_without_touching_the_gpu():
     assert rc == 1 and b"does not fit" in lib.sd_last_error()
     rc = lib.sd_im2col(fake, 1, 1, 1, 1, fake, 4, 1, 1, 4, 4, 3, 3, 0, 0, 1, 1, 1, 1, None, None, 0, 0, None)
     assert rc == 1 and b"cols_ld" in lib.sd_last_error()
+    # the implicit-GEMM conv entry points: argument errors are reported (1), geometries without a kernel are
+    # declined (2) -- both before anything is launched
+    # x [1, 8, 4, 4], 3x3 without padding: P = Q = 2
+    conv = [1, 8, 4, 4, 64, 3, 3, 0, 0, 1, 1, 1, 1]  # n, c, h, w, k_out, r, s, pads, strides, dilations
+    rc = lib.sd_conv2d_dsd_lists(fake, 128, 16, 4, 1, fake, 72, None, 64, *conv, None, None, 64, 1.0, 0, None)
+    assert rc == 1 and b"null pointer" in lib.sd_last_error()
+    rc = lib.sd_conv2d_dsd_lists(fake, 128, 16, 4, 1, fake, 72, fake, 64, *conv, fake, None, 64, 1.0, 0, None)
+    assert rc == 1 and b"both be given" in lib.sd_last_error()
+    rc = lib.sd_conv2d_dsd_lists(fake, 128, 16, 4, 1, fake, 8, fake, 64, *conv, None, None, 64, 1.0, 0, None)
+    assert rc == 1 and b"leading dimensions" in lib.sd_last_error()
+    rc = lib.sd_conv2d_dsd_lists(fake, 128, 16, 4, 1, fake, 72, fake, 64, *conv, None, None, 64, 1.0, 0, None)
+    assert rc == 2  # P * Q = 4 is not a multiple of 64
+    rc = lib.sd_conv2d_dx(fake, 64, fake, 72, None, 128, 16, 4, 1, None, 0, 0, *conv, 64, 1.0, 0, None)
+    assert rc == 1 and b"null pointer" in lib.sd_last_error()
+    rc = lib.sd_conv2d_dx(fake, 64, fake, 72, fake, 128, 16, 4, 1, None, 0, 0, *conv[:9], 0, 1, 1, 1, 64, 1.0, 0, None)
+    assert rc == 1 and b"strides" in lib.sd_last_error()
+    rc = lib.sd_conv2d_dx(fake, 64, fake, 72, fake, 128, 16, 4, 1, fake, 1, 1, *conv, 128, 1.0, 0, None)
+    assert rc == 2  # a mask at another block size than 64
+    rc = lib.sd_conv2d_dw_lists(fake, 128, 16, 4, 1, fake, 64, None, 72, *conv, None, None, 64, 1.0, 0, None, 0, None)
+    assert rc == 1 and b"null pointer" in lib.sd_last_error()
+    assert lib.sd_conv2d_dw_workspace_bytes(128, 64, 128, 3, 3, 32, 32) >= 2 * 576 * 128 * 4
+    assert lib.sd_conv2d_dw_workspace_bytes(0, 64, 128, 3, 3, 32, 32) == 0
 
 
 def test_python_shim_rejects_cpu_and_fp32_operands():
