@@ -1,10 +1,11 @@
 """Whole-model forward + backward time as the drop rate varies (reference: benchmark/model.py:119-229).
 
-    python -m benchmark.model --model mlp vit-ffn --p 0 0.1 0.3 0.5 0.7
+    python -m benchmark.model --model mlp mlp-784 vit-ffn --p 0 0.1 0.3 0.5 0.7
 
 Models are built from ``DropoutMM`` the way the reference's evaluation models are:
   mlp      flattened 32x32 images -> [hidden]*layers -> 10 classes padded to 128, ReLU between, dropout on
            the input of every linear but the first (eval/mlp/model.py: BasicNet); batch 1024, hidden 1024
+  mlp-784  the same on 4096 unresized 28x28 images with 10 unpadded classes: 784 -> 1024 -> 1024 -> 10
   vit-ffn  one transformer feed-forward block on 64x256 tokens: 384 -> 1536 -> GELU -> 384, dropout on the
            inputs of both linears
 Each is timed with variant "none" (dense), "vanilla" (element dropout + dense) and "blockwise[hip]"."""
@@ -47,8 +48,17 @@ class VitFfn(nn.Module):
         return self.down(nn.functional.gelu(self.up(x)))
 
 
+class Mlp784(Mlp):
+    """28 x 28 images without the reference's resize and class padding: 784 -> 1024 -> 1024 -> 10, so the first
+    product has a ragged reduction (784 = 12 * 64 + 16) and the last one 10 output columns."""
+
+    def __init__(self, variant, p, block_size):
+        super().__init__(variant, p, block_size, in_dim=784, hidden=1024, layers=2, classes=10)
+
+
 MODELS = {
     "mlp": (Mlp, lambda: torch.rand(1024, 1, 32, 32)),
+    "mlp-784": (Mlp784, lambda: torch.rand(4096, 1, 28, 28)),
     "vit-ffn": (VitFfn, lambda: torch.randn(64, 256, 384)),
 }
 
