@@ -29,7 +29,10 @@ constexpr int TILE = BS * BS * 2;
 constexpr int THREADS = 512;
 constexpr int NB = 4;           // row blocks of dY per workgroup
 constexpr int KS_LIMIT = 4;     // 64-wide reduction steps at most: K_out <= 256
-constexpr int STAGE_LD = 68;    // halfs per staged row: 64 + 4 so that the two half-waves of a store hit different banks
+// A staged tile is kept column by column: [64 columns][64 positions + 4].  A lane's four accumulator registers of
+// one group are four consecutive positions of one column, i.e. one 8-byte store (the 136-byte column pitch puts the 32
+// columns of a store on all 64 banks once), and the fold's lanes, which run along w, read consecutive halfs.
+constexpr int STAGE_LD = 68;
 // LDS of an instance for K_out <= 64 * KS_MAX: two W tiles (one per buffer) of KS_MAX * 8 KB, the staging area, the ring
 template <int KS_MAX>
 struct DxLds {
@@ -172,13 +175,13 @@ __global__ __launch_bounds__(THREADS) void conv_dx_kernel(DxArgs g) {
       const bool ok = t >= 0 && p * g.sth == t && p < g.P && h < g.H;
       const int b = ok ? (p >> g.rpb_shift) - pb0 : 0;
       tap_keep[rr] = ok ? keep[b] : 0ull;
-      tap_row[rr] = (b * BS + (p - (pb0 + b) * rpb) * g.Q) * STAGE_LD;
+      tap_row[rr] = b * BS * STAGE_LD + (p - (pb0 + b) * rpb) * g.Q;
     }
 #pragma unroll
     for (int ss = 0; ss < ST; ++ss) {
       const int u = wq + g.pad_w - ss * g.dlw;
       const int q = u >= 0 ? u / g.stw : 0;
-      tap_col[ss] = (u >= 0 && q * g.stw == u && q < g.Q) ? q * STAGE_LD : -1;
+      tap_col[ss] = (u >= 0 && q * g.stw == u && q < g.Q) ? q : -1;
     }
   }
 
@@ -208,13 +211,17 @@ __global__ __launch_bounds__(THREADS) void conv_dx_kernel(DxArgs g) {
           }
         }
       }
-      uint16_t* st = stage + (t_blk * BS + half * 32) * STAGE_LD;
+      // accumulator register v of lane l is position 8*(v/4) + 4*(l/32) + v%4 of the wave's 32, column l%32
+      uint16_t* st = stage + t_blk * BS * STAGE_LD + half * 32 + 4 * (lane / 32);
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int row = 8 * (v / 4) + 4 * (lane / 32) + (v % 4);
-          st[row * STAGE_LD + nt * 32 + lane % 32] = T::from_float(acc[nt][v] * g.scale);
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const uint32_t lo = (uint32_t)T::from_float(acc[nt][4 * q4] * g.scale) |
+                              ((uint32_t)T::from_float(acc[nt][4 * q4 + 1] * g.scale) << 16);
+          const uint32_t hi = (uint32_t)T::from_float(acc[nt][4 * q4 + 2] * g.scale) |
+                              ((uint32_t)T::from_float(acc[nt][4 * q4 + 3] * g.scale) << 16);
+          *reinterpret_cast<u32x2*>(st + (nt * 32 + lane % 32) * STAGE_LD + 8 * q4) = u32x2{lo, hi};
         }
     }
     // the next W tile has had the products to arrive; so have the stores of the previous block's sums
@@ -236,7 +243,7 @@ __global__ __launch_bounds__(THREADS) void conv_dx_kernel(DxArgs g) {
 #pragma unroll
               for (int ss = 0; ss < ST; ++ss, ++k)
                 if (row_ok && tap_col[ss] >= 0 && (unsigned)k < (unsigned)BS)
-                  sum += T::to_float(stage[tap_row[rr] + tap_col[ss] + k]);
+                  sum += T::to_float(stage[tap_row[rr] + tap_col[ss] + k * STAGE_LD]);
             }
           } else {
             for (int rr = 0; rr < g.R; ++rr) {
@@ -244,12 +251,12 @@ __global__ __launch_bounds__(THREADS) void conv_dx_kernel(DxArgs g) {
               const int p = t >= 0 ? t / g.sth : 0;
               const int b = (p >> g.rpb_shift) - pb0;
               const bool row_ok = t >= 0 && p * g.sth == t && p < g.P && ((keep[b & (NB - 1)] >> j) & 1ull);
-              const uint16_t* srow = stage + ((b & (NB - 1)) * BS + (p - (pb0 + b) * rpb) * g.Q) * STAGE_LD;
+              const uint16_t* srow = stage + (b & (NB - 1)) * BS * STAGE_LD + (p - (pb0 + b) * rpb) * g.Q;
               for (int ss = 0; ss < g.S; ++ss, ++k) {
                 const int u = wq + g.pad_w - ss * g.dlw;
                 const int q = u >= 0 ? u / g.stw : 0;
                 if (row_ok && k >= 0 && k < BS && u >= 0 && q * g.stw == u && q < g.Q)
-                  sum += T::to_float(srow[q * STAGE_LD + k]);
+                  sum += T::to_float(srow[q + k * STAGE_LD]);
               }
             }
           }
