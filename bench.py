@@ -173,7 +173,21 @@ def cpu_baseline(size: int, bs: int, p: float, reps: int):
     finally:
         torch.set_num_threads(threads)
     t1 = statistics.median(t1s)
+    # the reference's own CPU-runnable case: 1024^3, median of 20 repetitions after 3 warm-ups, all threads
+    c1 = min(size, 1024)
+    xc, wc, dyc = x[:c1, :c1].contiguous(), w[:c1, :c1].contiguous(), dy[:c1, :c1].contiguous()
+    mc = mask[: c1 // bs, : c1 // bs].contiguous()
+    for _ in range(3):
+        naive_torch.forward_backward(xc, wc, dyc, mc, bs, p)
+    tcs = []
+    for _ in range(20):
+        t0 = time.perf_counter()
+        naive_torch.forward_backward(xc, wc, dyc, mc, bs, p)
+        tcs.append(time.perf_counter() - t0)
+    tc = statistics.median(tcs)
     return {
+        "small_case": {"value": round(6.0 * c1 ** 3 / tc / 1e12, 4), "unit": "TFLOP/s", "cores": threads,
+                       "sample": f"same path at M=N=K={c1}, median of 20 reps after 3 warm-ups ({tc * 1e3:.2f} ms each)"},
         "one_core": {"value": round(6.0 * small ** 3 / t1 / 1e12, 4), "unit": "TFLOP/s", "cores": 1,
                      "sample": f"same path, torch.set_num_threads(1), M=N=K={small}, median of 3 reps ({t1 * 1e3:.1f} ms each)"},
         "value": round(6.0 * size ** 3 / t / 1e12, 4),
