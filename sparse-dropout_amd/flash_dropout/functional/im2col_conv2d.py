@@ -37,7 +37,10 @@ def _pair(v) -> tuple[int, int]:
 def _to_matrix_grad(grad_output: torch.Tensor, dtype) -> torch.Tensor:
     """(N, K, P, Q) gradient -> [N*P*Q, K] row-major (free when it is channels-last in memory)."""
     n, k, p, q = grad_output.shape
-    return grad_output.to(dtype).permute(0, 2, 3, 1).reshape(n * p * q, k)
+    dy2 = grad_output.to(dtype).permute(0, 2, 3, 1).reshape(n * p * q, k)
+    if dy2.stride(1) != 1 or dy2.stride(0) < k:  # e.g. the expanded (stride 0) gradient of a sum()
+        dy2 = dy2.contiguous()
+    return dy2
 
 
 class _Im2colConv2d(torch.autograd.Function):

@@ -336,6 +336,32 @@ def test_implicit_and_explicit_conv_routes_agree(stride, dilation, padding):
         assert rel_fro(a, to_np(b)) <= 1e-3, what
 
 
+@pytest.mark.parametrize("dropout", [True, False])
+def test_conv_backward_takes_an_expanded_gradient(dropout):
+    """out.sum().backward() hands the backward a gradient with all strides zero; it must be laid out before the
+    kernels see it (the result is then the gradient of the sum: compare with a materialised gradient of ones)."""
+    import flash_dropout.functional as F
+
+    gen = torch.Generator().manual_seed(3)
+    x = torch.randn(4, 16, 16, 16, generator=gen).half().cuda()
+    k = (torch.randn(64, 16, 3, 3, generator=gen) * 0.08).half().cuda()
+    mask = (torch.rand(16, 3, generator=gen) < 0.5).cuda()
+    grads = []
+    for expanded in (True, False):
+        xg, kg = x.clone().requires_grad_(), k.clone().requires_grad_()
+        if dropout:
+            out = F.blockwise_dropout_conv2d_mask(xg, mask, 64, 0.5, kg, padding=(1, 1))
+        else:
+            out = F.im2col_conv2d(xg, kg, padding=(1, 1), stride=(1, 1), dilation=(1, 1))
+        if expanded:
+            out.sum().backward()
+        else:
+            out.backward(torch.ones_like(out))
+        grads.append((xg.grad, kg.grad))
+    assert torch.equal(grads[0][0], grads[1][0]) and torch.equal(grads[0][1], grads[1][1])
+    assert grads[0][0].abs().sum().item() > 0
+
+
 def test_dense_im2col_conv_matches_conv2d():
     """The reference's implied check for its im2col path: equal to F.conv2d (benchmark/conv.py:20-75)."""
     import flash_dropout.functional as F
