@@ -727,9 +727,10 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
 // column blocks, chosen greedily along the row so that it has at most GW column blocks with anything
 // kept and at most 16 kept tiles: 4 + 6 operand tiles per step for about 12 kept tiles at p = 0.5, the
 // same 4 + 4 for 16 as the patch kernel at p = 0.  Column blocks with nothing kept in these 4 rows
-// cost nothing (zeros are stored for them).  Group boundaries depend on the mask, so every workgroup of
-// a row quad repeats the same scan over the quad's per-column keep flags and takes the group whose index
-// it was launched with (the grid has the worst case ceil(Cb/4) groups per quad; surplus workgroups exit).
+// cost nothing (zeros are stored for them).  Group boundaries depend on the mask, so a workgroup is launched for
+// (window of 4 * GW column blocks, index of the group inside it), scans the quad's keep flags of that window and
+// takes the group with its index (the grid has the worst case number of groups per window; surplus workgroups
+// exit).  Groups never straddle a window, which keeps the workgroups of different row quads on the same W tiles.
 // A wave owns up to two WHOLE kept tiles (tile t of the group goes to wave t%8, so the two waves of a
 // SIMD always carry equal work +-1): 2x2 MFMAs per 16-wide step from 2 + 2 fragments, accumulators
 // statically indexed by the wave's slot, operand tiles addressed dynamically.
@@ -747,6 +748,11 @@ struct SddShape {
   static constexpr int STAGE = (R + GW) * TILE;
   static constexpr int SMEM = 2 * STAGE;
   static constexpr int MINCOLS = GW < MAXT / R ? GW : MAXT / R;  // column blocks a group is sure to cover
+  // Groups never straddle a multiple of WINDOW column blocks, and a workgroup is launched for (window, group in
+  // the window): whatever the masks of two row quads, their workgroups of one window need the same W tiles, so
+  // the quads that share an XCD find each other's W tiles in its L2.
+  static constexpr int WINDOW = 4 * GW;
+  static constexpr int GPW = WINDOW / MINCOLS;  // groups a whole window can have at most
 };
 using SddBig = SddShape<4, 6, 2>;
 using SddMid = SddShape<2, 4, 1>;
@@ -790,32 +796,36 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
 
   // ---- the group this workgroup was launched for ---------------------------------------------------------
   if (wave == 0) {
-    int grp = 0, start = 0, width = 0, cnt = 0, lo = -1, hi = -1;
-    for (int base = 0; base < Cb && hi < 0; base += 64) {
-      const uint32_t fv = (base + lane < Cb) ? flags[base + lane] : 0u;
-      const int lim = Cb - base < 64 ? Cb - base : 64;
-      for (int i = 0; i < lim; ++i) {
+    // whole windows, the last one taking the remainder as well (so that the grid is as large as without windows)
+    const int nwin = Cb / G::WINDOW > 1 ? Cb / G::WINDOW : 1;
+    const int win = gi / G::GPW < nwin - 1 ? gi / G::GPW : nwin - 1, want = gi - win * G::GPW;
+    const int w_lo = win * G::WINDOW, w_hi = win == nwin - 1 ? Cb : w_lo + G::WINDOW;
+    int grp = 0, start = w_lo, width = 0, cnt = 0, lo = -1, hi = -1;
+    static_assert(2 * G::WINDOW <= 64, "a window's flags are read by one wave-wide load");
+    if (w_hi - w_lo <= 64) {
+      const uint32_t fv = (w_lo + lane < w_hi) ? flags[w_lo + lane] : 0u;
+      for (int i = 0; i < w_hi - w_lo; ++i) {
         const uint32_t f = (uint32_t)__builtin_amdgcn_readlane((int)fv, i);
         if (f == 0) continue;
         const int a = __builtin_popcount(f);
         if (width == GW || cnt + a > G::MAXT) {  // the group ends in front of this column block
-          if (grp == gi) {
+          if (grp == want) {
             lo = start;
-            hi = base + i;
+            hi = w_lo + i;
             break;
           }
           ++grp;
-          start = base + i;
+          start = w_lo + i;
           width = 0;
           cnt = 0;
         }
         ++width;
         cnt += a;
       }
-    }
-    if (hi < 0 && grp == gi) {  // the last group runs to the end of the row
-      lo = start;
-      hi = Cb;
+      if (hi < 0 && grp == want) {  // the window's last group runs to its end
+        lo = start;
+        hi = w_hi;
+      }
     }
     int n = 0;
     uint32_t kept = 0;  // bit 4*j + r
