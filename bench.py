@@ -33,9 +33,9 @@ PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA peak
 # (profiles/bench_8192_p50_pmc.txt: read factor 2.0, write factor 1.0).  Only reported when the
 # benchmark runs that workload; a counter run cannot be made from inside this process.
 MEASURED_TRAFFIC_BYTES = {
-    "dsd_forward": int((1041.4 + 130.1) * 2**20),
-    "sdd_dx": int((1744.4 + 128.3) * 2**20),
-    "dsd_dw": int((1154.3 + 143.5) * 2**20),
+    "dsd_forward": int((1034.2 + 129.8) * 2**20),
+    "sdd_dx": int((2087.1 + 128.6) * 2**20),
+    "dsd_dw": int((1159.2 + 144.2) * 2**20),
 }
 METRIC = "fwd+bwd ms & effective TFLOP/s vs p (0–0.75) at 8192³ fp16; % of MFMA peak"
 
