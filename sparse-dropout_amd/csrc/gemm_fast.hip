@@ -1154,11 +1154,17 @@ int launch_sdd_shape(const GemmArgs& g, hipStream_t stream) {
   return check_launch("sdd_group_kernel");
 }
 
-// the big shape when its grid (at p = 0: a workgroup per 4 x 4 tiles) gives more than half of the CUs a workgroup
+// the big shape when its grid (a workgroup per 4 x 4 tiles, per 4 x 6 at high drop rates) gives more than half of
+// the CUs a workgroup
 template <typename T, bool EDGE>
 int launch_sdd_group(const GemmArgs& g, hipStream_t stream) {
   const int64_t Mb = (g.M + BS - 1) / BS, Cb = (g.N + BS - 1) / BS;
-  const int64_t big = ((Mb + 3) / 4) * ((Cb + 3) / 4);
+  // workgroups the big shape would have: a group spans 4 column blocks with everything kept, 6 once few enough tiles
+  // are kept for the width and not the tile count to end a group (measured: worth counting that way from p = 0.7);
+  // callers pass scale = 1 / (1 - p), which is the only hint of the kept fraction the host has
+  const float keep = (g.row_ptr && g.scale > 1.f) ? 1.f / g.scale : 1.f;
+  const int64_t cols = keep <= 0.3f ? SddBig::GW : SddBig::MINCOLS;
+  const int64_t big = ((Mb + 3) / 4) * ((Cb + cols - 1) / cols);
   const int policy = tile_policy.load(std::memory_order_relaxed);
   const bool mid = policy == kTileMid || (policy == kTileAuto && big <= 128);
   return mid ? launch_sdd_shape<T, EDGE, SddMid>(g, stream) : launch_sdd_shape<T, EDGE, SddBig>(g, stream);
