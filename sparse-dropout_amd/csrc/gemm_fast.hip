@@ -1030,7 +1030,7 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
         __builtin_amdgcn_sched_barrier(0);
         mfma_unit(std::integral_constant<int, 0>{}, u);
         __builtin_amdgcn_sched_barrier(0);
-        if (u == 1 && mid) issue_loads(step + 1, stage ^ 1);
+        if (u == 2 && mid) issue_loads(step + 1, stage ^ 1);
       }
       if constexpr (SLOTS == 2) {
         if (act[1]) {
