@@ -186,6 +186,25 @@ int sd_gemm_sdd(const void* A, int64_t a_stride_r, int64_t a_stride_c,
                 int64_t M, int64_t N, int64_t K, int64_t block_size, float scale, int dtype,
                 void* workspace, int64_t workspace_bytes, void* stream);
 
+/* sd_gemm_dsd without a workspace argument and without any allocation: the kept-block list is built into an
+ * array in device memory that is part of the library image (SD_NOALLOC_SCRATCH_BYTES; every GPU the library is
+ * used on holds its own copy until the process ends).  No counterpart in the reference; it is for callers that
+ * cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  Same arguments, results and errors as sd_gemm_dsd otherwise, except that the reduction is never
+ * split over workgroups (there is no scratch for partial tiles).  Limits: round16(sd_workspace_bytes(grid)) of
+ * the 64-granular block grid must fit the array, i.e. about 2^18 mask blocks (a 32768 x 32768 operand at block
+ * size 64); larger operands return SD_ERR_INVALID and launch nothing.  Nothing in the array has to start at
+ * zero (the list builder writes every entry the product reads), but all calls on one GPU share it: calls that
+ * overlap on one GPU (two streams, two host threads) race on the list and must be serialised by the caller. */
+#define SD_NOALLOC_SCRATCH_BYTES 1114112 /* 16-byte padded row_ptr of up to 16383 row blocks + 2^18 int32 */
+int64_t sd_noalloc_scratch_bytes(void);
+int sd_gemm_dsd_noalloc(const void* A, int64_t a_stride_r, int64_t a_stride_c,
+                        const void* B, int64_t b_stride_r, int64_t b_stride_c,
+                        void* C, int64_t c_stride_r, int64_t c_stride_c,
+                        const uint8_t* mask, int64_t mask_stride_r, int64_t mask_stride_c,
+                        int64_t M, int64_t N, int64_t K, int64_t block_size, float scale, int dtype,
+                        void* stream);
+
 int sd_gemm_dsd_lists(const void* A, int64_t a_stride_r, int64_t a_stride_c,
                       const void* B, int64_t b_stride_r, int64_t b_stride_c,
                       void* C, int64_t c_stride_r, int64_t c_stride_c,

@@ -35,6 +35,9 @@ SIGNATURES = {
     "sd_gemm": (c_int, [*_mat, *_mat, *_mat, c_int64, c_int64, c_int64, c_int, c_void_p, c_int64, c_void_p]),
     "sd_gemm_dsd": (c_int, [*_mat, *_mat, *_mat, *_mat, c_int64, c_int64, c_int64, c_int64,
                             c_float, c_int, c_void_p, c_int64, c_void_p]),
+    "sd_noalloc_scratch_bytes": (c_int64, []),
+    "sd_gemm_dsd_noalloc": (c_int, [*_mat, *_mat, *_mat, *_mat, c_int64, c_int64, c_int64, c_int64,
+                                    c_float, c_int, c_void_p]),
     "sd_gemm_sdd": (c_int, [*_mat, *_mat, *_mat, *_mat, c_int64, c_int64, c_int64, c_int64,
                             c_float, c_int, c_void_p, c_int64, c_void_p]),
     "sd_gemm_dsd_lists": (c_int, [*_mat, *_mat, *_mat, c_void_p, c_void_p, c_int64, c_int64,

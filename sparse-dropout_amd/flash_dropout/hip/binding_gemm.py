@@ -231,6 +231,20 @@ class GEMM:
         (reference: binding_gemm.py:29-37)."""
         return self._masked(self.lib.sd_gemm_dsd, "K", A, B, mask, block_size, scale, out, transposed_out)
 
+    def gemm_dsd_noalloc(self, A, B, mask, block_size, scale, out: torch.Tensor) -> torch.Tensor:
+        """:meth:`gemm_dsd` into the caller's ``out`` through the entry point that allocates nothing: the
+        kept-block list goes into an array inside the library (about 2**18 mask blocks at most), so calls
+        that overlap on one GPU race on it."""
+        self._check_pair(A, B)
+        bs = _block_size(block_size)
+        M, N, K = A.shape[0], B.shape[0], A.shape[1]
+        mask = _check_mask(mask, (ceil(M / bs), ceil(K / bs)), A)
+        C = self._out(A, B, out, False)
+        with _guard(A.device):
+            self._call(self.lib.sd_gemm_dsd_noalloc, *_mat(A), *_mat(B), *_mat(C), mask.data_ptr(),
+                       *_mask_strides(mask), M, N, K, bs, float(scale), _DTYPES[A.dtype], self._stream(A))
+        return C
+
     def gemm_sdd(self, A, B, mask, block_size, scale, out=None, transposed_out=False) -> torch.Tensor:
         """``scale * (A @ B.T) ⊙ keep`` with ``mask`` [ceil(M/bs), ceil(N/bs)] over the output; dropped
         tiles are written as zeros (reference: binding_gemm.py:39-47)."""
