@@ -6,13 +6,15 @@
 // one 256x64 tile of W (shared by everybody) and the 64x64 X tiles of just the row blocks that keep
 // this K block, and issues MFMAs only for those.  The 8 waves are (column slice ns = wave%4) x
 // (row-block pair rh = wave/4): a wave multiplies its 64-column slice of the W tile (held in
-// registers for the step) with each kept X tile of its pair.  Waves w and w+4 land on the same SIMD,
+// registers for the step) with each kept X tile of its pair, in v_mfma_f32_16x16x32 tiles (measured on
+// N(0,1) operands, where the clock is power-limited, that instruction sustains about 17 % more FLOP/s than
+// v_mfma_f32_32x32x16).  Waves w and w+4 land on the same SIMD,
 // so every SIMD sees exactly (#kept row blocks) x 64x64x64 of MFMA work per step whatever the mask
 // looks like: dropped blocks cost neither loads nor MFMAs and no wave idles behind a barrier.
 //
 // Global->LDS goes through global_load_lds_dwordx4 (no VGPR staging), two stages, one barrier per
 // step.  A tile row is 128 B (64 halfs) and its 16-byte chunks are XOR-swizzled with (row>>1)&7,
-// which makes the MFMA fragment reads (ds_read_b128, 32 rows x one chunk per half-wave) hit all
+// which makes the MFMA fragment reads (ds_read_b128, 16 rows x one chunk per 16-lane group) hit all
 // 64 LDS banks; the swizzle is applied on the global side (which chunk a lane fetches), because the
 // LDS side of a direct load is fixed at lane*16.
 //
@@ -49,7 +51,7 @@ constexpr int MAX_STEPS = 1024;
 // step table: one uint32 per step of the union walk, reduction block | keep flags << 16, followed by
 // STEP_PAD zero entries so that look-ahead reads past the end are harmless
 constexpr int STEP_PAD = 4;
-// Shape of a DSD workgroup: RH groups of RW row blocks x NS column slices of NT 32-column MFMA tiles; wave
+// Shape of a DSD workgroup: RH groups of RW row blocks x NS column slices of NT * 32 columns; wave
 // (rh, ns) multiplies its slice of the W tile with the kept X tiles of its RW row blocks.  Waves (rh, ns)
 // with equal ns share a SIMD, so a SIMD's MFMA work per step depends on how many row blocks keep the K
 // block, not on which.
@@ -140,6 +142,14 @@ __device__ inline u32x2 lds_read_tr(const char* p) {
   s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p);
   return __builtin_bit_cast(u32x2, v);
 }
+
+// Chunk swizzles of tiles kept in memory order [reduction row][columns] (read with ds_read_b64_tr_b16).  One
+// transposing read takes, per 16-lane group, 4 consecutive reduction rows x 32 bytes, and the groups of a wave
+// are 8 reduction rows apart.  A 64-column tile has rows of 128 B: rows r and r+2 would share banks, so bit 2 of
+// the 16-byte chunk index follows bit 1 of the row; rows 8 apart would too, so bit 1 follows bit 3 of the row.
+// Rows of a 256- or 128-column tile are a multiple of 256 B apart: chunk bits 2-3 follow the row's low two bits.
+__device__ inline int swz_x(int row) { return (((row >> 1) & 1) << 2) ^ (((row >> 3) & 1) << 1); }
+__device__ inline int swz_w(int row) { return ((row & 3) << 2) ^ (((row >> 3) & 1) << 1); }
 
 // TRANS = false: A[row][red], B[col][red] with the reduction index contiguous (forward / dense)
 // TRANS = true : A and B are given as transposed views, the reduction index is the strided one (dW)
@@ -387,7 +397,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   };
   // this thread's 16 bytes of the tile [64 positions][64 columns of row block r] from a step's copy
   [[maybe_unused]] auto gather_tile_t = [&](int r, const uint16_t* copy, char* tile) {
-    const int lc = gat_pc ^ (((gat_row >> 1) & 1) << 2);  // logical chunk: columns r*64 + lc*8 .. +7 of the workgroup
+    const int lc = gat_pc ^ swz_x(gat_row);  // logical chunk: columns r*64 + lc*8 .. +7 of the workgroup
     const u16x8 off = *reinterpret_cast<const u16x8*>(ktab + r * BS + lc * 8);
     const char* pb = reinterpret_cast<const char*>(copy) + gat_base[0];
     uint32_t v[8];
@@ -409,33 +419,32 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   };
 
   // ---- per-lane constants ---------------------------------------------------------------------
-  // fragment reads
-  int a_off[4], b_off[4];  // byte offsets inside an X tile / the W tile, per 16-wide reduction step
+  // fragment reads for v_mfma_f32_16x16x32: lane l supplies row (column of C) l%16 of its operand and the 8
+  // reduction elements 8*(l/16) .. +7 of a 32-wide reduction step kk
+  int a_off[2], b_off[2];  // byte offsets inside an X tile / the W tile, per reduction step; 16-row tile 0
   if (!TRANS) {
-    // rows of 128 B; lane -> tile row lane%32 (+32*tile), logical 16 B chunk 2*ks + lane/32,
-    // physical chunk = logical ^ ((row>>1)&7)
-    const int fr_row = lane % 32;
+    // rows of 128 B; lane -> tile row lane%16 (+16*tile), logical 16 B chunk 4*kk + lane/16,
+    // physical chunk = logical ^ ((row>>1)&7): 16 consecutive lanes hit all 64 banks once
+    const int fr_row = lane % 16;
     const int fr_sw = (lane >> 1) & 7;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const int ko = ((2 * ks + lane / 32) ^ fr_sw) * 16;
-      a_off[ks] = fr_row * 128 + ko;
-      b_off[ks] = (ns * 32 * NT + fr_row) * 128 + ko;
+    for (int kk = 0; kk < 2; ++kk) {
+      const int ko = ((4 * kk + lane / 16) ^ fr_sw) * 16;
+      a_off[kk] = fr_row * 128 + ko;
+      b_off[kk] = (ns * 32 * NT + fr_row) * 128 + ko;
     }
   } else {
     // rows are reduction indices.  16-lane group b = lane/16, lane = 16b + 4e + j reads 8 bytes of
-    // row (8*(b/2) + e) [+16*ks, +4 for the second half], columns 16*(b%2) + 4j .. +3 [+32*tile].
+    // row (8*b + e) [+32*kk, +4 for the second half], columns 4j .. +3 [+16*tile].
     const int b4 = lane / 16, e = (lane % 16) / 4, j = lane % 4;
-    const int row = 8 * (b4 / 2) + e;
-    const int colchunk = 2 * (b4 % 2) + j / 2;  // 16 B chunk inside a 32-column tile
-    // X tile rows are 128 B (8 chunks): physical chunk = logical ^ (((row>>1)&1)<<2)
-    const int a_ch = colchunk ^ (((e >> 1) & 1) << 2);
-    // W tile rows are 2*BN bytes (32 or 16 chunks): physical chunk = logical ^ ((row&3)<<2)
-    const int b_ch = (ns * 4 * NT + colchunk) ^ (e << 2);
+    const int row = 8 * b4 + e;
+    // X tile rows are 128 B (8 chunks), W tile rows 2*BN bytes (32 or 16 chunks); see swz_x / swz_w
+    const int a_ch = (j / 2) ^ swz_x(row);
+    const int b_ch = (ns * 4 * NT + j / 2) ^ swz_w(row);
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      a_off[ks] = (16 * ks + row) * 128 + a_ch * 16 + (j % 2) * 8;
-      b_off[ks] = (16 * ks + row) * (2 * BN) + b_ch * 16 + (j % 2) * 8;
+    for (int kk = 0; kk < 2; ++kk) {
+      a_off[kk] = (32 * kk + row) * 128 + a_ch * 16 + (j % 2) * 8;
+      b_off[kk] = (32 * kk + row) * (2 * BN) + b_ch * 16 + (j % 2) * 8;
     }
   }
 
@@ -494,7 +503,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
 #pragma unroll
     for (int jj = 0; jj < BL; ++jj) {
       const int row = (wave * BL + jj) * (64 / CPR) + lane / CPR;
-      const int col = ((lane % CPR) ^ ((row & 3) << 2)) * 8;
+      const int col = ((lane % CPR) ^ swz_w(row)) * 8;
       b_lane[jj] = (uint32_t)(row * g.b.sc + col) * 2u;
       b_valid[jj] = col < nvalid;
       const int rc = (kb_tail >= 0 && row >= k_valid) ? k_valid - 1 : row;
@@ -502,7 +511,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
     }
     auto chunk_at = [&](int row, bool clamp_m, bool clamp_k) {
       const int rc = (clamp_k && row >= k_valid) ? k_valid - 1 : row;
-      int c = (lane % 8) ^ (((row >> 1) & 1) << 2);
+      int c = (lane % 8) ^ swz_x(row);
       if (clamp_m && c * 8 >= m_valid) c = 0;
       return (uint32_t)(rc * g.a.sc + c * 8) * 2u;
     };
@@ -553,92 +562,94 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
         }
       }
   };
-  // zeroes the elements of a fragment whose reduction index (16*ks + 8*(lane/32) + 0..7 inside the
+  // zeroes the elements of a fragment whose reduction index (32*kk + 8*(lane/16) + 0..7 inside the
   // block) is not below k_valid
-  auto mask_fragment = [&](u32x4& f, int ks) {
-    const int n = k_valid - (16 * ks + 8 * (lane / 32));  // valid elements among the lane's 8
+  auto mask_fragment = [&](u32x4& f, int kk) {
+    const int n = k_valid - (32 * kk + 8 * (lane / 16));  // valid elements among the lane's 8
     f.x &= n >= 2 ? ~0u : (n == 1 ? 0xffffu : 0u);
     f.y &= n >= 4 ? ~0u : (n == 3 ? 0xffffu : 0u);
     f.z &= n >= 6 ? ~0u : (n == 5 ? 0xffffu : 0u);
     f.w &= n >= 8 ? ~0u : (n == 7 ? 0xffffu : 0u);
   };
 
-  f32x16 acc[RW][2][NT];  // [row block of the wave][m tile][n tile]
+  constexpr int NT16 = 2 * NT;  // 16-column MFMA tiles of the wave's column slice
+  f32x4 acc[RW][4][NT16];  // [row block of the wave][16-row tile][16-column tile]
 #pragma unroll
   for (int a = 0; a < RW; ++a)
 #pragma unroll
-    for (int b = 0; b < 2; ++b)
+    for (int b = 0; b < 4; ++b)
 #pragma unroll
-      for (int c = 0; c < NT; ++c)
+      for (int c = 0; c < NT16; ++c)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[a][b][c][v] = 0.f;
+        for (int v = 0; v < 4; ++v) acc[a][b][c][v] = 0.f;
 
-  // fragment reads for one 16-wide reduction step ks: both 32-row tiles of an X tile / of the W slice
-  auto read_a = [&](const char* at, int ks, u32x4 (&dst)[2]) {
+  // fragment reads for one 32-wide reduction step kk: the four 16-row tiles of an X tile / the 16-column
+  // tiles of the W slice
+  auto read_a = [&](const char* at, int kk, u32x4 (&dst)[4]) {
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
+    for (int mt = 0; mt < 4; ++mt) {
       if (!TRANS) {
-        dst[mt] = *reinterpret_cast<const u32x4*>(at + a_off[ks] + mt * 32 * 128);
+        dst[mt] = *reinterpret_cast<const u32x4*>(at + a_off[kk] + mt * 16 * 128);
       } else {
-        // the 32-column tile toggles bit 2 of the chunk index, i.e. 64 bytes, under the XOR swizzle
-        const char* p = at + (a_off[ks] ^ (mt * 64));
+        // the 16-column tile sits in bits 1-2 of the chunk index, i.e. 32 bytes, under the XOR swizzle
+        const char* p = at + (a_off[kk] ^ (mt * 32));
         const u32x2 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * 128);
         dst[mt] = u32x4{lo.x, lo.y, hi.x, hi.y};
       }
     }
   };
-  auto read_b = [&](const char* st, int ks, u32x4 (&dst)[NT][4]) {
+  auto read_b = [&](const char* st, int kk, u32x4 (&dst)[NT16][2]) {
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
+    for (int nt = 0; nt < NT16; ++nt) {
       if (!TRANS) {
-        dst[nt][ks] = *reinterpret_cast<const u32x4*>(st + b_off[ks] + nt * 32 * 128);
+        dst[nt][kk] = *reinterpret_cast<const u32x4*>(st + b_off[kk] + nt * 16 * 128);
       } else {
-        const char* p = st + (b_off[ks] ^ (nt * 64));
+        const char* p = st + (b_off[kk] ^ (nt * 32));
         const u32x2 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * 2 * BN);
-        dst[nt][ks] = u32x4{lo.x, lo.y, hi.x, hi.y};
+        dst[nt][kk] = u32x4{lo.x, lo.y, hi.x, hi.y};
       }
     }
   };
 
   // One step of MFMA work for this wave, specialised on which of its two row blocks keep the K block
-  // (MINE = 1, 2 or 3).  The work is a chain of units (row block, ks); the LDS reads of unit u+1 are
-  // issued before the MFMAs of unit u so that their latency hides behind 4 MFMAs (128 cycles).  The W
+  // (MINE = 1, 2 or 3).  The work is a chain of units (row block, kk); the LDS reads of unit u+1 are
+  // issued before the MFMAs of unit u so that their latency hides behind 4 * NT16 MFMAs.  The W
   // fragments are read during the first row block's units and stay in registers for the second.
   auto compute = [&](auto mine_c, const char* st, bool mid_loads, uint32_t mid_entry, int mid_stage,
                      bool red_tail) {
     constexpr int MINE = decltype(mine_c)::value;
     constexpr int NR = (MINE == 3) ? 2 : 1;
     constexpr int R0 = (MINE == 2) ? 1 : 0;
-    u32x4 bf[NT][4];
+    u32x4 bf[NT16][2];
     const char* at0 = st + A_OFF + (RW * rh + R0) * TILE;
-    u32x4 af[2][2];
+    u32x4 af[2][4];
     read_b(st, 0, bf);
     read_a(at0, 0, af[0]);
 #pragma unroll
-    for (int u = 0; u < NR * 4; ++u) {
-      const int rr = R0 + u / 4, ks = u % 4;
-      if (u + 1 < NR * 4) {
-        const int ks1 = (u + 1) % 4;
-        if (u + 1 < 4) read_b(st, ks1, bf);
-        read_a(at0 + ((u + 1) / 4) * TILE, ks1, af[(u + 1) & 1]);
+    for (int u = 0; u < NR * 2; ++u) {
+      const int rr = R0 + u / 2, kk = u % 2;
+      if (u + 1 < NR * 2) {
+        const int kk1 = (u + 1) % 2;
+        if (u + 1 < 2) read_b(st, kk1, bf);
+        read_a(at0 + ((u + 1) / 2) * TILE, kk1, af[(u + 1) & 1]);
       }
       __builtin_amdgcn_sched_barrier(0);
       if (RAGGED && red_tail) {  // ragged reduction block: nothing past the end may reach the MFMAs
-        mask_fragment(af[u & 1][0], ks);
-        mask_fragment(af[u & 1][1], ks);
-        if (u < 4) {
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt) mask_fragment(bf[nt][ks], ks);
+        for (int mt = 0; mt < 4; ++mt) mask_fragment(af[u & 1][mt], kk);
+        if (u < 2) {
+#pragma unroll
+          for (int nt = 0; nt < NT16; ++nt) mask_fragment(bf[nt][kk], kk);
         }
       }
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
+      for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          acc[rr][mt][nt] = CM ? T::mfma32(bf[nt][ks], af[u & 1][mt], acc[rr][mt][nt])
-                               : T::mfma32(af[u & 1][mt], bf[nt][ks], acc[rr][mt][nt]);
+        for (int nt = 0; nt < NT16; ++nt)
+          acc[rr][mt][nt] = CM ? T::mfma16(bf[nt][kk], af[u & 1][mt], acc[rr][mt][nt])
+                               : T::mfma16(af[u & 1][mt], bf[nt][kk], acc[rr][mt][nt]);
       __builtin_amdgcn_sched_barrier(0);
-      if (u == NR * 2 - 1 && mid_loads) issue_loads(mid_entry, mid_stage);
+      if (u == NR - 1 && mid_loads) issue_loads(mid_entry, mid_stage);
     }
   };
 
@@ -691,7 +702,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   }
 
   // ---- epilogue: scale, round once, store ---------------------------------------------------------
-  // accumulator register v of lane l is element (8*(v/4) + 4*(l/32) + v%4, l%32) of the 32x32 product
+  // accumulator register v of lane l is element (4*(l/16) + v, l%16) of the 16x16 product
   // (first MFMA operand's rows) x (second operand's rows); lanes run along C's contiguous index.
   if (ns * 32 * NT >= nvalid) return;  // this wave's column slice overhangs N: nothing of it is stored
   float* part = nsplit > 1 ? g.ws + (int64_t)split * g.M * g.N : nullptr;
@@ -700,15 +711,15 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
     const int rb = rb0 + RW * rh + rr;
     if (rb >= Mb) continue;
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
+    for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
+      for (int nt = 0; nt < NT16; ++nt)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int reg_i = 8 * (v / 4) + 4 * (lane / 32) + (v % 4);
-          const int lane_i = lane % 32;
-          const int64_t m = (int64_t)rb * BS + mt * 32 + (CM ? lane_i : reg_i);
-          const int64_t n = n0 + ns * 32 * NT + nt * 32 + (CM ? reg_i : lane_i);
+        for (int v = 0; v < 4; ++v) {
+          const int reg_i = 4 * (lane / 16) + v;
+          const int lane_i = lane % 16;
+          const int64_t m = (int64_t)rb * BS + mt * 16 + (CM ? lane_i : reg_i);
+          const int64_t n = n0 + ns * 32 * NT + nt * 16 + (CM ? reg_i : lane_i);
           if (RAGGED && (m >= g.M || n >= g.N)) continue;  // ragged last row block / column slice
           if (part)  // unscaled fp32 partial in C's own element order; the reduce pass scales and rounds
             part[CM ? n * g.M + m : m * g.N + n] = acc[rr][mt][nt][v];
@@ -890,16 +901,18 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
   __syncthreads();  // flags and rec are dead: the stages may be written
 
   // ---- per-lane constants -----------------------------------------------------------------------------
-  int a_off[4], b_off[4];
+  // fragments of v_mfma_f32_16x16x32 per 32-wide reduction step kk (see dsd_kernel): dY tiles are
+  // reduction-contiguous (b128 reads), W tiles reduction-strided (transposing reads)
+  int a_off[2], b_off[2];
   {
     const int fr_sw = (lane >> 1) & 7;
     const int b4 = lane / 16, e = (lane % 16) / 4, j = lane % 4;
-    const int row = 8 * (b4 / 2) + e;
-    const int b_ch = (2 * (b4 % 2) + j / 2) ^ (((e >> 1) & 1) << 2);
+    const int row = 8 * b4 + e;
+    const int b_ch = (j / 2) ^ swz_x(row);
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      a_off[ks] = (lane % 32) * 128 + ((2 * ks + lane / 32) ^ fr_sw) * 16;  // + 32*128 for the second 32 rows
-      b_off[ks] = (16 * ks + row) * 128 + b_ch * 16 + (j % 2) * 8;           // ^ 64 for the second 32 columns
+    for (int kk = 0; kk < 2; ++kk) {
+      a_off[kk] = (lane % 16) * 128 + ((4 * kk + lane / 16) ^ fr_sw) * 16;  // + 16*128 per 16-row tile
+      b_off[kk] = (32 * kk + row) * 128 + b_ch * 16 + (j % 2) * 8;           // ^ 32 per 16-column tile
     }
   }
   const int nsteps = (int)((g.K + BS - 1) / BS);
@@ -927,7 +940,7 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
     };
     auto b_at = [&](bool clamp_c, bool clamp_k) {  // rows of a W tile are reduction indices
       const int rc = (clamp_k && row >= k_valid) ? k_valid - 1 : row;
-      int c = pch ^ (((row >> 1) & 1) << 2);
+      int c = pch ^ swz_x(row);
       if (clamp_c && c * 8 >= n_valid) c = 0;
       return (uint32_t)(rc * g.b.sc + c * 8) * 2u;
     };
@@ -960,10 +973,10 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
         load16_to_lds(bp + (int64_t)cols[j] * (BS * 2), off, st + G_BOFF + j * TILE);
       }
   };
-  // zeroes the elements of a fragment whose reduction index (16*ks + 8*(lane/32) + 0..7 inside the
+  // zeroes the elements of a fragment whose reduction index (32*kk + 8*(lane/16) + 0..7 inside the
   // block) is not below k_valid
-  auto mask_fragment = [&](u32x4& f, int ks) {
-    const int n = k_valid - (16 * ks + 8 * (lane / 32));
+  auto mask_fragment = [&](u32x4& f, int kk) {
+    const int n = k_valid - (32 * kk + 8 * (lane / 16));
     f.x &= n >= 2 ? ~0u : (n == 1 ? 0xffffu : 0u);
     f.y &= n >= 4 ? ~0u : (n == 3 ? 0xffffu : 0u);
     f.z &= n >= 6 ? ~0u : (n == 5 ? 0xffffu : 0u);
@@ -972,15 +985,15 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
   // the two waves of a SIMD (w and w + 4) issue their loads half a step apart
   const bool late = wave >= 4;
 
-  f32x16 acc[SLOTS][2][2];  // [slot][32-row half][32-column half]
+  f32x4 acc[SLOTS][4][4];  // [slot][16-row tile][16-column tile]
 #pragma unroll
   for (int k = 0; k < SLOTS; ++k)
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+    for (int a = 0; a < 4; ++a)
 #pragma unroll
-      for (int b = 0; b < 2; ++b)
+      for (int b = 0; b < 4; ++b)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[k][a][b][v] = 0.f;
+        for (int v = 0; v < 4; ++v) acc[k][a][b][v] = 0.f;
 
   issue_loads(0, 0);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -993,52 +1006,58 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
     if (more && !mid) issue_loads(step + 1, stage ^ 1);
     if (act[0]) {
       const char* st = smem + stage * G_STAGE;
-      // units u = 4*slot + ks; the fragments of unit u+1 are read before the MFMAs of unit u.  Slot 1's
+      // units u = 2*slot + kk; the fragments of unit u+1 are read before the MFMAs of unit u.  Slot 1's
       // first fragments are read whether it is active or not (its tile indices are valid either way).
-      u32x4 af[2][2], bf[2][2];
+      u32x4 af[2][4], bf[2][4];
       auto read_unit = [&](int u) {
-        const int k = u / 4, ks = u % 4;
+        const int k = u / 2, kk = u % 2;
         const char* at = st + my_r[k] * TILE;
         const char* bt = st + G_BOFF + my_j[k] * TILE;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          af[u & 1][h] = *reinterpret_cast<const u32x4*>(at + a_off[ks] + h * 32 * 128);
-          const char* p = bt + (b_off[ks] ^ (h * 64));
+        for (int h = 0; h < 4; ++h) {
+          af[u & 1][h] = *reinterpret_cast<const u32x4*>(at + a_off[kk] + h * 16 * 128);
+          const char* p = bt + (b_off[kk] ^ (h * 32));
           const u32x2 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * 128);
           bf[u & 1][h] = u32x4{lo.x, lo.y, hi.x, hi.y};
         }
       };
       const bool red_tail = EDGE && step == s_tail;
-      auto mfma_unit = [&](auto k_c, int u) {
+      // the late waves of slot 0's second unit issue the next step's loads half-way through its MFMAs
+      auto mfma_unit = [&](auto k_c, int u, bool loads_inside) {
         constexpr int k = decltype(k_c)::value;
         if (EDGE && red_tail) {  // nothing past the end of the reduction may reach the MFMAs
 #pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            mask_fragment(af[u & 1][h], u % 4);
-            mask_fragment(bf[u & 1][h], u % 4);
+          for (int h = 0; h < 4; ++h) {
+            mask_fragment(af[u & 1][h], u % 2);
+            mask_fragment(bf[u & 1][h], u % 2);
           }
         }
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
+        for (int mt = 0; mt < 4; ++mt) {
 #pragma unroll
-          for (int nt = 0; nt < 2; ++nt) acc[k][mt][nt] = T::mfma32(af[u & 1][mt], bf[u & 1][nt], acc[k][mt][nt]);
+          for (int nt = 0; nt < 4; ++nt) acc[k][mt][nt] = T::mfma16(af[u & 1][mt], bf[u & 1][nt], acc[k][mt][nt]);
+          if (mt == 1) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (loads_inside) issue_loads(step + 1, stage ^ 1);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
       };
       read_unit(0);
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        if (u + 1 < 4 * SLOTS) read_unit(u + 1);
+      for (int u = 0; u < 2; ++u) {
+        if (u + 1 < 2 * SLOTS) read_unit(u + 1);
         __builtin_amdgcn_sched_barrier(0);
-        mfma_unit(std::integral_constant<int, 0>{}, u);
+        mfma_unit(std::integral_constant<int, 0>{}, u, u == 1 && mid);
         __builtin_amdgcn_sched_barrier(0);
-        if (u == 2 && mid) issue_loads(step + 1, stage ^ 1);
       }
       if constexpr (SLOTS == 2) {
         if (act[1]) {
 #pragma unroll
-          for (int u = 4; u < 8; ++u) {
-            if (u + 1 < 8) read_unit(u + 1);
+          for (int u = 2; u < 4; ++u) {
+            if (u + 1 < 4) read_unit(u + 1);
             __builtin_amdgcn_sched_barrier(0);
-            mfma_unit(std::integral_constant<int, 1>{}, u);
+            mfma_unit(std::integral_constant<int, 1>{}, u, false);
             __builtin_amdgcn_sched_barrier(0);
           }
         }
@@ -1053,13 +1072,13 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
   for (int k = 0; k < SLOTS; ++k) {
     if (!act[k]) continue;
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
+    for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
+      for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int64_t m = (int64_t)(rb0 + my_r[k]) * BS + mt * 32 + 8 * (v / 4) + 4 * (lane / 32) + (v % 4);
-          const int64_t n = (int64_t)my_c[k] * BS + nt * 32 + (lane % 32);
+        for (int v = 0; v < 4; ++v) {
+          const int64_t m = (int64_t)(rb0 + my_r[k]) * BS + mt * 16 + 4 * (lane / 16) + v;
+          const int64_t n = (int64_t)my_c[k] * BS + nt * 16 + (lane % 16);
           if (m < g.M && (!EDGE || n < g.N)) g.c[m * g.c_sr + n] = T::from_float(acc[k][mt][nt][v] * g.scale);
         }
   }
