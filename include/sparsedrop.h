@@ -65,12 +65,30 @@ const char* sd_last_error(void);
  * the fast path.  No counterpart in the reference. */
 const char* sd_last_kernel(void);
 
+/* What that call ran on, in more detail: kernel family, workgroup shape and reduction splits, e.g. "dsd:big splits=1",
+ * "dsd:mid:strided:ragged splits=4", "sdd:mid", "generic", "conv_fwd:implicit:rows-per-step", "conv_dw:implicit
+ * splits=85", "conv_dx:fused".  The conv entry points that return SD_ERR_UNSUPPORTED leave it unchanged (the caller's
+ * explicit route then shows its own GEMM here).  Diagnostic text, not a stable format. */
+const char* sd_last_kernel_detail(void);
+
+/* Hash of the source files the library was built from (written by csrc/build.py); the Python loader compares it
+ * with the tree next to it and refuses a stale library.  No counterpart in the reference. */
+const char* sd_source_hash(void);
+
+/* The workgroup-to-tile map of the specialised kernels, evaluated on the host: launch index `block` of a
+ * tiles_m x tiles_n grid -> (tile_m, tile_n); kind 0 = DSD / dense order, 1 = SDD order.  The hardware deals
+ * consecutive workgroup ids round-robin to the 8 XCDs; the map gives each XCD a compact patch of the grid.  It
+ * must be a bijection onto the grid, which tests check through this entry point; the reference's counterpart is
+ * threadblock_swizzle (flash_dropout/cuda/src/gemm.cuh:84-97). */
+int sd_tile_of_block(int kind, int64_t block, int64_t tiles_m, int64_t tiles_n, int32_t* tile_m, int32_t* tile_n);
+
 /* Workgroup shape of the specialised DSD / dense kernels: SD_TILE_AUTO picks from the shape (256 x 256
  * output tiles when there are more than 128 of them, 128 x 128 otherwise; the SDD kernel's group shape follows the
  * same rule), the other two
  * force one shape for every later call of the process (SD_TILE_BIG also makes sd_conv2d_dsd_lists keep one
  * LDS copy of all channels' input rows instead of a copy per step where both fit).  Returns the previous setting, -1 for an unknown
- * value.  A tuning and test hook; results do not depend on it beyond fp32 summation order.  No
+ * value.  A tuning and test hook, process-global and not thread-safe against concurrent GEMM calls (a call that
+ * races with it runs with either shape); not for production use.  Results do not depend on it beyond fp32 summation order.  No
  * counterpart in the reference (its tile is a compile-time GemmConfig, gemm_configs/gemm_config.cuh:19-100). */
 #define SD_TILE_AUTO 0
 #define SD_TILE_BIG 1
@@ -218,6 +236,17 @@ int sd_gemm_sdd_lists(const void* A, int64_t a_stride_r, int64_t a_stride_c,
                       const int32_t* row_ptr, const int32_t* col_idx,
                       int64_t M, int64_t N, int64_t K, int64_t block_size, float scale, int dtype,
                       void* stream);
+
+/* sd_gemm_sdd_lists with its options spelled out.  kept_only != 0: as sd_gemm_sdd_lists_kept below.  keep_hint: the
+ * caller's estimate of the fraction of blocks kept (1 - p), or negative for unknown; the lists live on the device,
+ * so this is all the host has to choose the workgroup shape by (it counts the workgroups the large shape would
+ * have; unknown counts as everything kept).  It never changes results.  `scale` plays no part in that choice. */
+int sd_gemm_sdd_lists_ex(const void* A, int64_t a_stride_r, int64_t a_stride_c,
+                         const void* B, int64_t b_stride_r, int64_t b_stride_c,
+                         void* C, int64_t c_stride_r, int64_t c_stride_c,
+                         const int32_t* row_ptr, const int32_t* col_idx,
+                         int64_t M, int64_t N, int64_t K, int64_t block_size, float scale, int dtype,
+                         int kept_only, float keep_hint, void* stream);
 
 /* sd_gemm_sdd_lists for a consumer that reads kept tiles only (sd_col2im with the same mask does): the
  * dropped tiles of C are left untouched instead of being written as zeros, which for half of a large C

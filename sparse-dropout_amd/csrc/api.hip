@@ -1,5 +1,6 @@
 // extern "C" surface of libsparsedrop: argument validation and dispatch.  No kernels here.
 #include "common.h"
+#include "tile_map.h"
 
 #include <cstdlib>
 #include <cstring>
@@ -8,6 +9,11 @@ namespace sd {
 
 char* last_error_buf() {
   static thread_local char buf[512] = {0};
+  return buf;
+}
+
+char* kernel_detail_buf() {
+  static thread_local char buf[96] = {0};
   return buf;
 }
 
@@ -101,6 +107,7 @@ GemmArgs make_args(const void* A, int64_t asr, int64_t asc, const void* B, int64
   g.ws = ws_ok ? static_cast<float*>(ws) : nullptr;
   g.ws_bytes = ws_ok ? ws_bytes : 0;
   g.kept_only = false;
+  g.keep_hint = -1.f;
   return g;
 }
 
@@ -148,11 +155,36 @@ static ImplicitConv conv_geometry(const void* x, int64_t sn, int64_t sc, int64_t
 
 extern "C" {
 
-int sd_version(void) { return 100; }
+int sd_version(void) { return 110; }
+
+// build.py writes the hash of the sources this library was compiled from into build/source_hash.inc
+#if __has_include("source_hash.inc")
+#include "source_hash.inc"
+#else
+#define SD_SOURCE_HASH "unknown"
+#endif
+const char* sd_source_hash(void) { return SD_SOURCE_HASH; }
 
 const char* sd_last_error(void) { return last_error_buf(); }
 
 const char* sd_last_kernel(void) { return last_kernel; }
+
+const char* sd_last_kernel_detail(void) { return kernel_detail_buf(); }
+
+int sd_tile_of_block(int kind, int64_t block, int64_t tiles_m, int64_t tiles_n, int32_t* tile_m, int32_t* tile_n) {
+  SD_REQUIRE(kind == 0 || kind == 1, "tile_of_block: kind must be 0 (DSD order) or 1 (SDD order)");
+  SD_REQUIRE(tile_m && tile_n, "tile_of_block: null output");
+  SD_REQUIRE(tiles_m > 0 && tiles_n > 0 && tiles_m * tiles_n < kMaxDim, "tile_of_block: bad grid");
+  SD_REQUIRE(block >= 0 && block < tiles_m * tiles_n, "tile_of_block: block outside the grid");
+  int tm = 0, tn = 0;
+  if (kind == 0)
+    tile_of_block<DSD_GROUP_M>((int)block, (int)tiles_m, (int)tiles_n, tm, tn);
+  else
+    tile_of_block<SDD_GROUP_M>((int)block, (int)tiles_m, (int)tiles_n, tm, tn);
+  *tile_m = tm;
+  *tile_n = tn;
+  return SD_OK;
+}
 
 int sd_set_tile_policy(int policy) { return sd::set_tile_policy(policy); }
 
@@ -261,6 +293,20 @@ int sd_gemm_sdd_lists(const void* A, int64_t asr, int64_t asc, const void* B, in
   if (int rc = check_sparse(bs, scale)) return rc;
   SD_REQUIRE(row_ptr && col_idx, "gemm_sdd: null list");
   GemmArgs g = make_args(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, bs, scale, row_ptr, col_idx);
+  return run(g, kSdd, dtype, (hipStream_t)stream);
+}
+
+int sd_gemm_sdd_lists_ex(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc,
+                         void* C, int64_t csr, int64_t csc, const int32_t* row_ptr, const int32_t* col_idx,
+                         int64_t M, int64_t N, int64_t K, int64_t bs, float scale, int dtype, int kept_only,
+                         float keep_hint, void* stream) {
+  if (int rc = check_common(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, dtype)) return rc;
+  if (int rc = check_sparse(bs, scale)) return rc;
+  SD_REQUIRE(row_ptr && col_idx, "gemm_sdd: null list");
+  SD_REQUIRE(!(keep_hint > 1.f), "gemm_sdd: keep_hint must be a fraction in [0, 1], or negative for unknown");
+  GemmArgs g = make_args(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, bs, scale, row_ptr, col_idx);
+  g.kept_only = kept_only != 0;
+  g.keep_hint = keep_hint == keep_hint ? keep_hint : -1.f;
   return run(g, kSdd, dtype, (hipStream_t)stream);
 }
 

@@ -9,6 +9,7 @@ hipcc cross-compiles for gfx950 without a GPU present.
 from __future__ import annotations
 
 import argparse
+import hashlib
 import os
 import subprocess
 import sys
@@ -33,11 +34,22 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     f"-I{ROOT / 'include'}",
     f"-I{CSRC}",
+    f"-I{OBJ_DIR}",
 ]
 
 
 def sources() -> list[Path]:
     return sorted(CSRC.glob("*.hip"))
+
+
+def source_hash() -> str:
+    """Hash of everything the library is compiled from; the library reports the one it was built with
+    (sd_source_hash) and the loader refuses a library whose sources have changed since."""
+    h = hashlib.sha256()
+    for f in [*sources(), *sorted(CSRC.glob("*.h")), *sorted((ROOT / "include").glob("*.h"))]:
+        h.update(f.name.encode())
+        h.update(f.read_bytes())
+    return h.hexdigest()[:16]
 
 
 def _stale(target: Path, deps: list[Path]) -> bool:
@@ -59,6 +71,11 @@ def build(force: bool = False, verbose: bool = False) -> Path:
     OUT_DIR.mkdir(parents=True, exist_ok=True)
     OBJ_DIR.mkdir(parents=True, exist_ok=True)
     headers = sorted(CSRC.glob("*.h")) + sorted((ROOT / "include").glob("*.h"))
+    inc = OBJ_DIR / "source_hash.inc"
+    line = f'#define SD_SOURCE_HASH "{source_hash()}"\n'
+    if not inc.exists() or inc.read_text() != line:
+        inc.write_text(line)  # newer than api.o: api.hip, which includes it, is recompiled below
+    headers.append(inc)
     jobs = []
     objs = []
     for src in sources():

@@ -22,6 +22,15 @@ inline int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+// Records which kernel (and workgroup shape) the calling thread's last launch used: sd_last_kernel_detail().
+char* kernel_detail_buf();  // thread-local, 96 bytes (api.hip)
+inline void note_kernel(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(kernel_detail_buf(), 96, fmt, ap);
+  va_end(ap);
+}
+
 #define SD_REQUIRE(cond, ...)                                  \
   do {                                                         \
     if (!(cond)) return ::sd::fail(SD_ERR_INVALID, __VA_ARGS__); \
@@ -107,6 +116,7 @@ struct GemmArgs {
   float* ws;         // optional split-K workspace (fp32 partial tiles), may be null
   int64_t ws_bytes;
   bool kept_only;    // SDD: dropped tiles of C are left untouched instead of being zeroed
+  float keep_hint;   // SDD: the caller's estimate of the kept fraction of blocks (picks the workgroup shape); < 0 = unknown
 };
 
 // Geometry of a convolution whose patch matrix the DSD kernel gathers itself (implicit GEMM):

@@ -19,6 +19,8 @@
 // elements that fall in this block from the staging area.  A channel's R*S columns span at most two
 // consecutive blocks, so its sums are carried in a small fp32 ring in LDS and written out once, when its last
 // column has been seen.  Every sum has one owner and a fixed order: the result is deterministic.
+#include <atomic>
+
 #include "common.h"
 
 namespace sd {
@@ -281,17 +283,18 @@ template <typename T, int RT, int ST, int KS_MAX>
 int launch_t(const DxArgs& g, int64_t wgs, hipStream_t stream) {
   const int smem = DxLds<KS_MAX>::OFF_ACC + g.ring_n * g.HB * g.W * 4;
   if (smem > DxLds<KS_MAX>::DYN_LDS_MAX) return SD_ERR_UNSUPPORTED;  // the ring of open channel sums does not fit
-  static bool configured[16] = {};
+  static std::atomic<bool> configured[16] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16)
     return fail(SD_ERR_RUNTIME, "hipGetDevice failed or device index out of range");
-  if (!configured[dev]) {
+  if (!configured[dev].load(std::memory_order_acquire)) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_dx_kernel<T, RT, ST, KS_MAX>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, DxLds<KS_MAX>::DYN_LDS_MAX);
     if (e != hipSuccess) return fail(SD_ERR_RUNTIME, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured[dev] = true;
+    configured[dev].store(true, std::memory_order_release);
   }
   hipLaunchKernelGGL((conv_dx_kernel<T, RT, ST, KS_MAX>), dim3((unsigned)wgs), dim3(THREADS), smem, stream, g);
+  note_kernel("conv_dx:fused");
   return check_launch("conv_dx_kernel");
 }
 

@@ -38,6 +38,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include "tile_map.h"
 
 namespace sd {
 namespace {
@@ -110,28 +111,6 @@ __device__ inline void load16_to_lds(const char* base, uint32_t lane_off, char* 
   const uint32_t a = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_void*)lds_dst);
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(sb), "s"(a)
                : "memory");
-}
-
-// Maps the launch index to an output tile so that the workgroups resident on one XCD (the hardware
-// deals consecutive workgroup ids round-robin over the 8 XCDs, each with its own L2) cover a compact
-// patch of the tile grid: each XCD gets a contiguous run of the tile order, and the order walks
-// GROUP_M tile rows at a time (column by column inside a group).
-// tile rows walked together: 8 for the DSD kernels (their row panels are the sparse, smaller operand),
-// 4 for SDD (8 measured 25 % slower there)
-constexpr int DSD_GROUP_M = 8, SDD_GROUP_M = 4;
-template <int GROUP_M>
-__device__ inline void tile_of_block(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
-  constexpr int XCDS = 8;
-  const int total = tiles_m * tiles_n;
-  const int per = total / XCDS, rem = total % XCDS;
-  const int x = bid % XCDS, i = bid / XCDS;
-  const int lin = x * per + (x < rem ? x : rem) + i;
-  const int group = lin / (GROUP_M * tiles_n);
-  const int first_m = group * GROUP_M;
-  const int gm = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
-  const int in_group = lin - group * GROUP_M * tiles_n;
-  tm = first_m + in_group % gm;
-  tn = in_group / gm;
 }
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -1089,14 +1068,15 @@ bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0;
 // Raises a kernel's dynamic LDS limit once per device (the attribute belongs to the device's copy of the
 // kernel); `done` is the caller's per-kernel record.
 constexpr int kMaxDevices = 64;
-int allow_big_lds(const void* kernel, int bytes, bool (&done)[kMaxDevices]) {
+int allow_big_lds(const void* kernel, int bytes, std::atomic<bool> (&done)[kMaxDevices]) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
     return fail(SD_ERR_RUNTIME, "hipGetDevice failed or device index out of range");
-  if (!done[dev]) {
+  // concurrent first calls may both set the attribute (to the same value): harmless
+  if (!done[dev].load(std::memory_order_acquire)) {
     hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
     if (e != hipSuccess) return fail(SD_ERR_RUNTIME, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    done[dev] = true;
+    done[dev].store(true, std::memory_order_release);
   }
   return SD_OK;
 }
@@ -1105,7 +1085,7 @@ std::atomic<int> tile_policy{0};
 
 template <typename T, bool TRANS, bool CM, bool RAGGED, typename S>
 int launch_dsd_s(const GemmArgs& g, int splits, hipStream_t stream) {
-  static bool configured[kMaxDevices] = {};
+  static std::atomic<bool> configured[kMaxDevices] = {};
   if (int rc = allow_big_lds(reinterpret_cast<const void*>(&dsd_kernel<T, TRANS, CM, RAGGED, S>), S::SMEM_BYTES,
                              configured))
     return rc;
@@ -1114,6 +1094,8 @@ int launch_dsd_s(const GemmArgs& g, int splits, hipStream_t stream) {
   hipLaunchKernelGGL((dsd_kernel<T, TRANS, CM, RAGGED, S>), dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits),
                      dim3(S::THREADS), S::SMEM_BYTES, stream, g, tiles_m, tiles_n, Mb, Kb, ImplicitConv{});
   if (int rc = check_launch("dsd_kernel")) return rc;
+  note_kernel("dsd:%s%s%s splits=%d", S::R * BS == 256 && S::BN == 256 ? "big" : "mid", TRANS ? ":strided" : "",
+              RAGGED ? ":ragged" : "", splits);
   if (splits > 1) return launch_splitk_reduce(g, splits, CM, T::id, stream);
   return SD_OK;
 }
@@ -1163,13 +1145,14 @@ DsdPlan plan_dsd(int64_t M, int64_t N, int64_t K) {
 
 template <typename T, bool EDGE, typename G>
 int launch_sdd_shape(const GemmArgs& g, hipStream_t stream) {
-  static bool configured[kMaxDevices] = {};
+  static std::atomic<bool> configured[kMaxDevices] = {};
   if (int rc = allow_big_lds(reinterpret_cast<const void*>(&sdd_group_kernel<T, EDGE, G>), G::SMEM, configured)) return rc;
   const int Mb = (int)((g.M + BS - 1) / BS), Cb = (int)((g.N + BS - 1) / BS);
   // the grid provides for the most groups a row of the block grid can split into
   const int tiles_m = (Mb + G::R - 1) / G::R, gmax = (Cb + G::MINCOLS - 1) / G::MINCOLS;
   hipLaunchKernelGGL((sdd_group_kernel<T, EDGE, G>), dim3((unsigned)(tiles_m * gmax)), dim3(THREADS), G::SMEM, stream,
                      g, tiles_m, gmax, Mb, Cb);
+  note_kernel("sdd:%s%s", G::R == 4 ? "big" : "mid", EDGE ? ":ragged" : "");
   return check_launch("sdd_group_kernel");
 }
 
@@ -1179,9 +1162,9 @@ template <typename T, bool EDGE>
 int launch_sdd_group(const GemmArgs& g, hipStream_t stream) {
   const int64_t Mb = (g.M + BS - 1) / BS, Cb = (g.N + BS - 1) / BS;
   // workgroups the big shape would have: a group spans 4 column blocks with everything kept, 6 once few enough tiles
-  // are kept for the width and not the tile count to end a group (measured: worth counting that way from p = 0.7);
-  // callers pass scale = 1 / (1 - p), which is the only hint of the kept fraction the host has
-  const float keep = (g.row_ptr && g.scale > 1.f) ? 1.f / g.scale : 1.f;
+  // are kept for the width and not the tile count to end a group (measured: worth counting that way from p = 0.7).
+  // The kept fraction is the caller's hint (the lists live on the device); unknown counts as everything kept.
+  const float keep = (g.row_ptr && g.keep_hint >= 0.f && g.keep_hint <= 1.f) ? g.keep_hint : 1.f;
   const int64_t cols = keep <= 0.3f ? SddBig::GW : SddBig::MINCOLS;
   const int64_t big = ((Mb + 3) / 4) * ((Cb + cols - 1) / cols);
   const int policy = tile_policy.load(std::memory_order_relaxed);
@@ -1207,19 +1190,20 @@ int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
 
 template <typename T, bool RAGGED, int FORM>
 int launch_conv_t(const GemmArgs& g, const ImplicitConv& cg, int smem, hipStream_t stream) {
-  static bool configured[kMaxDevices] = {};
+  static std::atomic<bool> configured[kMaxDevices] = {};
   auto* kernel = &dsd_kernel<T, false, false, RAGGED, DsdConv, FORM>;
   if (int rc = allow_big_lds(reinterpret_cast<const void*>(kernel), 163840, configured)) return rc;
   const int Mb = (int)(g.M / BS), Kb = (int)((g.K + BS - 1) / BS);
   const int tiles_m = (Mb + DsdConv::R - 1) / DsdConv::R, tiles_n = (int)((g.N + DsdConv::BN - 1) / DsdConv::BN);
   hipLaunchKernelGGL(kernel, dim3((unsigned)(tiles_m * tiles_n), 1u), dim3(DsdConv::THREADS), smem, stream, g,
                      tiles_m, tiles_n, Mb, Kb, cg);
+  note_kernel("conv_fwd:implicit:%s", FORM == 2 ? "rows-per-step" : "rows-resident");
   return check_launch("dsd_kernel (implicit conv)");
 }
 
 template <typename T, bool RAGGED>
 int launch_conv_dw_t(const GemmArgs& g, const ImplicitConv& cg, int smem, int splits, hipStream_t stream) {
-  static bool configured[kMaxDevices] = {};
+  static std::atomic<bool> configured[kMaxDevices] = {};
   auto* kernel = &dsd_kernel<T, true, true, RAGGED, DsdConv, 1>;
   if (int rc = allow_big_lds(reinterpret_cast<const void*>(kernel), 163840, configured)) return rc;
   const int Mb = (int)((g.M + BS - 1) / BS), Kb = (int)(g.K / BS);
@@ -1227,6 +1211,7 @@ int launch_conv_dw_t(const GemmArgs& g, const ImplicitConv& cg, int smem, int sp
   hipLaunchKernelGGL(kernel, dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits), dim3(DsdConv::THREADS), smem, stream,
                      g, tiles_m, tiles_n, Mb, Kb, cg);
   if (int rc = check_launch("dsd_kernel (implicit conv weight gradient)")) return rc;
+  note_kernel("conv_dw:implicit splits=%d", splits);
   if (splits > 1) return launch_splitk_reduce(g, splits, true, T::id, stream);
   return SD_OK;
 }

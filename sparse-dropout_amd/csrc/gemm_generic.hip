@@ -325,6 +325,7 @@ int launch_t(const GemmArgs& g, hipStream_t stream) {
   else
     hipLaunchKernelGGL((gemm_generic_kernel<T, MODE, false, false>), grid, block, 0, stream, g,
                        (int)tiles_n, a_kc, b_kc, a_vec, b_vec);
+  note_kernel("generic");
   return check_launch("gemm_generic");
 }
 

@@ -18,7 +18,7 @@ from __future__ import annotations
 
 import torch
 
-from ..hip.binding_gemm import GEMM, KeptLists, _block_size
+from ..hip.binding_gemm import GEMM, KeptLists, _block_size, as_matrix
 
 
 class BlockwiseDropoutMatmulHIP(torch.autograd.Function):
@@ -46,12 +46,12 @@ class BlockwiseDropoutMatmulHIP(torch.autograd.Function):
         ext = GEMM()
         if grad_output.dtype != input.dtype:
             grad_output = grad_output.to(input.dtype)
-        if grad_output.stride(0) != 1 and grad_output.stride(1) != 1:
-            grad_output = grad_output.contiguous()
+        grad_output = as_matrix(grad_output)  # expanded (stride 0) and doubly strided gradients are laid out first
         grad_input = grad_weight = None
         if ctx.needs_input_grad[0]:
             # dA (M K sparse) = dC (M N) * B.T (K N): the mask is over the output
-            grad_input = ext.gemm_sdd_lists(grad_output, weight.t(), lists, ctx.block_size, ctx.scale)
+            grad_input = ext.gemm_sdd_lists(grad_output, weight.t(), lists, ctx.block_size, ctx.scale,
+                                            keep_hint=1.0 / ctx.scale)
         if ctx.needs_input_grad[1]:
             # dB.T (K N) = A.T (K M sparse) * dC.T (N M), written straight into a row-major [N, K]
             grad_weight = ext.gemm_dsd_lists(input.t(), grad_output.t(), lists.transposed(),
@@ -77,11 +77,7 @@ def _prepare(input: torch.Tensor, weight: torch.Tensor):
     if torch.is_autocast_enabled("cuda"):
         dt = torch.get_autocast_dtype("cuda")
         input, weight = input.to(dt), weight.to(dt)
-    if input.stride(0) != 1 and input.stride(1) != 1:
-        input = input.contiguous()
-    if weight.stride(0) != 1 and weight.stride(1) != 1:
-        weight = weight.contiguous()
-    return input, weight
+    return as_matrix(input), as_matrix(weight)
 
 
 def blockwise_dropout_matmul_mask(input: torch.Tensor, mask: torch.Tensor, block_size, p: float,

@@ -97,7 +97,8 @@ class _Im2colConv2d(torch.autograd.Function):
                                        ch_last)
                 if dx is None:
                     # col2im skips the dropped blocks, so the SDD need not zero them
-                    dcols = ext.gemm_sdd_lists(dy2, w2.t(), lists, kernel_bs, scale, kept_only=True)
+                    dcols = ext.gemm_sdd_lists(dy2, w2.t(), lists, kernel_bs, scale, kept_only=True,
+                                                keep_hint=1.0 / scale)
                     dx = ext.col2im(dcols, x_shape, (r, s), padding, stride, dilation, mask, block_size, ch_last)
             if ctx.needs_input_grad[1]:
                 if ctx.implicit:  # the forward kept the input, not the patch matrix

@@ -1,12 +1,14 @@
 """ctypes loader for libsparsedrop.so (the C ABI declared in include/sparsedrop.h).
 
 The library is built ahead of time by ``sparse-dropout_amd/csrc/build.py``; there is no JIT step and
-no fallback: if the shared object is missing, loading raises.
+no fallback: if the shared object is missing, or was built from other sources than the ones next to it,
+loading raises.
 """
 from __future__ import annotations
 
 import ctypes
 from ctypes import c_char_p, c_float, c_int, c_int64, c_uint64, c_void_p
+import hashlib
 from functools import lru_cache
 from pathlib import Path
 
@@ -18,7 +20,10 @@ _mat = [c_void_p, c_int64, c_int64]  # ptr, stride_r, stride_c
 SIGNATURES = {
     "sd_version": (c_int, []),
     "sd_last_error": (c_char_p, []),
+    "sd_source_hash": (c_char_p, []),
     "sd_last_kernel": (c_char_p, []),
+    "sd_last_kernel_detail": (c_char_p, []),
+    "sd_tile_of_block": (c_int, [c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
     "sd_set_tile_policy": (c_int, [c_int]),
     "sd_workspace_bytes": (c_int64, [c_int64, c_int64]),
     "sd_build_lists": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64,
@@ -44,6 +49,8 @@ SIGNATURES = {
                                   c_int64, c_int64, c_float, c_int, c_void_p, c_int64, c_void_p]),
     "sd_gemm_sdd_lists": (c_int, [*_mat, *_mat, *_mat, c_void_p, c_void_p, c_int64, c_int64,
                                   c_int64, c_int64, c_float, c_int, c_void_p]),
+    "sd_gemm_sdd_lists_ex": (c_int, [*_mat, *_mat, *_mat, c_void_p, c_void_p, c_int64, c_int64,
+                                     c_int64, c_int64, c_float, c_int, c_int, c_float, c_void_p]),
     "sd_gemm_sdd_lists_kept": (c_int, [*_mat, *_mat, *_mat, c_void_p, c_void_p, c_int64, c_int64,
                                   c_int64, c_int64, c_float, c_int, c_void_p]),
     "sd_conv2d_dsd_lists": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64,
@@ -67,6 +74,21 @@ SIGNATURES = {
 }
 
 
+def source_hash() -> str | None:
+    """Hash of the sources the library is built from (the same function as build.py's), or None when the
+    sources are not there (an installed library without its source tree)."""
+    csrc = LIB_PATH.parent.parent.parent / "csrc"
+    include = csrc.parent.parent / "include"
+    files = [*sorted(csrc.glob("*.hip")), *sorted(csrc.glob("*.h")), *sorted(include.glob("*.h"))]
+    if not files:
+        return None
+    h = hashlib.sha256()
+    for f in files:
+        h.update(f.name.encode())
+        h.update(f.read_bytes())
+    return h.hexdigest()[:16]
+
+
 @lru_cache(maxsize=None)
 def load() -> ctypes.CDLL:
     if not LIB_PATH.exists():
@@ -79,4 +101,10 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)  # AttributeError here = header and library disagree
         fn.restype = res
         fn.argtypes = args
+    built, now = lib.sd_source_hash().decode(), source_hash()
+    if now is not None and built != now:
+        raise RuntimeError(
+            f"{LIB_PATH} was built from other sources (library {built}, tree {now}): rebuild it with "
+            "`python sparse-dropout_amd/csrc/build.py`"
+        )
     return lib

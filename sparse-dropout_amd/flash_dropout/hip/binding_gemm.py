@@ -100,7 +100,30 @@ def _check_operand(name: str, x: torch.Tensor) -> None:
 
 
 def _mat(x: torch.Tensor):
-    return x.data_ptr(), max(x.stride(0), 1), max(x.stride(1), 1)
+    """(pointer, row stride, column stride) in elements.  The stride of an extent-1 dimension is arbitrary in
+    torch and normalised here; a zero stride over a real extent (an expanded tensor) is not a matrix in memory."""
+    sr, sc = x.stride()
+    rows, cols = x.shape
+    if (rows > 1 and sr == 0) or (cols > 1 and sc == 0):
+        raise ValueError(f"operand is an expanded view (strides {x.stride()}): call .contiguous() first")
+    if rows <= 1 and sc == 1:
+        sr = max(cols, 1)
+    if cols <= 1 and sr == 1:
+        sc = max(rows, 1)
+    return x.data_ptr(), max(sr, 1), max(sc, 1)
+
+
+def as_matrix(x: torch.Tensor) -> torch.Tensor:
+    """``x`` itself when it is a row- or column-major matrix in memory (unit stride along one index, the other
+    stride at least the contiguous extent), else a contiguous copy: expanded gradients (stride 0, e.g. from
+    ``y.sum(0)``), overlapping or doubly strided views."""
+    rows, cols = x.shape
+    sr, sc = x.stride()
+    if sc == 1 and (rows <= 1 or sr >= cols):
+        return x
+    if sr == 1 and (cols <= 1 or sc >= rows):
+        return x
+    return x.contiguous()
 
 
 def _check_mask(mask: torch.Tensor, shape: tuple[int, int], like: torch.Tensor) -> torch.Tensor:
@@ -134,6 +157,10 @@ class GEMM:
     def last_kernel(self) -> str:
         """"specialised" or "generic": the kernel family this thread's last GEMM call ran on."""
         return self.lib.sd_last_kernel().decode()
+
+    def last_kernel_detail(self) -> str:
+        """Kernel, workgroup shape and reduction splits of this thread's last launch, e.g. "sdd:big"."""
+        return self.lib.sd_last_kernel_detail().decode()
 
     TILE_POLICIES = {"auto": 0, "big": 1, "mid": 2}
 
@@ -291,17 +318,29 @@ class GEMM:
     def manual_seed(self, seed: int, device=None) -> None:
         """(Re)starts the device-resident mask generator of ``device`` at (seed, offset 0).  Without this
         call the generator starts from ``torch.initial_seed()`` at first use and restarts whenever that
-        value changes (``torch.manual_seed`` with a new seed)."""
+        value changes (``torch.manual_seed`` with a new seed).
+
+        The state is ONE int64[4] tensor per device for the life of the process, reseeded in place by a copy
+        on the current stream: reseeding is ordered with the draws on that stream, and a captured graph (which
+        holds the tensor's address) follows a later reseed instead of reading freed memory."""
         dev = _device(device)
         seed = int(seed) & (2 ** 64 - 1)
         as_i64 = seed if seed < 2 ** 63 else seed - 2 ** 64
-        state = torch.tensor([as_i64, 0, 0, 0], dtype=torch.int64, device=dev)
+        host = torch.tensor([as_i64, 0, 0, 0], dtype=torch.int64)
+        entry = self._rng.get(dev.index)
+        if entry is None:
+            state = host.to(dev)
+        else:
+            state = entry[1]
+            with _guard(dev):
+                state.copy_(host)
         self._rng[dev.index] = (torch.initial_seed(), state)
 
     def rng_state(self, device=None) -> torch.Tensor:
         """int64[4] device tensor {seed, offset, 0, 0} behind the draws that are given no explicit seed; every
         such draw advances the offset by one on the stream it runs on.  Create it (one draw, or
-        :meth:`manual_seed`) before capturing a graph: the first use copies the seed from the host."""
+        :meth:`manual_seed`) before capturing a graph: the first use copies the seed from the host.  The same
+        tensor is returned for the life of the process."""
         dev = _device(device)
         entry = self._rng.get(dev.index)
         if entry is None or entry[0] != torch.initial_seed():
@@ -397,11 +436,25 @@ class GEMM:
         return self._listed(self.lib.sd_gemm_dsd_lists, "K", A, B, lists, block_size, scale, out, transposed_out)
 
     def gemm_sdd_lists(self, A, B, lists: KeptLists, block_size, scale, out=None, transposed_out=False,
-                       kept_only=False):
+                       kept_only=False, keep_hint: float | None = None):
         """``kept_only``: dropped tiles of the result are left as they are (uninitialised for a fresh buffer)
-        instead of being zeroed, for a consumer that never reads them (:meth:`col2im` with the mask)."""
-        fn = self.lib.sd_gemm_sdd_lists_kept if kept_only else self.lib.sd_gemm_sdd_lists
-        return self._listed(fn, "N", A, B, lists, block_size, scale, out, transposed_out)
+        instead of being zeroed, for a consumer that never reads them (:meth:`col2im` with the mask).
+        ``keep_hint``: expected fraction of kept blocks (1 - p) when the caller knows it; it only steers the
+        choice of workgroup shape (the lists live on the device), never the result."""
+        self._check_pair(A, B)
+        bs = _block_size(block_size)
+        M, N, K = A.shape[0], B.shape[0], A.shape[1]
+        want = (ceil(M / bs), ceil(N / bs))
+        if tuple(lists.shape) != want:
+            raise ValueError(f"lists are for a {lists.shape} mask, operands need {want}")
+        C = self._out(A, B, out, transposed_out)
+        if M == 0 or N == 0:
+            return C
+        with _guard(A.device):
+            self._call(self.lib.sd_gemm_sdd_lists_ex, *_mat(A), *_mat(B), *_mat(C), lists.row_ptr.data_ptr(),
+                       lists.col_idx.data_ptr(), M, N, K, bs, float(scale), _DTYPES[A.dtype],
+                       1 if kept_only else 0, -1.0 if keep_hint is None else float(keep_hint), self._stream(A))
+        return C
 
     # ------------------------------------------------------------------ conv feed
     @staticmethod

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 import torch
 
-from _util import REL_FRO_TOL, cpu_mask, rel_fro, to_np
+from _util import REL_FRO_TOL, max_tile_rel_fro, cpu_mask, rel_fro, to_np
 from oracle import naive_torch
 from oracle import sparsedrop_oracle as O
 
@@ -38,9 +38,9 @@ def test_cfg1_cpu_reference_configuration():
     ry, rdx, rdw = naive_torch.forward_backward(xh.float(), wh.float(), dyh.float(), mask, 64, 0.5)
     y, dx, dw = _fwd_bwd(xh.cuda(), wh.cuda(), dyh.cuda(), mask.cuda(), 64, 0.5)
     assert y.dtype == torch.float16 and dw.is_contiguous() and dw.shape == (1024, 1024)
-    assert rel_fro(y, ry) <= REL_FRO_TOL
-    assert rel_fro(dx, rdx) <= REL_FRO_TOL
-    assert rel_fro(dw, rdw) <= REL_FRO_TOL
+    assert max_tile_rel_fro(y, ry) <= REL_FRO_TOL
+    assert max_tile_rel_fro(dx, rdx) <= REL_FRO_TOL
+    assert max_tile_rel_fro(dw, rdw) <= REL_FRO_TOL
     # and against the unrounded fp32 problem the reference's tolerances still hold
     fy, fdx, fdw = naive_torch.forward_backward(x, w, dy, mask, 64, 0.5)
     torch.testing.assert_close(y.float().cpu(), fy, atol=0.2, rtol=0.01)
@@ -73,11 +73,11 @@ def test_cfg4_transformer_mlp(p):
     ar = torch.nn.functional.gelu(hr)
     yr = naive_torch.forward(ar, w2r, m2, 64, p)
     yr.backward(dy.float())
-    assert rel_fro(h, hr) <= REL_FRO_TOL
-    assert rel_fro(y, yr) <= REL_FRO_TOL
-    assert rel_fro(xg.grad, xr.grad) <= REL_FRO_TOL
-    assert rel_fro(w1g.grad, w1r.grad) <= REL_FRO_TOL
-    assert rel_fro(w2g.grad, w2r.grad) <= REL_FRO_TOL
+    assert max_tile_rel_fro(h, hr) <= REL_FRO_TOL
+    assert max_tile_rel_fro(y, yr) <= REL_FRO_TOL
+    assert max_tile_rel_fro(xg.grad, xr.grad) <= REL_FRO_TOL
+    assert max_tile_rel_fro(w1g.grad, w1r.grad) <= REL_FRO_TOL
+    assert max_tile_rel_fro(w2g.grad, w2r.grad) <= REL_FRO_TOL
 
 
 def test_cfg3_mlp_on_28x28_images_through_layers():
@@ -115,9 +115,9 @@ def test_cfg3_mlp_on_28x28_images_through_layers():
     masks = [O.random_mask((64, -(-dims[i] // 64)), 0.5, 123, offset=i) for i in range(3)]
     for i, l in enumerate(mods):
         a, g, w = to_np(ins[i]), to_np(outs[i].grad), to_np(l.weight)
-        assert rel_fro(outs[i], O.dsd_forward(a, w, masks[i], 64, 0.5, np.float32)) <= REL_FRO_TOL, f"Y{i}"
-        assert rel_fro(ins[i].grad, O.sdd_dx(g, w, masks[i], 64, 0.5, np.float32)) <= REL_FRO_TOL, f"dX{i}"
-        assert rel_fro(l.weight.grad, O.dsd_dw(g, a, masks[i], 64, 0.5, np.float32)) <= REL_FRO_TOL, f"dW{i}"
+        assert max_tile_rel_fro(outs[i], O.dsd_forward(a, w, masks[i], 64, 0.5, np.float32)) <= REL_FRO_TOL, f"Y{i}"
+        assert max_tile_rel_fro(ins[i].grad, O.sdd_dx(g, w, masks[i], 64, 0.5, np.float32)) <= REL_FRO_TOL, f"dX{i}"
+        assert max_tile_rel_fro(l.weight.grad, O.dsd_dw(g, a, masks[i], 64, 0.5, np.float32)) <= REL_FRO_TOL, f"dW{i}"
         assert l.weight.grad.shape == l.weight.shape
 
 
@@ -136,7 +136,7 @@ def test_layer_eval_and_3d_inputs_and_bf16():
     assert y.shape == (8, 256, 256) and y.dtype == torch.bfloat16
     mask = O.random_mask((32, 6), 0.3, 9, offset=0)  # first draw after the restart
     ref = O.dsd_forward(to_np(x.reshape(-1, 384)), to_np(layer.weight), mask, 64, 0.3, np.float32)
-    assert rel_fro(y.reshape(-1, 256), ref) <= REL_FRO_TOL
+    assert max_tile_rel_fro(y.reshape(-1, 256), ref) <= REL_FRO_TOL
 
 
 def test_autocast_contract():
@@ -156,10 +156,10 @@ def test_autocast_contract():
         y.float().sum().backward()
         assert x.grad.dtype == torch.float32 and w.grad.dtype == torch.float32
         ref = O.dsd_forward(to_np(x.to(dt)), to_np(w.to(dt)), mask.cpu().numpy(), 64, 0.5, np.float32)
-        assert rel_fro(y, ref) <= REL_FRO_TOL
+        assert max_tile_rel_fro(y, ref) <= REL_FRO_TOL
         ones = np.ones((256, 128), dtype=np.float32)
-        assert rel_fro(x.grad, O.sdd_dx(ones, to_np(w.to(dt)), mask.cpu().numpy(), 64, 0.5, np.float32)) <= REL_FRO_TOL
-        assert rel_fro(w.grad, O.dsd_dw(ones, to_np(x.to(dt)), mask.cpu().numpy(), 64, 0.5, np.float32)) <= REL_FRO_TOL
+        assert max_tile_rel_fro(x.grad, O.sdd_dx(ones, to_np(w.to(dt)), mask.cpu().numpy(), 64, 0.5, np.float32)) <= REL_FRO_TOL
+        assert max_tile_rel_fro(w.grad, O.dsd_dw(ones, to_np(x.to(dt)), mask.cpu().numpy(), 64, 0.5, np.float32)) <= REL_FRO_TOL
 
 
 def test_public_names_and_p_range():
@@ -172,7 +172,7 @@ def test_public_names_and_p_range():
     with pytest.raises(ValueError, match=r"\[0, 1\)"):
         F.cuda_blockwise_dropout_matmul(x, x, 64, 1.0)
     y = F.cuda_blockwise_dropout_matmul(x, x, 64, 0.0)
-    assert rel_fro(y, to_np(x) @ to_np(x).T) <= REL_FRO_TOL
+    assert max_tile_rel_fro(y, to_np(x) @ to_np(x).T) <= REL_FRO_TOL
     # statistical sanity of the fresh mask: about p of the blocks are dropped
     big = torch.ones(4096, 4096, device="cuda", dtype=torch.float16)
     eye = torch.eye(4096, device="cuda", dtype=torch.float16)
@@ -181,3 +181,27 @@ def test_public_names_and_p_range():
     frac_dropped = (out == 0).float().mean().item()
     assert abs(frac_dropped - 0.25) < 0.03
     assert torch.all((out == 0) | (out == torch.tensor(1 / 0.75, dtype=torch.float16, device="cuda")))
+
+
+def test_backward_takes_an_expanded_gradient():
+    """y.sum(0).sum().backward() hands the backward a gradient with strides (0, 1); it is laid out before the
+    kernels see it, and the result is the gradient of a materialised all-ones dY."""
+    import flash_dropout.functional as F
+
+    gen = torch.Generator().manual_seed(12)
+    x = torch.randn(256, 192, generator=gen).half().cuda()
+    w = (torch.randn(128, 192, generator=gen) * 192 ** -0.5).half().cuda()
+    mask = cpu_mask((4, 3), 0.5, gen).cuda()
+    grads = []
+    for expanded in (True, False):
+        xg, wg = x.clone().requires_grad_(), w.clone().requires_grad_()
+        y = F.hip_blockwise_dropout_matmul_mask(xg, mask, 64, 0.5, wg)
+        if expanded:
+            y.sum(0).sum().backward()
+        else:
+            y.backward(torch.ones_like(y))
+        grads.append((xg.grad, wg.grad))
+    assert torch.equal(grads[0][0], grads[1][0]) and torch.equal(grads[0][1], grads[1][1])
+    ones = np.ones((256, 128), dtype=np.float32)
+    assert max_tile_rel_fro(grads[0][0], O.sdd_dx(ones, to_np(w), mask.cpu().numpy(), 64, 0.5, np.float32)) <= REL_FRO_TOL
+    assert max_tile_rel_fro(grads[0][1], O.dsd_dw(ones, to_np(x), mask.cpu().numpy(), 64, 0.5, np.float32)) <= REL_FRO_TOL

@@ -182,3 +182,68 @@ def test_dropout_conv_layer_host_logic():
         assert DropoutConv2d(3, 4, (3, 3), padding=(1, 1), variant=variant)(x).shape == (2, 4, 8, 8)
     with pytest.raises(ValueError, match="Unknown variant"):
         DropoutConv2d(3, 4, (3, 3), variant="nope")(x)
+
+
+@pytest.mark.parametrize("kind", [0, 1])
+def test_tile_map_is_a_bijection_onto_the_tile_grid(kind):
+    """The workgroup-to-tile map of the specialised kernels (the counterpart of the reference's
+    threadblock_swizzle, gemm.cuh:84-97) must hit every tile of the grid exactly once, for every grid up to
+    40 x 40 — totals that are not multiples of the 8 XCDs and tile-row counts that are not multiples of the
+    group height included."""
+    from flash_dropout.hip import _loader
+
+    lib = _loader.load()
+    tm, tn = ctypes.c_int32(), ctypes.c_int32()
+    for tiles_m in range(1, 41):
+        for tiles_n in range(1, 41):
+            seen = set()
+            for b in range(tiles_m * tiles_n):
+                assert lib.sd_tile_of_block(kind, b, tiles_m, tiles_n, ctypes.byref(tm), ctypes.byref(tn)) == 0
+                assert 0 <= tm.value < tiles_m and 0 <= tn.value < tiles_n, (tiles_m, tiles_n, b)
+                seen.add((tm.value, tn.value))
+            assert len(seen) == tiles_m * tiles_n, (tiles_m, tiles_n)
+    # outside the grid: an error, not a tile
+    assert lib.sd_tile_of_block(kind, 12, 3, 4, ctypes.byref(tm), ctypes.byref(tn)) == 1
+    assert lib.sd_tile_of_block(2, 0, 3, 4, ctypes.byref(tm), ctypes.byref(tn)) == 1
+
+
+def test_tile_map_keeps_an_xcd_on_a_compact_patch():
+    """What the map is for: the 32 workgroups an XCD holds at a time (launch indices x, x+8, x+16, ...) cover
+    at most 8 tile rows x 4+1 tile columns of a large grid, not a scattered set."""
+    from flash_dropout.hip import _loader
+
+    lib = _loader.load()
+    tm, tn = ctypes.c_int32(), ctypes.c_int32()
+    tiles_m = tiles_n = 32
+    for x in range(8):
+        rows, cols = set(), set()
+        for i in range(32):
+            lib.sd_tile_of_block(0, x + 8 * i, tiles_m, tiles_n, ctypes.byref(tm), ctypes.byref(tn))
+            rows.add(tm.value)
+            cols.add(tn.value)
+        assert len(rows) <= 8 and len(cols) <= 5, (x, sorted(rows), sorted(cols))
+
+
+def test_loader_refuses_a_library_built_from_other_sources(monkeypatch):
+    from flash_dropout.hip import _loader
+
+    lib = _loader.load()
+    assert lib.sd_source_hash().decode() == _loader.source_hash()
+    monkeypatch.setattr(_loader, "source_hash", lambda: "0" * 16)
+    with pytest.raises(RuntimeError, match="built from other sources"):
+        _loader.load.__wrapped__()
+
+
+def test_as_matrix_lays_out_expanded_and_strided_views():
+    from flash_dropout.hip.binding_gemm import _mat, as_matrix
+
+    a = torch.zeros(6, 8)
+    at = a.t()
+    assert as_matrix(a) is a and as_matrix(at) is at
+    assert as_matrix(a[:, :4]) is not None and as_matrix(a[:, :4]).data_ptr() == a.data_ptr()  # row stride 8 >= 4
+    e = torch.zeros(1, 8).expand(6, 8)  # strides (0, 1): what y.sum(0) hands to backward
+    assert as_matrix(e).stride() == (8, 1)
+    assert as_matrix(a[::2, ::2]).stride() == (4, 1)
+    with pytest.raises(ValueError, match="expanded view"):
+        _mat(e)
+    assert _mat(torch.zeros(1, 8))[1:] == (8, 1)
