@@ -260,6 +260,44 @@ int sd_gemm_sdd_lists_kept(const void* A, int64_t a_stride_r, int64_t a_stride_c
                            void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * The reference's autograd function in two calls (one launch path each instead of two), for small layers whose
+ * step time is the host's launch path.
+ *
+ * sd_dropout_matmul_forward = BlockwiseDropoutMatmulCUDA.forward,
+ * flash_dropout/functional/blockwise_dropout_matmul_cuda.py:10-32: the block mask (given: `mask`, [ceil(M/bs),
+ * ceil(K/bs)] bytes with strides, non-zero = dropped; or drawn with probability p: from the device-resident state
+ * `rng_state` as sd_random_lists_state does, or, when that is NULL too, from (seed, offset) as sd_random_lists does;
+ * a drawn mask is stored to mask_out), its kept-block lists, and Y = (keep . X) / (1 - p) . W^T.  The lists are left
+ * in the caller's arrays for the backward call; they are built at the granularity the kernels run at:
+ * g = 64 when block_size is a multiple of 64 (else block_size), i.e. row_ptr[ceil(M/g) + 1], col_idx[ceil(M/g) *
+ * ceil(K/g)], col_ptr[ceil(K/g) + 1], row_idx[same capacity]; the CSC pair may be NULL when no weight gradient
+ * will be asked for.  workspace: optional split-reduction scratch (sd_splitk_workspace_bytes(M, N, K, g, 1)).
+ *
+ * sd_dropout_matmul_backward = BlockwiseDropoutMatmulCUDA.backward, same file :36-53: dX = (dY . W) . keep / (1 - p)
+ * (written in full, zeros where dropped) and dW = dY^T . (keep . X) / (1 - p), each skipped when its pointer is NULL.
+ * dW is written through its own strides: pass a row-major [N, K] tensor to get what the reference returns as a
+ * transposed view.  workspace: optional split-reduction scratch for dW (sd_splitk_workspace_bytes(K, N, M, g, 1)).
+ * ------------------------------------------------------------------------------------------- */
+int sd_dropout_matmul_forward(const void* X, int64_t x_stride_r, int64_t x_stride_c,
+                              const void* W, int64_t w_stride_r, int64_t w_stride_c,
+                              void* Y, int64_t y_stride_r, int64_t y_stride_c,
+                              const uint8_t* mask, int64_t mask_stride_r, int64_t mask_stride_c,
+                              uint64_t* rng_state, uint64_t seed, uint64_t offset, float p, uint8_t* mask_out,
+                              int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx,
+                              int64_t M, int64_t N, int64_t K, int64_t block_size, int dtype,
+                              void* workspace, int64_t workspace_bytes, void* stream);
+
+int sd_dropout_matmul_backward(const void* dY, int64_t dy_stride_r, int64_t dy_stride_c,
+                               const void* W, int64_t w_stride_r, int64_t w_stride_c,
+                               const void* X, int64_t x_stride_r, int64_t x_stride_c,
+                               void* dX, int64_t dx_stride_r, int64_t dx_stride_c,
+                               void* dW, int64_t dw_stride_r, int64_t dw_stride_c,
+                               const int32_t* row_ptr, const int32_t* col_idx,
+                               const int32_t* col_ptr, const int32_t* row_idx,
+                               int64_t M, int64_t N, int64_t K, int64_t block_size, float p, int dtype,
+                               void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * (e) im2col gather feeding the same GEMMs for conv.
  *
  * cols[(n*P+p)*Q+q, c*R*S + r*S + s] = x[n, c, p*stride_h + r*dil_h - pad_h, q*stride_w + s*dil_w - pad_w]

@@ -384,6 +384,67 @@ int sd_gemm_sdd(const void* A, int64_t asr, int64_t asc, const void* B, int64_t 
                            dtype, stream);
 }
 
+// granularity of the lists the fused calls build and take: 64 for block sizes that are multiples of 64
+static int64_t list_granule(int64_t bs) { return bs % 64 == 0 ? 64 : bs; }
+
+int sd_dropout_matmul_forward(const void* X, int64_t xsr, int64_t xsc, const void* W, int64_t wsr, int64_t wsc,
+                              void* Y, int64_t ysr, int64_t ysc, const uint8_t* mask, int64_t msr, int64_t msc,
+                              uint64_t* rng_state, uint64_t seed, uint64_t offset, float p, uint8_t* mask_out,
+                              int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx, int64_t M,
+                              int64_t N, int64_t K, int64_t bs, int dtype, void* workspace, int64_t workspace_bytes,
+                              void* stream) {
+  if (int rc = check_common(X, xsr, xsc, W, wsr, wsc, Y, ysr, ysc, M, N, K, dtype)) return rc;
+  SD_REQUIRE(p >= 0.f && p < 1.f, "dropout_matmul_forward: p must be in [0, 1) (got %g)", (double)p);
+  if (int rc = check_sparse(bs, 1.f)) return rc;
+  SD_REQUIRE(M > 0 && K > 0, "dropout_matmul_forward: empty operand");
+  SD_REQUIRE(row_ptr && col_idx, "dropout_matmul_forward: the CSR list arrays are required");
+  const int64_t g = list_granule(bs), split = bs / g;
+  const int64_t mb = ceil_div(M, bs), kb = ceil_div(K, bs), out_mb = ceil_div(M, g), out_kb = ceil_div(K, g);
+  if (mask) {
+    if (int rc = sd_build_lists_split(mask, mb, kb, msr, msc, split, out_mb, out_kb, row_ptr, col_idx, col_ptr, row_idx,
+                                      stream))
+      return rc;
+  } else if (rng_state) {
+    if (int rc = sd_random_lists_state(rng_state, p, mb, kb, mask_out, split, out_mb, out_kb, row_ptr, col_idx, col_ptr,
+                                       row_idx, stream))
+      return rc;
+  } else {
+    if (int rc = sd_random_lists(seed, offset, p, mb, kb, mask_out, split, out_mb, out_kb, row_ptr, col_idx, col_ptr,
+                                 row_idx, stream))
+      return rc;
+  }
+  if (N == 0) return SD_OK;
+  return sd_gemm_dsd_lists(X, xsr, xsc, W, wsr, wsc, Y, ysr, ysc, row_ptr, col_idx, M, N, K, g, 1.f / (1.f - p), dtype,
+                           workspace, workspace_bytes, stream);
+}
+
+int sd_dropout_matmul_backward(const void* dY, int64_t gsr, int64_t gsc, const void* W, int64_t wsr, int64_t wsc,
+                               const void* X, int64_t xsr, int64_t xsc, void* dX, int64_t dxsr, int64_t dxsc,
+                               void* dW, int64_t dwsr, int64_t dwsc, const int32_t* row_ptr, const int32_t* col_idx,
+                               const int32_t* col_ptr, const int32_t* row_idx, int64_t M, int64_t N, int64_t K,
+                               int64_t bs, float p, int dtype, void* workspace, int64_t workspace_bytes, void* stream) {
+  SD_REQUIRE(p >= 0.f && p < 1.f, "dropout_matmul_backward: p must be in [0, 1) (got %g)", (double)p);
+  if (int rc = check_sparse(bs, 1.f)) return rc;
+  SD_REQUIRE(dX || dW, "dropout_matmul_backward: nothing to compute");
+  const int64_t g = list_granule(bs);
+  const float scale = 1.f / (1.f - p);
+  if (dX) {
+    // dX[M,K] = scale * (dY[M,N] . W[N,K]) where kept: A = dY, B = W^T as the [K, N] view of W
+    SD_REQUIRE(row_ptr && col_idx, "dropout_matmul_backward: dX needs the CSR lists");
+    if (int rc = sd_gemm_sdd_lists_ex(dY, gsr, gsc, W, wsc, wsr, dX, dxsr, dxsc, row_ptr, col_idx, M, K, N, g, scale,
+                                      dtype, 0, 1.f - p, stream))
+      return rc;
+  }
+  if (dW) {
+    // dW^T[K,N] = scale * X^T[K,M] (kept blocks) . dY[M,N]: A = X^T, B = dY^T, C = dW^T, lists of the transposed mask
+    SD_REQUIRE(col_ptr && row_idx, "dropout_matmul_backward: dW needs the CSC lists");
+    if (int rc = sd_gemm_dsd_lists(X, xsc, xsr, dY, gsc, gsr, dW, dwsc, dwsr, col_ptr, row_idx, K, N, M, g, scale, dtype,
+                                   workspace, workspace_bytes, stream))
+      return rc;
+  }
+  return SD_OK;
+}
+
 int sd_im2col(const void* x, int64_t sn, int64_t sc, int64_t sh, int64_t sw, void* cols, int64_t ld,
               int64_t n, int64_t c, int64_t h, int64_t w, int64_t r, int64_t s, int64_t pad_h,
               int64_t pad_w, int64_t stride_h, int64_t stride_w, int64_t dil_h, int64_t dil_w,

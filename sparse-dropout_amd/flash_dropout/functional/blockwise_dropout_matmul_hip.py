@@ -26,17 +26,14 @@ class BlockwiseDropoutMatmulHIP(torch.autograd.Function):
     def forward(ctx, input: torch.Tensor, weight: torch.Tensor, mask: torch.Tensor | None,
                 block_size: int, p: float, seed: int | None = None):
         ext = GEMM()
-        scale = 1.0 / (1.0 - p)
-        # mask given, or drawn in the list-building launch (reference: blockwise_dropout_mask, …_cuda.py:24)
-        mask, lists, kernel_bs = ext.kept_lists(input.shape[0], input.shape[1], block_size, mask, p, seed,
-                                                input.device)
-        # C (M N) = A (M K sparse) * B (N K)
-        out = ext.gemm_dsd_lists(input, weight, lists, kernel_bs, scale)
+        # mask given, or drawn in the list-building launch (reference: blockwise_dropout_mask, …_cuda.py:24);
+        # C (M N) = A (M K sparse) * B (N K); one library call for mask, lists and product
+        out, mask, lists, kernel_bs = ext.dropout_matmul_forward(input, weight, block_size, p, mask, seed)
         ctx.save_for_backward(input, weight, mask, lists.row_ptr, lists.col_idx, lists.col_ptr,
                               lists.row_idx)
         ctx.block_size = kernel_bs
         ctx.list_shape = lists.shape
-        ctx.scale = scale
+        ctx.p = p
         return out
 
     @staticmethod
@@ -47,15 +44,10 @@ class BlockwiseDropoutMatmulHIP(torch.autograd.Function):
         if grad_output.dtype != input.dtype:
             grad_output = grad_output.to(input.dtype)
         grad_output = as_matrix(grad_output)  # expanded (stride 0) and doubly strided gradients are laid out first
-        grad_input = grad_weight = None
-        if ctx.needs_input_grad[0]:
-            # dA (M K sparse) = dC (M N) * B.T (K N): the mask is over the output
-            grad_input = ext.gemm_sdd_lists(grad_output, weight.t(), lists, ctx.block_size, ctx.scale,
-                                            keep_hint=1.0 / ctx.scale)
-        if ctx.needs_input_grad[1]:
-            # dB.T (K N) = A.T (K M sparse) * dC.T (N M), written straight into a row-major [N, K]
-            grad_weight = ext.gemm_dsd_lists(input.t(), grad_output.t(), lists.transposed(),
-                                             ctx.block_size, ctx.scale, transposed_out=True).t()
+        # dA (M K sparse) = dC (M N) * B.T (K N), the mask over the output; dB.T (K N) = A.T (K M sparse) * dC.T (N M),
+        # written straight into a row-major [N, K] (reference: …_cuda.py:46-51); one library call for both
+        grad_input, grad_weight = ext.dropout_matmul_backward(grad_output, weight, input, lists, ctx.block_size, ctx.p,
+                                                              ctx.needs_input_grad[0], ctx.needs_input_grad[1])
         return grad_input, grad_weight, None, None, None, None
 
 

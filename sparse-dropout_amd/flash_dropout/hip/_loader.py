@@ -53,6 +53,12 @@ SIGNATURES = {
                                      c_int64, c_int64, c_float, c_int, c_int, c_float, c_void_p]),
     "sd_gemm_sdd_lists_kept": (c_int, [*_mat, *_mat, *_mat, c_void_p, c_void_p, c_int64, c_int64,
                                   c_int64, c_int64, c_float, c_int, c_void_p]),
+    "sd_dropout_matmul_forward": (c_int, [*_mat, *_mat, *_mat, *_mat, c_void_p, c_uint64, c_uint64, c_float, c_void_p,
+                                          c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                          c_int, c_void_p, c_int64, c_void_p]),
+    "sd_dropout_matmul_backward": (c_int, [*_mat, *_mat, *_mat, *_mat, *_mat, c_void_p, c_void_p, c_void_p, c_void_p,
+                                           c_int64, c_int64, c_int64, c_int64, c_float, c_int, c_void_p, c_int64,
+                                           c_void_p]),
     "sd_conv2d_dsd_lists": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64,
                                     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
@@ -79,9 +85,10 @@ def source_hash() -> str | None:
     sources are not there (an installed library without its source tree)."""
     csrc = LIB_PATH.parent.parent.parent / "csrc"
     include = csrc.parent.parent / "include"
-    files = [*sorted(csrc.glob("*.hip")), *sorted(csrc.glob("*.h")), *sorted(include.glob("*.h"))]
-    if not files:
+    hips = sorted(csrc.glob("*.hip"))
+    if not hips:
         return None
+    files = [*hips, *sorted(csrc.glob("*.h")), *sorted(include.glob("*.h"))]
     h = hashlib.sha256()
     for f in files:
         h.update(f.name.encode())

@@ -456,6 +456,85 @@ class GEMM:
                        1 if kept_only else 0, -1.0 if keep_hint is None else float(keep_hint), self._stream(A))
         return C
 
+    # ------------------------------------------------------------------ the autograd function's two calls
+    def dropout_matmul_forward(self, x: torch.Tensor, w: torch.Tensor, block_size, p: float,
+                               mask: torch.Tensor | None = None, seed: int | None = None):
+        """Mask (given, or drawn on the device: pinned by ``seed``, else from the device-resident generator),
+        kept-block lists and ``Y = (keep ⊙ x)/(1-p) @ w.T`` in one library call -> (y, mask, lists, kernel block
+        size).  The lists are at the granularity the kernels run at (64 for block sizes that are multiples of
+        64) and serve :meth:`dropout_matmul_backward`."""
+        self._check_pair(x, w)
+        bs = _block_size(block_size)
+        if not 0.0 <= p < 1.0:
+            raise ValueError(f"p must be in [0, 1), got {p}")
+        M, K, N = x.shape[0], x.shape[1], w.shape[0]
+        g = 64 if bs % 64 == 0 else bs
+        mb, kb, out_mb, out_kb = ceil(M / bs), ceil(K / bs), ceil(M / g), ceil(K / g)
+        if mb == 0 or kb == 0:
+            raise ValueError("mask must be non-empty")
+        dev = x.device
+        state = None
+        if mask is None:
+            mask = torch.empty((mb, kb), dtype=torch.bool, device=dev)
+            given = (None, 0, 0)
+            if seed is None:
+                state = self.rng_state(dev)
+        else:
+            mask = _check_mask(mask, (mb, kb), x)
+            given = (mask.data_ptr(), *_mask_strides(mask))
+        row_ptr, col_ptr, col_idx, row_idx = self._list_buffers(out_mb, out_kb, dev)
+        y = torch.empty((M, N), dtype=x.dtype, device=dev)
+        ws, ws_ptr, ws_bytes = self._splitk_scratch(x, w, g, 1)
+        with _guard(dev):
+            self._call(self.lib.sd_dropout_matmul_forward, *_mat(x), *_mat(w), *_mat(y), *given,
+                       None if state is None else state.data_ptr(), (int(seed) & (2 ** 64 - 1)) if seed is not None else 0,
+                       0, float(p), mask.data_ptr(), row_ptr.data_ptr(), col_idx.data_ptr(), col_ptr.data_ptr(),
+                       row_idx.data_ptr(), M, N, K, bs, _DTYPES[x.dtype], ws_ptr, ws_bytes, self._stream(x))
+        return y, mask, KeptLists(row_ptr, col_idx, col_ptr, row_idx, (out_mb, out_kb)), g
+
+    def dropout_matmul_backward(self, dy: torch.Tensor, w: torch.Tensor, x: torch.Tensor, lists: KeptLists,
+                                block_size, p: float, need_dx: bool = True, need_dw: bool = True):
+        """``dX = (dy @ w) ⊙ keep / (1-p)`` and ``dW = dy.T @ (keep ⊙ x) / (1-p)`` (a contiguous [N, K] tensor) in
+        one library call; either may be skipped -> (dx or None, dw or None)."""
+        self._check_pair(x, w)
+        _check_operand("dy", dy)
+        bs = _block_size(block_size)
+        M, K, N = x.shape[0], x.shape[1], w.shape[0]
+        if tuple(dy.shape) != (M, N) or dy.dtype != x.dtype or dy.device != x.device:
+            raise ValueError(f"dy must be a [{M}, {N}] {x.dtype} tensor on {x.device}")
+        g = 64 if bs % 64 == 0 else bs
+        if tuple(lists.shape) != (ceil(M / g), ceil(K / g)):
+            raise ValueError(f"lists are for a {lists.shape} mask, operands need {(ceil(M / g), ceil(K / g))}")
+        if N % 8 and N > 0 and M > 0 and K > 0 and (need_dx or need_dw):
+            # An output width that is not a multiple of 8 (a 10-class head) would put 16-byte loads across row
+            # ends in both products.  Zero-padded copies of dY and W (the reference pads its head to 128 outputs
+            # up front, eval/mlp/model.py:22-24,40) keep them on the specialised kernels: the extra columns of dY
+            # are zeros, so dX is unchanged, and the extra rows of dW are dropped.
+            n_pad = (N + 7) // 8 * 8
+            dy_pad = dy.new_zeros((M, n_pad))
+            dy_pad[:, :N] = dy
+            w_pad = w.new_zeros((n_pad, K))
+            if need_dx:
+                w_pad[:N] = w
+            dx, dw = self.dropout_matmul_backward(dy_pad, w_pad, x, lists, bs, p, need_dx, need_dw)
+            return dx, (dw[:N] if dw is not None else None)
+        dx = torch.empty((M, K), dtype=x.dtype, device=x.device) if need_dx else None
+        dw = torch.empty((N, K), dtype=x.dtype, device=x.device) if need_dw else None
+        if not (need_dx or need_dw) or M == 0 or K == 0:
+            return dx, dw
+        if N == 0:
+            return (dx.zero_() if need_dx else None), dw
+        ws_ptr, ws_bytes, ws = None, 0, None
+        if need_dw:  # the weight gradient of a tall activation matrix splits its reduction over workgroups
+            ws, ws_ptr, ws_bytes = self._splitk_scratch(x.t(), dy.t(), g, 1)
+        with _guard(x.device):
+            self._call(self.lib.sd_dropout_matmul_backward, *_mat(dy), *_mat(w), *_mat(x),
+                       *(_mat(dx) if need_dx else (None, 0, 0)), *(_mat(dw) if need_dw else (None, 0, 0)),
+                       lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(), lists.col_ptr.data_ptr(),
+                       lists.row_idx.data_ptr(), M, N, K, bs, float(p), _DTYPES[x.dtype], ws_ptr, ws_bytes,
+                       self._stream(x))
+        return dx, dw
+
     # ------------------------------------------------------------------ conv feed
     @staticmethod
     def conv_out_hw(h, w, r, s, padding, stride, dilation):

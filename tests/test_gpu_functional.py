@@ -205,3 +205,75 @@ def test_backward_takes_an_expanded_gradient():
     ones = np.ones((256, 128), dtype=np.float32)
     assert max_tile_rel_fro(grads[0][0], O.sdd_dx(ones, to_np(w), mask.cpu().numpy(), 64, 0.5, np.float32)) <= REL_FRO_TOL
     assert max_tile_rel_fro(grads[0][1], O.dsd_dw(ones, to_np(x), mask.cpu().numpy(), 64, 0.5, np.float32)) <= REL_FRO_TOL
+
+
+def test_narrow_head_stays_on_the_specialised_kernels():
+    """The 10-class head of the MLP configuration (1024 -> 10): forward, input gradient and weight gradient all run
+    on the specialised kernels (the backward pads the 10 output columns to 16 with zeros, as the reference pads its
+    head to 128, eval/mlp/model.py:22-24,40) and match the oracle."""
+    import flash_dropout.functional as F
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(14)
+    M, K, N, p = 4096, 1024, 10, 0.5
+    x = torch.rand(M, K, generator=gen).half()
+    w = ((torch.rand(N, K, generator=gen) * 2 - 1) * K ** -0.5).half()
+    dy = torch.randn(M, N, generator=gen).half()
+    mask = cpu_mask((M // 64, K // 64), p, gen)
+    a, b, g, mk = to_np(x), to_np(w), to_np(dy), mask.numpy()
+    # the library calls the autograd function makes (its backward runs on autograd's own thread, and which kernel
+    # ran is recorded per thread)
+    y, _, lists, g_bs = ext.dropout_matmul_forward(x.cuda(), w.cuda(), 64, p, mask=mask.cuda())
+    assert ext.last_kernel() == "specialised"
+    dx, none = ext.dropout_matmul_backward(dy.cuda(), w.cuda(), x.cuda(), lists, g_bs, p, need_dw=False)
+    assert none is None and ext.last_kernel() == "specialised" and ext.last_kernel_detail().startswith("sdd:")
+    none, dw = ext.dropout_matmul_backward(dy.cuda(), w.cuda(), x.cuda(), lists, g_bs, p, need_dx=False)
+    assert none is None and ext.last_kernel() == "specialised" and ext.last_kernel_detail().startswith("dsd:")
+    assert dw.shape == (N, K)
+    ry, rdx, rdw = (O.dsd_forward(a, b, mk, 64, p, np.float32), O.sdd_dx(g, b, mk, 64, p, np.float32),
+                    O.dsd_dw(g, a, mk, 64, p, np.float32))
+    for got, ref in ((y, ry), (dx, rdx), (dw, rdw)):
+        assert max_tile_rel_fro(got, ref) <= REL_FRO_TOL
+    # and through autograd
+    xg, wg = x.cuda().requires_grad_(), w.cuda().requires_grad_()
+    F.hip_blockwise_dropout_matmul_mask(xg, mask.cuda(), 64, p, wg).backward(dy.cuda())
+    assert wg.grad.shape == (N, K)
+    assert max_tile_rel_fro(xg.grad, rdx) <= REL_FRO_TOL
+    assert max_tile_rel_fro(wg.grad, rdw) <= REL_FRO_TOL
+
+
+@pytest.mark.parametrize("bs", [64, 128])
+def test_fused_forward_and_backward_calls_match_the_separate_ones(bs):
+    """sd_dropout_matmul_forward / _backward (mask, lists and product in one library call; both gradients in one)
+    against the calls they bundle, bit for bit, with a given mask, a seeded draw and the device-resident generator."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(15)
+    M, K, N, p = 640, 448, 200, 0.3
+    x = torch.randn(M, K, generator=gen).half().cuda()
+    w = (torch.randn(N, K, generator=gen) * K ** -0.5).half().cuda()
+    dy = torch.randn(M, N, generator=gen).half().cuda()
+    s = 1 / (1 - p)
+    # given mask
+    mask = cpu_mask(O.mask_shape(M, K, bs), p, gen).cuda()
+    y, m2, lists, g = ext.dropout_matmul_forward(x, w, bs, p, mask=mask)
+    assert g == 64 and torch.equal(m2, mask)
+    assert torch.equal(y, ext.gemm_dsd(x, w, mask, bs, s))
+    dx, dw = ext.dropout_matmul_backward(dy, w, x, lists, g, p)
+    assert torch.equal(dx, ext.gemm_sdd(dy, w.t(), mask, bs, s))
+    assert dw.is_contiguous() and torch.equal(dw, ext.gemm_dsd(x.t(), dy.t(), mask.t(), bs, s, transposed_out=True).t())
+    only_dx, none = ext.dropout_matmul_backward(dy, w, x, lists, g, p, need_dw=False)
+    assert none is None and torch.equal(only_dx, dx)
+    # seeded draw: the mask of the oracle's generator
+    y, m3, lists, g = ext.dropout_matmul_forward(x, w, bs, p, seed=77)
+    want = O.random_mask(O.mask_shape(M, K, bs), p, 77)
+    assert np.array_equal(m3.cpu().numpy(), want)
+    assert max_tile_rel_fro(y, O.dsd_forward(to_np(x), to_np(w), want, bs, p, np.float32)) <= REL_FRO_TOL
+    # device-resident generator: follows manual_seed and advances
+    ext.manual_seed(5)
+    _, m4, _, _ = ext.dropout_matmul_forward(x, w, bs, p)
+    _, m5, _, _ = ext.dropout_matmul_forward(x, w, bs, p)
+    assert np.array_equal(m4.cpu().numpy(), O.random_mask(O.mask_shape(M, K, bs), p, 5, offset=0))
+    assert np.array_equal(m5.cpu().numpy(), O.random_mask(O.mask_shape(M, K, bs), p, 5, offset=1))
