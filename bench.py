@@ -28,15 +28,26 @@ for _p in (ROOT, ROOT / "sparse-dropout_amd"):
 
 PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA peak
 
-# HBM/fabric bytes per launch of the three GEMM kernels at the headline workload (M=N=K=8192, p=0.5),
-# from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a 128 MiB device copy in the same run
-# (profiles/bench_8192_p50_pmc.txt: read factor 2.0, write factor 1.0).  Only reported when the
-# benchmark runs that workload; a counter run cannot be made from inside this process.
-MEASURED_TRAFFIC_BYTES = {
-    "dsd_forward": int((1034.2 + 129.8) * 2**20),
-    "sdd_dx": int((2087.1 + 128.6) * 2**20),
-    "dsd_dw": int((1159.2 + 144.2) * 2**20),
-}
+# HBM/fabric bytes per launch of the three GEMM kernels at the headline workload (M=N=K=8192, p=0.5) are not
+# measured by this process (a counter run cannot be made from inside it): they are read from the stored summary of
+# the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command, profiles/bench_8192_p50_pmc.txt (its
+# "traffic_json:" line), which names the commit it was taken at; the JSON line says so next to the figure.
+TRAFFIC_FILE = ROOT / "profiles" / "bench_8192_p50_pmc.txt"
+
+
+def stored_traffic(kernel: str):
+    """(bytes per launch, provenance) of `kernel` from the stored counter summary, or (None, None)."""
+    try:
+        line = next(l for l in TRAFFIC_FILE.read_text().splitlines() if l.startswith("traffic_json:"))
+        doc = json.loads(line[len("traffic_json:"):])
+        entry = doc["kernels"][kernel]
+        return int(entry["fetch_bytes"] + entry["write_bytes"]), {
+            "file": str(TRAFFIC_FILE.relative_to(ROOT)), "taken_at_commit": doc.get("commit"),
+            "read_factor": doc.get("read_factor"), "write_factor": doc.get("write_factor")}
+    except (OSError, KeyError, ValueError, StopIteration):
+        return None, None
+
+
 METRIC = "fwd+bwd ms & effective TFLOP/s vs p (0–0.75) at 8192³ fp16; % of MFMA peak"
 
 
@@ -54,6 +65,9 @@ def _padded(t, dev):
     return view
 
 
+ZERO_DATA = False  # --zero-data: all-zero operands (same instructions and traffic, no switching activity in the multipliers)
+
+
 def make_problem(size: int, p: float, bs: int, seed: int = 0):
     import torch
 
@@ -63,6 +77,9 @@ def make_problem(size: int, p: float, bs: int, seed: int = 0):
     x = _padded(torch.randn(M, K, generator=gen).half(), dev)
     w = _padded((torch.randn(N, K, generator=gen) / K ** 0.5).half(), dev)
     dy = _padded(torch.randn(M, N, generator=gen).half(), dev)
+    if ZERO_DATA:
+        for t in (x, w, dy):
+            t.zero_()
     mask = (torch.rand(M // bs, K // bs, generator=gen) < p).to(dev)  # CPU generator: device independent
     return x, w, dy, mask
 
@@ -213,11 +230,16 @@ def main() -> int:
     ap.add_argument("--cpu-size", type=int, default=8192)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 128 MiB device copy 3 times (known traffic, for scaling rocprof's FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--dense-reference", action="store_true",
+                    help="also time the dense products on the same tensors: torch.matmul (hipBLASLt) and this library's sd_gemm")
+    ap.add_argument("--zero-data", action="store_true",
+                    help="all-zero operands: what the kernels do when the chip's power limit is out of the picture")
     ap.add_argument("--ld-pad", type=int, default=0,
                     help="pad every leading dimension by this many elements (experiment: power-of-two row strides)")
     args = ap.parse_args()
-    global LD_PAD
+    global LD_PAD, ZERO_DATA
     LD_PAD = args.ld_pad
+    ZERO_DATA = args.zero_data
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
               "(the path has no collectives: row blocks would shard over GPUs with one reduction for dW)", file=sys.stderr)
@@ -255,6 +277,8 @@ def main() -> int:
     }
     dominant = max(("dsd_forward", "sdd_dx", "dsd_dw"), key=lambda k: kern_ms[k])
     achieved = step.flops_fwd / (kern_ms[dominant] * 1e-3) / 1e12  # each GEMM does 2*kept_area*N flops
+    headline = size == 8192 and args.p == 0.5 and bs == 64 and LD_PAD == 0 and not ZERO_DATA
+    traffic, traffic_source = stored_traffic(dominant) if headline else (None, None)
     roofline = {
         "bound": "mfma",
         "kernel": dominant,
@@ -262,8 +286,10 @@ def main() -> int:
         "peak": PEAK_FP16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": round(achieved / PEAK_FP16_TFLOPS, 4),
-        "traffic": MEASURED_TRAFFIC_BYTES.get(dominant) if (size == 8192 and args.p == 0.5 and bs == 64 and LD_PAD == 0) else None,
-        "traffic_unit": "bytes per launch (HBM/fabric reads + writes, rocprofv3 FETCH_SIZE/WRITE_SIZE, see profiles/)",
+        "traffic": traffic,
+        "traffic_unit": "bytes per launch (HBM/fabric reads + writes); not measured by this run: stored rocprofv3 "
+                        "FETCH_SIZE/WRITE_SIZE figures of the same command, see traffic_source",
+        "traffic_source": traffic_source,
         "flops_per_launch": step.flops_fwd,
         "avg_launch_ms": round(kern_ms[dominant], 4),
         "all_kernels_ms": {k: round(v, 4) for k, v in kern_ms.items()},
@@ -304,6 +330,25 @@ def main() -> int:
         ratio = round(t_by_p[0.5] / t_by_p[0.0], 4)
         del flush
 
+    dense_reference = None
+    if args.dense_reference:
+        flush = torch.empty(512 << 20, dtype=torch.int8, device="cuda")
+        x, w, dy = step.x, step.w, step.dy
+        y = torch.empty_like(step.y)
+        for _ in range(3):  # library heuristics and kernel loading happen on the first calls
+            torch.matmul(x, w.t(), out=y)
+            step.ext.gemm(x, w, out=y)
+            step.ext.gemm(dy, w.t(), out=step.dx)
+        torch.cuda.synchronize()
+        dense_reference = {
+            "workload": f"one dense product Y = X.W^T at M=N=K={size} on the benchmark's tensors, L2 flushed before each call, "
+                        "HIP-event average",
+            "torch_matmul_ms": round(time_kernel_events(lambda: torch.matmul(x, w.t(), out=y), reps, flush), 4),
+            "sd_gemm_ms": round(time_kernel_events(lambda: step.ext.gemm(x, w, out=y), reps, flush), 4),
+            "sd_gemm_dx_layout_ms": round(time_kernel_events(lambda: step.ext.gemm(dy, w.t(), out=step.dx), reps, flush), 4),
+        }
+        del flush
+
     out = {
         "metric": METRIC,
         "value": round(value, 2),
@@ -329,6 +374,10 @@ def main() -> int:
         "sweep": sweep,
         "roofline": roofline,
     }
+    if ZERO_DATA:
+        out["data"] = "synthetic, all-zero operands (--zero-data)"
+    if dense_reference is not None:
+        out["dense_reference"] = dense_reference
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.cpu_size, bs, args.p, reps=4)
     print(json.dumps(out))
