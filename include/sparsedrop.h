@@ -52,6 +52,9 @@ enum sd_status {
 
 enum sd_dtype { SD_F16 = 0, SD_BF16 = 1 };
 
+/* activations the GEMM epilogues can apply; GELU is the exact (erf) form, torch.nn.GELU's default */
+enum sd_act { SD_ACT_NONE = 0, SD_ACT_RELU = 1, SD_ACT_GELU = 2 };
+
 /* Library version (major*10000 + minor*100 + patch). No reference counterpart. */
 int sd_version(void);
 
@@ -247,6 +250,33 @@ int sd_gemm_sdd_lists_ex(const void* A, int64_t a_stride_r, int64_t a_stride_c,
                          const int32_t* row_ptr, const int32_t* col_idx,
                          int64_t M, int64_t N, int64_t K, int64_t block_size, float scale, int dtype,
                          int kept_only, float keep_hint, void* stream);
+
+/* The two products with the activation that sits between dropout-linear layers fused into their stores (the
+ * reference's models interleave exactly these: eval/mlp/model.py:21-28 DropoutMM, ReLU, DropoutMM, ...;
+ * eval/llm/model.py:58-60 Linear, GELU, DropoutMM; its kernels have no epilogue, gemm.cuh:55-66):
+ *   sd_gemm_dsd_lists_act:      C = act(v), v = scale * sum over kept blocks, applied to the fp32 accumulator before
+ *                               the one rounding; pre_out (NULL, or a matrix of C's shape with its own strides)
+ *                               receives v itself, which the GELU backward needs.
+ *   sd_gemm_sdd_lists_actgrad:  C = v * act'(act_at[m, n]) where kept, exactly 0 where dropped: the input gradient
+ *                               of a layer whose input was act(act_at), i.e. the gradient with respect to the
+ *                               previous layer's pre-activation.  For ReLU act_at may be the activated tensor itself
+ *                               (same sign).  act_at has C's shape and its own strides.
+ * act = SD_ACT_NONE makes them sd_gemm_dsd_lists / sd_gemm_sdd_lists_ex. */
+int sd_gemm_dsd_lists_act(const void* A, int64_t a_stride_r, int64_t a_stride_c,
+                          const void* B, int64_t b_stride_r, int64_t b_stride_c,
+                          void* C, int64_t c_stride_r, int64_t c_stride_c,
+                          const int32_t* row_ptr, const int32_t* col_idx,
+                          int64_t M, int64_t N, int64_t K, int64_t block_size, float scale, int dtype,
+                          int act, void* pre_out, int64_t pre_stride_r, int64_t pre_stride_c,
+                          void* workspace, int64_t workspace_bytes, void* stream);
+
+int sd_gemm_sdd_lists_actgrad(const void* A, int64_t a_stride_r, int64_t a_stride_c,
+                              const void* B, int64_t b_stride_r, int64_t b_stride_c,
+                              void* C, int64_t c_stride_r, int64_t c_stride_c,
+                              const int32_t* row_ptr, const int32_t* col_idx,
+                              int64_t M, int64_t N, int64_t K, int64_t block_size, float scale, int dtype,
+                              int act, const void* act_at, int64_t at_stride_r, int64_t at_stride_c,
+                              float keep_hint, void* stream);
 
 /* sd_gemm_sdd_lists for a consumer that reads kept tiles only (sd_col2im with the same mask does): the
  * dropped tiles of C are left untouched instead of being written as zeros, which for half of a large C

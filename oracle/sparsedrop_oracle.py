@@ -31,6 +31,11 @@ Parity status of each function (what pins it is in tests/test_oracle.py):
                                            random STREAM is not part of the contract (parity is defined for
                                            a given mask), only the distribution is
   split_mask                               pinned: expand_keep identity (same element mask at both sizes)
+  act_apply / act_grad / dsd_forward_act /
+  sdd_dx_actgrad / mlp_forward_backward    pinned: torch's relu / gelu (erf form) and their autograd derivatives;
+                                           the MLP against torch autograd through the literal naive.py
+                                           restatement with torch activations in between (the composition the
+                                           reference's models make, eval/mlp/model.py:31-40, eval/llm/model.py:58-66)
 No function here is "parity unpinned".
 """
 from __future__ import annotations
@@ -54,6 +59,11 @@ __all__ = [
     "dsd_forward",
     "sdd_dx",
     "dsd_dw",
+    "act_apply",
+    "act_grad",
+    "dsd_forward_act",
+    "sdd_dx_actgrad",
+    "mlp_forward_backward",
     "conv_out_hw",
     "im2col",
     "col2im",
@@ -232,6 +242,89 @@ def dsd_dw(dy, x, mask, block_size: int, p: float, dtype=np.float64) -> np.ndarr
     dy = np.asarray(dy, dtype=dtype)
     mask = np.asarray(mask, dtype=bool)
     return gemm_dsd(x.T, dy.T, mask.T, block_size, 1.0 / (1.0 - p), dtype).T
+
+
+# --------------------------------------------------------------------------------------
+# activations between dropout-linear layers (what the fused epilogues compute)
+# --------------------------------------------------------------------------------------
+_erf = np.vectorize(math.erf, otypes=[np.float64])
+
+
+def act_apply(x, act: str | None) -> np.ndarray:
+    """relu(x) = max(x, 0); gelu(x) = x * Phi(x), the exact (erf) form that torch.nn.GELU() defaults to
+    (the reference's models: nn.ReLU eval/mlp/model.py:29, nn.GELU eval/llm/model.py:59)."""
+    x = np.asarray(x, dtype=np.float64)
+    if act in (None, "none"):
+        return x
+    if act == "relu":
+        return np.maximum(x, 0.0)
+    if act == "gelu":
+        return 0.5 * x * (1.0 + _erf(x / math.sqrt(2.0)))
+    raise ValueError(f"unknown activation {act!r}")
+
+
+def act_grad(x, act: str | None) -> np.ndarray:
+    """d act(x) / dx: relu' = [x > 0]; gelu' = Phi(x) + x * phi(x)."""
+    x = np.asarray(x, dtype=np.float64)
+    if act in (None, "none"):
+        return np.ones_like(x)
+    if act == "relu":
+        return (x > 0).astype(np.float64)
+    if act == "gelu":
+        return 0.5 * (1.0 + _erf(x / math.sqrt(2.0))) + x * np.exp(-0.5 * x * x) / math.sqrt(2.0 * math.pi)
+    raise ValueError(f"unknown activation {act!r}")
+
+
+def dsd_forward_act(x, w, mask, block_size: int, p: float, act: str | None, dtype=np.float64):
+    """(act(Y), Y) with Y = dsd_forward(...): the activation follows the dropout-linear layer
+    (eval/mlp/model.py:33-34: ``x = self.in_proj(x); x = self.act(x)``)."""
+    pre = dsd_forward(x, w, mask, block_size, p, np.float64)
+    return act_apply(pre, act).astype(dtype), pre.astype(dtype)
+
+
+def sdd_dx_actgrad(dy, w, mask, block_size: int, p: float, act: str | None, act_at, dtype=np.float64):
+    """Input gradient of a dropout-linear layer whose input was act(act_at), taken one step further to the
+    gradient with respect to act_at: sdd_dx(...) * act'(act_at) (chain rule through eval/mlp/model.py:34)."""
+    dx = sdd_dx(dy, w, mask, block_size, p, np.float64)
+    return (dx * act_grad(act_at, act)).astype(dtype)
+
+
+def mlp_forward_backward(x, weights, masks, block_size: int, p: float, act: str | None, dy, dtype=np.float64,
+                         hidden_dtype=None):
+    """The reference's MLPs (eval/mlp/model.py:31-40; eval/llm/model.py:62-66): dropout-linear layers with an
+    activation between consecutive ones (none after the last).  Returns (out, dx, [dW_i]) for the upstream
+    gradient dy, by the chain rule over dsd_forward / sdd_dx / dsd_dw.
+
+    ``hidden_dtype`` (e.g. np.float16): hidden tensors are stored in that type between layers, as they are under
+    the reference's autocast contract (blockwise_dropout_matmul_cuda.py:9): the pre-activation and the activated
+    tensor are each rounded once, the next layer and the activation's derivative see the rounded values, and the
+    backward is the exact chain rule of that computation with the roundings taken as identities.  Without it
+    nothing is rounded.  (It matters for ReLU: a rounding upstream moves pre-activations near zero across the
+    kink, which a comparison must not count as an error of the products.)"""
+    rnd = (lambda a: a) if hidden_dtype is None else (lambda a: a.astype(hidden_dtype).astype(np.float64))
+    h = np.asarray(x, dtype=np.float64)
+    inputs, pres = [], []
+    for i, (w, m) in enumerate(zip(weights, masks)):
+        inputs.append(h)
+        pre = dsd_forward(h, np.asarray(w, dtype=np.float64), m, block_size, p, np.float64)
+        if i + 1 < len(weights):
+            pres.append(rnd(pre))
+            h = rnd(act_apply(pre, act))
+        else:
+            pres.append(pre)
+            h = pre
+    out = h
+    g = np.asarray(dy, dtype=np.float64)  # gradient with respect to the current layer's pre-activation
+    dws = [None] * len(weights)
+    for i in reversed(range(len(weights))):
+        w = np.asarray(weights[i], dtype=np.float64)
+        dws[i] = dsd_dw(g, inputs[i], masks[i], block_size, p, np.float64).astype(dtype)
+        g = sdd_dx(g, w, masks[i], block_size, p, np.float64)
+        if i > 0:
+            # ReLU's derivative can be read off either tensor (same sign); GELU's is evaluated at the stored
+            # pre-activation
+            g = g * act_grad(inputs[i] if act == "relu" else pres[i - 1], act)
+    return out.astype(dtype), g.astype(dtype), dws
 
 
 # --------------------------------------------------------------------------------------

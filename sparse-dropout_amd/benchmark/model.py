@@ -8,7 +8,9 @@ Models are built from ``DropoutMM`` the way the reference's evaluation models ar
   mlp-784  the same on 4096 unresized 28x28 images with 10 unpadded classes: 784 -> 1024 -> 1024 -> 10
   vit-ffn  one transformer feed-forward block on 64x256 tokens: 384 -> 1536 -> GELU -> 384, dropout on the
            inputs of both linears
-Each is timed with variant "none" (dense), "vanilla" (element dropout + dense) and "blockwise[hip]"."""
+Each is timed with variant "none" (dense), "vanilla" (element dropout + dense), "blockwise[hip]" and
+"blockwise[hip-fused]": the same layers as one autograd function whose GEMM stores apply the activation and
+its derivative (no activation kernels in either direction)."""
 from __future__ import annotations
 
 import argparse
@@ -18,6 +20,7 @@ import time
 import torch
 from torch import nn
 
+import flash_dropout.functional as F
 from flash_dropout.layers import DropoutMM
 
 from .utils import FLUSH_BYTES
@@ -46,6 +49,31 @@ class VitFfn(nn.Module):
 
     def forward(self, x):
         return self.down(nn.functional.gelu(self.up(x)))
+
+
+class FusedStack(nn.Module):
+    """The layers of ``Mlp`` / ``VitFfn`` (same shapes, same initialisation) run through
+    ``hip_blockwise_dropout_mlp``: activation and activation gradient in the GEMM epilogues."""
+
+    def __init__(self, dims, ps, activation, block_size):
+        super().__init__()
+        self.linears = nn.ModuleList(DropoutMM(dims[i], dims[i + 1], p=ps[i], variant="none")
+                                     for i in range(len(dims) - 1))  # parameter holders
+        self.ps, self.activation, self.block_size = tuple(ps), activation, block_size
+
+    def forward(self, x):
+        lead = x.shape[:-1] if x.dim() == 3 else None
+        x2 = x.flatten(1) if lead is None else x.reshape(-1, x.shape[-1])
+        y = F.hip_blockwise_dropout_mlp(x2, [l.weight for l in self.linears], self.block_size, self.ps, self.activation)
+        return y if lead is None else y.reshape(*lead, y.shape[-1])
+
+
+def fused_variant(name, p, block_size):
+    if name == "mlp":
+        return FusedStack([1024, 1024, 1024, 128], [0.0, p, p], "relu", block_size)
+    if name == "mlp-784":
+        return FusedStack([784, 1024, 1024, 10], [0.0, p, p], "relu", block_size)
+    return FusedStack([384, 1536, 384], [p, p], "gelu", block_size)
 
 
 class Mlp784(Mlp):
@@ -119,12 +147,14 @@ def main() -> None:
         cls, make_x = MODELS[name]
         x = make_x().cuda().half()
         print(f"=== {name}  input {tuple(x.shape)}  block_size {args.block_size}{'  (graph replay)' if args.graph else ''}")
-        for variant, ps in (("none", [0.0]), ("vanilla", [0.5]), ("blockwise[hip]", args.p)):
+        for variant, ps in (("none", [0.0]), ("vanilla", [0.5]), ("blockwise[hip]", args.p),
+                            ("blockwise[hip-fused]", args.p)):
             for p in ps:
-                model = cls(variant, p, args.block_size).cuda().half().train()
+                model = (fused_variant(name, p, args.block_size) if variant.endswith("fused]")
+                         else cls(variant, p, args.block_size)).cuda().half().train()
                 ts = time_model(model, x, warmup=0.2, rep=args.rep, graph=args.graph)
                 sem = statistics.stdev(ts) / len(ts) ** 0.5 if len(ts) > 1 else 0.0
-                print(f"{variant:<16} p={p:<4} median {statistics.median(ts):8.4f} ms  "
+                print(f"{variant:<21} p={p:<4} median {statistics.median(ts):8.4f} ms  "
                       f"mean {statistics.mean(ts):8.4f} +- {1.96 * sem:.4f}  n={len(ts)}")
 
 

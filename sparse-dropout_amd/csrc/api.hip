@@ -108,6 +108,9 @@ GemmArgs make_args(const void* A, int64_t asr, int64_t asc, const void* B, int64
   g.ws_bytes = ws_ok ? ws_bytes : 0;
   g.kept_only = false;
   g.keep_hint = -1.f;
+  g.act = SD_ACT_NONE;
+  g.aux = nullptr;
+  g.aux_sr = g.aux_sc = 0;
   return g;
 }
 
@@ -307,6 +310,51 @@ int sd_gemm_sdd_lists_ex(const void* A, int64_t asr, int64_t asc, const void* B,
   GemmArgs g = make_args(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, bs, scale, row_ptr, col_idx);
   g.kept_only = kept_only != 0;
   g.keep_hint = keep_hint == keep_hint ? keep_hint : -1.f;
+  return run(g, kSdd, dtype, (hipStream_t)stream);
+}
+
+static int check_act(int act, const void* aux, int64_t xsr, int64_t xsc, int64_t M, int64_t N, bool aux_required) {
+  SD_REQUIRE(act == SD_ACT_NONE || act == SD_ACT_RELU || act == SD_ACT_GELU, "act must be SD_ACT_NONE, SD_ACT_RELU or SD_ACT_GELU (got %d)", act);
+  if (act == SD_ACT_NONE) return SD_OK;
+  SD_REQUIRE(!aux_required || aux != nullptr, "the activation gradient needs the tensor it is evaluated at");
+  if (aux) return check_mat("aux", aux, xsr, xsc, M, N);
+  return SD_OK;
+}
+
+int sd_gemm_dsd_lists_act(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc,
+                          void* C, int64_t csr, int64_t csc, const int32_t* row_ptr, const int32_t* col_idx,
+                          int64_t M, int64_t N, int64_t K, int64_t bs, float scale, int dtype, int act, void* pre_out,
+                          int64_t pre_stride_r, int64_t pre_stride_c, void* workspace, int64_t workspace_bytes,
+                          void* stream) {
+  if (int rc = check_common(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, dtype)) return rc;
+  if (int rc = check_sparse(bs, scale)) return rc;
+  SD_REQUIRE(row_ptr && col_idx, "gemm_dsd: null list");
+  if (int rc = check_act(act, pre_out, pre_stride_r, pre_stride_c, M, N, false)) return rc;
+  GemmArgs g = make_args(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, bs, scale, row_ptr, col_idx,
+                         workspace, workspace_bytes);
+  g.act = act;
+  g.aux = act != SD_ACT_NONE ? static_cast<uint16_t*>(pre_out) : nullptr;
+  g.aux_sr = pre_stride_r;
+  g.aux_sc = pre_stride_c;
+  return run(g, kDsd, dtype, (hipStream_t)stream);
+}
+
+int sd_gemm_sdd_lists_actgrad(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc,
+                              void* C, int64_t csr, int64_t csc, const int32_t* row_ptr, const int32_t* col_idx,
+                              int64_t M, int64_t N, int64_t K, int64_t bs, float scale, int dtype, int act,
+                              const void* act_at, int64_t at_stride_r, int64_t at_stride_c, float keep_hint,
+                              void* stream) {
+  if (int rc = check_common(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, dtype)) return rc;
+  if (int rc = check_sparse(bs, scale)) return rc;
+  SD_REQUIRE(row_ptr && col_idx, "gemm_sdd: null list");
+  SD_REQUIRE(!(keep_hint > 1.f), "gemm_sdd: keep_hint must be a fraction in [0, 1], or negative for unknown");
+  if (int rc = check_act(act, act_at, at_stride_r, at_stride_c, M, N, true)) return rc;
+  GemmArgs g = make_args(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, bs, scale, row_ptr, col_idx);
+  g.keep_hint = keep_hint == keep_hint ? keep_hint : -1.f;
+  g.act = act;
+  g.aux = act != SD_ACT_NONE ? const_cast<uint16_t*>(static_cast<const uint16_t*>(act_at)) : nullptr;
+  g.aux_sr = at_stride_r;
+  g.aux_sc = at_stride_c;
   return run(g, kSdd, dtype, (hipStream_t)stream);
 }
 

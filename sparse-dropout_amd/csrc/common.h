@@ -117,6 +117,12 @@ struct GemmArgs {
   int64_t ws_bytes;
   bool kept_only;    // SDD: dropped tiles of C are left untouched instead of being zeroed
   float keep_hint;   // SDD: the caller's estimate of the kept fraction of blocks (picks the workgroup shape); < 0 = unknown
+  // fused epilogue (0 = none): DSD / dense: C = act(v), and v itself to `aux` when that is given (the pre-activation
+  // the backward needs); SDD: C = v * act'(aux[m, n]) (aux: the pre-activation, or for ReLU the activated tensor).
+  // v is the scaled fp32 accumulator; aux is addressed like C but with its own strides.
+  int act;
+  uint16_t* aux;
+  int64_t aux_sr, aux_sc;
 };
 
 // Geometry of a convolution whose patch matrix the DSD kernel gathers itself (implicit GEMM):
@@ -141,6 +147,123 @@ struct ImplicitConv {
 };
 
 enum Mode { kDense = 0, kDsd = 1, kSdd = 2 };
+
+// ---- fused epilogues --------------------------------------------------------------------------
+// GELU is the exact (erf) form, torch.nn.GELU's default: gelu(x) = x * Phi(x), gelu'(x) = Phi(x) + x * phi(x).
+// Phi comes from the rational approximation of erf in Abramowitz & Stegun 7.1.26 (absolute error below 1.5e-7, far
+// under the resolution of the fp16 / bf16 results): one exponential, one reciprocal and a degree-5 polynomial, a
+// third of the instructions of erff, which matters because the epilogue of a GEMM has nothing to hide them behind.
+// *pdf receives exp(-x^2 / 2), which the derivative needs as well.
+__device__ inline float normal_cdf(float x, float* pdf) {
+  const float z = fabsf(x) * 0.70710678118654752f;
+  const float e = __expf(-z * z);
+  const float t = __builtin_amdgcn_rcpf(1.f + 0.3275911f * z);
+  const float poly = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f + t * (-1.453152027f + t * 1.061405429f))));
+  const float tail = 0.5f * poly * e;  // Phi(-|x|)
+  *pdf = e;
+  return x >= 0.f ? 1.f - tail : tail;
+}
+__device__ inline float act_apply(int act, float x) {
+  if (act == SD_ACT_RELU) return x > 0.f ? x : 0.f;
+  if (act == SD_ACT_GELU) {
+    float e;
+    return x * normal_cdf(x, &e);
+  }
+  return x;
+}
+__device__ inline float act_derivative(int act, float x) {
+  if (act == SD_ACT_RELU) return x > 0.f ? 1.f : 0.f;
+  if (act == SD_ACT_GELU) {
+    float e;
+    const float cdf = normal_cdf(x, &e);
+    return cdf + x * 0.39894228040143268f * e;
+  }
+  return 1.f;
+}
+// Stores element (m, n) of the result: v is the scaled fp32 accumulator.  SDD multiplies by the derivative of the
+// activation at aux[m, n]; the others apply the activation and, if asked, also keep v.
+template <typename T, bool SDD>
+__device__ inline void store_result(const GemmArgs& g, int64_t m, int64_t n, float v) {
+  if (g.act != SD_ACT_NONE) {
+    if (SDD) {
+      if (v != 0.f) v *= act_derivative(g.act, T::to_float(g.aux[m * g.aux_sr + n * g.aux_sc]));  // dropped tiles stay exact zeros
+    } else {
+      if (g.aux) g.aux[m * g.aux_sr + n * g.aux_sc] = T::from_float(v);
+      v = act_apply(g.act, v);
+    }
+  }
+  g.c[m * g.c_sr + n * g.c_sc] = T::from_float(v);
+}
+
+// One wave's [ROWS][COLS] tile of unscaled fp32 accumulators, staged in the wave's own LDS region (pitch COLS + 4
+// floats) with COLS running along C's contiguous index, goes out in full 16-byte pieces: a lane takes 8 consecutive
+// elements of one row, scales them, applies the fused epilogue, rounds once and stores them (128-byte lines are
+// written whole by 8 neighbouring lanes).  s0 / c0: where the tile starts along C's strided / contiguous index
+// (c0 a multiple of 8); along_n: the contiguous index is n (row-major C).  part: fp32 partial sums of a split
+// reduction go to `part` (C's element order, unscaled) instead.
+template <typename T, bool SDD, int ROWS, int COLS>
+__device__ inline void store_staged_tile(const GemmArgs& g, const float* stg, int lane, bool along_n, int64_t s0,
+                                         int64_t c0, float* part) {
+  constexpr int PITCH = COLS + 4, LPR = COLS / 8, RPP = 64 / LPR;  // lanes per row, rows per pass
+  const int64_t s_ext = along_n ? g.M : g.N, c_ext = along_n ? g.N : g.M;
+  const int64_t ld = along_n ? g.c_sr : g.c_sc, unit = along_n ? g.c_sc : g.c_sr;
+  bool vec = unit == 1 && ld % 8 == 0 && reinterpret_cast<uintptr_t>(g.c) % 16 == 0;
+  const bool has_aux = g.act != SD_ACT_NONE && g.aux != nullptr;
+  const int64_t ald = along_n ? g.aux_sr : g.aux_sc, aunit = along_n ? g.aux_sc : g.aux_sr;
+  if (has_aux) vec = vec && aunit == 1 && ald % 8 == 0 && reinterpret_cast<uintptr_t>(g.aux) % 16 == 0;
+#pragma unroll
+  for (int pass = 0; pass < ROWS / RPP; ++pass) {
+    const int row = pass * RPP + lane / LPR, ch = lane % LPR;
+    const int64_t si = s0 + row, ci = c0 + ch * 8;
+    if (si >= s_ext || ci >= c_ext) continue;
+    const f32x4 lo = *reinterpret_cast<const f32x4*>(stg + row * PITCH + ch * 8);
+    const f32x4 hi = *reinterpret_cast<const f32x4*>(stg + row * PITCH + ch * 8 + 4);
+    float r[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    const int valid = c_ext - ci < 8 ? (int)(c_ext - ci) : 8;
+    if (part) {
+      float* dst = part + si * c_ext + ci;
+      if (valid == 8 && c_ext % 4 == 0) {
+        *reinterpret_cast<f32x4*>(dst) = lo;
+        *reinterpret_cast<f32x4*>(dst + 4) = hi;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if (i < valid) dst[i] = r[i];
+      }
+      continue;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] *= g.scale;
+    if (!(vec && valid == 8)) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (i < valid) store_result<T, SDD>(g, along_n ? si : ci + i, along_n ? ci + i : si, r[i]);
+      continue;
+    }
+    auto pack = [&](const float (&v)[8]) {
+      return u32x4{(uint32_t)T::from_float(v[0]) | ((uint32_t)T::from_float(v[1]) << 16),
+                   (uint32_t)T::from_float(v[2]) | ((uint32_t)T::from_float(v[3]) << 16),
+                   (uint32_t)T::from_float(v[4]) | ((uint32_t)T::from_float(v[5]) << 16),
+                   (uint32_t)T::from_float(v[6]) | ((uint32_t)T::from_float(v[7]) << 16)};
+    };
+    if (g.act != SD_ACT_NONE) {
+      if (SDD) {
+        const u32x4 a = *reinterpret_cast<const u32x4*>(g.aux + si * ald + ci);
+        const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const uint16_t h = (uint16_t)(i & 1 ? w[i / 2] >> 16 : w[i / 2] & 0xffffu);
+          if (r[i] != 0.f) r[i] *= act_derivative(g.act, T::to_float(h));  // dropped tiles stay exact zeros
+        }
+      } else {
+        if (has_aux) *reinterpret_cast<u32x4*>(g.aux + si * ald + ci) = pack(r);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r[i] = act_apply(g.act, r[i]);
+      }
+    }
+    *reinterpret_cast<u32x4*>(g.c + si * ld + ci) = pack(r);
+  }
+}
 
 // launchers (one per translation unit)
 int launch_generic(const GemmArgs& g, int mode, int dtype, hipStream_t stream);

@@ -241,7 +241,7 @@ __global__ __launch_bounds__(THREADS) void gemm_generic_kernel(GemmArgs g, int t
           const int64_t e = TRANS_OUT ? n * g.M + m : m * g.N + n;
           g.ws[(int64_t)blockIdx.y * g.M * g.N + e] = acc[j][v];
         } else {
-          g.c[m * g.c_sr + n * g.c_sc] = T::from_float(acc[j][v] * g.scale);
+          store_result<T, MODE == kSdd>(g, m, n, acc[j][v] * g.scale);
         }
       }
     }
@@ -288,7 +288,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs g, int spli
     const float sum = ((acc[v] + part[0][lane * 4 + v]) + part[1][lane * 4 + v]) + part[2][lane * 4 + v];
     const int64_t m = trans ? e % g.M : e / g.N;
     const int64_t n = trans ? e / g.M : e % g.N;
-    g.c[m * g.c_sr + n * g.c_sc] = T::from_float(sum * g.scale);
+    store_result<T, false>(g, m, n, sum * g.scale);  // only DSD and dense products split their reduction
   }
 }
 

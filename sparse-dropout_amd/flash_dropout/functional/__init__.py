@@ -3,6 +3,7 @@ are kept; ``cuda_blockwise_dropout_matmul`` and ``triton_blockwise_dropout_matmu
 the HIP implementation (there is one kernel backend here, not three)."""
 from .blockwise_dropout_matmul_hip import blockwise_dropout_matmul as hip_blockwise_dropout_matmul
 from .blockwise_dropout_matmul_hip import blockwise_dropout_matmul_mask as hip_blockwise_dropout_matmul_mask
+from .blockwise_dropout_mlp_hip import blockwise_dropout_mlp as hip_blockwise_dropout_mlp
 from .im2col_conv2d import (
     blockwise_dropout_conv2d,
     blockwise_dropout_conv2d_mask,

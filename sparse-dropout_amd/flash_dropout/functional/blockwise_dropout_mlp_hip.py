@@ -1,0 +1,123 @@
+"""A stack of dropout-linear layers with an activation between consecutive ones, as ONE autograd function whose
+GEMM epilogues do the activation work.
+
+The reference's models interleave exactly this (eval/mlp/model.py:31-40: DropoutMM, ReLU, DropoutMM, ..., DropoutMM;
+eval/llm/model.py:62-66: DropoutMM, GELU, DropoutMM) as separate modules, i.e. one elementwise kernel per
+activation in forward and one in backward, each a full pass over the hidden activations.  Here
+
+    forward   h_{i+1} = act(s_i (keep_i ⊙ h_i) W_i^T)     the activation is applied to the fp32 accumulator in the
+                                                            DSD kernel's store (sd_gemm_dsd_lists_act)
+    backward  g_{i-1} = (s_i (g_i W_i) ⊙ keep_i) ⊙ act'     the derivative is multiplied in the SDD kernel's store
+                                                            (sd_gemm_sdd_lists_actgrad); g_i is the gradient with
+                                                            respect to layer i's pre-activation
+              dW_i    = s_i g_i^T (keep_i ⊙ h_i)
+
+so no activation kernel is launched in either direction.  ReLU's derivative is read off the activated tensor
+(already kept as the next layer's input); GELU keeps the pre-activation as well.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..hip.binding_gemm import GEMM, KeptLists, _activation, _block_size, as_matrix
+from .blockwise_dropout_matmul_hip import _apply_outside_autocast
+
+
+class BlockwiseDropoutMLPHIP(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input: torch.Tensor, block_size: int, ps: tuple, activation, seed, masks, *weights):
+        ext = GEMM()
+        n = len(weights)
+        h = input
+        saved, shapes, kbs = [input], [], []
+        for i, w in enumerate(weights):
+            p = ps[i]
+            mask, lists, kernel_bs = ext.kept_lists(h.shape[0], h.shape[1], block_size,
+                                                    None if masks is None else masks[i], p,
+                                                    None if seed is None else seed + i, h.device)
+            last = i + 1 == n
+            out, pre = ext.gemm_dsd_lists_act(h, w, lists, kernel_bs, 1.0 / (1.0 - p), None if last else activation,
+                                              want_pre=(not last and activation == "gelu"))
+            # per layer: weight, mask, the four list arrays, what the activation's derivative is evaluated at
+            # (GELU: the pre-activation; ReLU: nothing extra, the activated output is the next layer's input)
+            saved += [w, mask, lists.row_ptr, lists.col_idx, lists.col_ptr, lists.row_idx]
+            saved.append(pre if pre is not None else out.new_empty(0))
+            if not last:
+                saved.append(out)
+            shapes.append(lists.shape)
+            kbs.append(kernel_bs)
+            h = out
+        ctx.save_for_backward(*saved)
+        ctx.n, ctx.ps, ctx.activation, ctx.shapes, ctx.kbs = n, ps, activation, shapes, kbs
+        return h
+
+    @staticmethod
+    def backward(ctx, grad_output: torch.Tensor):
+        ext = GEMM()
+        t = ctx.saved_tensors
+        n, act = ctx.n, ctx.activation
+        # unpack: input, then per layer (w, mask, row_ptr, col_idx, col_ptr, row_idx, pre, [out])
+        hs, layers, pos = [t[0]], [], 1
+        for i in range(n):
+            w, _, rp, ci, cp, ri, pre = t[pos:pos + 7]
+            pos += 7
+            layers.append((w, KeptLists(rp, ci, cp, ri, ctx.shapes[i]), pre))
+            if i + 1 < n:
+                hs.append(t[pos])
+                pos += 1
+        g = grad_output if grad_output.dtype == hs[0].dtype else grad_output.to(hs[0].dtype)
+        g = as_matrix(g)
+        grads_w = [None] * n
+        for i in reversed(range(n)):
+            w, lists, _ = layers[i]
+            scale = 1.0 / (1.0 - ctx.ps[i])
+            need_w = ctx.needs_input_grad[6 + i]
+            need_in = i > 0 or ctx.needs_input_grad[0]
+            if w.shape[0] % 8:  # a narrow head: zero-padded copies keep both products on the specialised kernels
+                n_pad = (w.shape[0] + 7) // 8 * 8
+                gp = g.new_zeros((g.shape[0], n_pad))
+                gp[:, : w.shape[0]] = g
+                wp = w.new_zeros((n_pad, w.shape[1]))
+                wp[: w.shape[0]] = w
+                g, w = gp, wp
+            if need_w:
+                dw = ext.gemm_dsd_lists(hs[i].t(), g.t(), lists.transposed(), ctx.kbs[i], scale, transposed_out=True).t()
+                grads_w[i] = dw[: layers[i][0].shape[0]]
+            if not need_in:
+                break
+            if i > 0:
+                prev_pre = layers[i - 1][2]
+                at = prev_pre if prev_pre.numel() else hs[i]  # GELU: pre-activation; ReLU: the activated input
+                g = ext.gemm_sdd_lists_actgrad(g, w.t(), lists, ctx.kbs[i], scale, act, at, keep_hint=1.0 / scale)
+            else:
+                g = ext.gemm_sdd_lists(g, w.t(), lists, ctx.kbs[i], scale, keep_hint=1.0 / scale)
+        grad_in = g if ctx.needs_input_grad[0] else None
+        return (grad_in, None, None, None, None, None, *grads_w)
+
+
+def blockwise_dropout_mlp(input: torch.Tensor, weights, block_size, p, activation: str | None = "relu",
+                          masks=None, seed: int | None = None) -> torch.Tensor:
+    """``W_n drop(act(... W_2 drop(act(W_1 drop(x))) ...))``: every layer drops blocks of its INPUT with
+    probability p (a number, or one per layer; 0 keeps everything) and scales by 1/(1-p), ``activation``
+    ("relu", "gelu" or None) sits between consecutive layers, none after the last.  ``masks`` (one bool mask per
+    layer, True = dropped) pins the masks, ``seed`` pins the draws (layer i uses seed + i); otherwise they come
+    from the device-resident generator.  ``input`` is [M, K], ``weights[i]`` is [out_i, in_i]."""
+    weights = list(weights)
+    if not weights:
+        raise ValueError("at least one layer is needed")
+    ps = tuple(float(p) for _ in weights) if isinstance(p, (int, float)) else tuple(float(v) for v in p)
+    if len(ps) != len(weights) or any(not 0 <= v < 1 for v in ps):
+        raise ValueError("p must be one probability in [0, 1), or one per layer")
+    _activation(activation)
+    if masks is not None and len(masks) != len(weights):
+        raise ValueError("one mask per layer is needed")
+    bs = _block_size(block_size)
+    if input.dim() != 2 or any(w.dim() != 2 for w in weights):
+        raise ValueError("input must be [M, K] and every weight [out, in]")
+    tensors = [input, *weights]
+    if torch.is_autocast_enabled("cuda"):  # the autocast contract of the single layer (…_cuda.py:9)
+        dt = torch.get_autocast_dtype("cuda")
+        tensors = [t.to(dt) for t in tensors]
+    x, *ws = (as_matrix(t) for t in tensors)
+    return _apply_outside_autocast(BlockwiseDropoutMLPHIP, x, bs, ps, activation, seed,
+                                   None if masks is None else tuple(masks), *ws)

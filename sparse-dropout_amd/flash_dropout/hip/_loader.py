@@ -51,6 +51,10 @@ SIGNATURES = {
                                   c_int64, c_int64, c_float, c_int, c_void_p]),
     "sd_gemm_sdd_lists_ex": (c_int, [*_mat, *_mat, *_mat, c_void_p, c_void_p, c_int64, c_int64,
                                      c_int64, c_int64, c_float, c_int, c_int, c_float, c_void_p]),
+    "sd_gemm_dsd_lists_act": (c_int, [*_mat, *_mat, *_mat, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                      c_float, c_int, c_int, *_mat, c_void_p, c_int64, c_void_p]),
+    "sd_gemm_sdd_lists_actgrad": (c_int, [*_mat, *_mat, *_mat, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                          c_float, c_int, c_int, *_mat, c_float, c_void_p]),
     "sd_gemm_sdd_lists_kept": (c_int, [*_mat, *_mat, *_mat, c_void_p, c_void_p, c_int64, c_int64,
                                   c_int64, c_int64, c_float, c_int, c_void_p]),
     "sd_dropout_matmul_forward": (c_int, [*_mat, *_mat, *_mat, *_mat, c_void_p, c_uint64, c_uint64, c_float, c_void_p,

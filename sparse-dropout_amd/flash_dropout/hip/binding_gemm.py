@@ -22,6 +22,13 @@ from . import _loader
 
 SD_F16, SD_BF16 = 0, 1
 _DTYPES = {torch.float16: SD_F16, torch.bfloat16: SD_BF16}
+ACTIVATIONS = {None: 0, "none": 0, "relu": 1, "gelu": 2}  # enum sd_act
+
+
+def _activation(act) -> int:
+    if act not in ACTIVATIONS:
+        raise ValueError(f"activation {act!r}: expected one of {sorted(k for k in ACTIVATIONS if k)} or None")
+    return ACTIVATIONS[act]
 
 
 class SparseDropError(RuntimeError):
@@ -454,6 +461,55 @@ class GEMM:
             self._call(self.lib.sd_gemm_sdd_lists_ex, *_mat(A), *_mat(B), *_mat(C), lists.row_ptr.data_ptr(),
                        lists.col_idx.data_ptr(), M, N, K, bs, float(scale), _DTYPES[A.dtype],
                        1 if kept_only else 0, -1.0 if keep_hint is None else float(keep_hint), self._stream(A))
+        return C
+
+    # ------------------------------------------------------------------ products with a fused activation
+    def gemm_dsd_lists_act(self, A, B, lists: KeptLists, block_size, scale, act, want_pre: bool = False):
+        """``act(scale * (A ⊙ keep) @ B.T)`` with the activation ("relu", "gelu" in its erf form, or None) applied
+        to the fp32 accumulator in the kernel's store -> (activated, pre-activation or None).  The pre-activation
+        is what the GELU backward is evaluated at; ReLU's can use the activated tensor."""
+        self._check_pair(A, B)
+        bs = _block_size(block_size)
+        code = _activation(act)
+        M, N, K = A.shape[0], B.shape[0], A.shape[1]
+        want = (ceil(M / bs), ceil(K / bs))
+        if tuple(lists.shape) != want:
+            raise ValueError(f"lists are for a {lists.shape} mask, operands need {want}")
+        C = torch.empty((M, N), dtype=A.dtype, device=A.device)
+        pre = torch.empty((M, N), dtype=A.dtype, device=A.device) if (want_pre and code) else None
+        if M == 0 or N == 0:
+            return C, pre
+        ws, ws_ptr, ws_bytes = self._splitk_scratch(A, B, bs, 1)
+        with _guard(A.device):
+            self._call(self.lib.sd_gemm_dsd_lists_act, *_mat(A), *_mat(B), *_mat(C), lists.row_ptr.data_ptr(),
+                       lists.col_idx.data_ptr(), M, N, K, bs, float(scale), _DTYPES[A.dtype], code,
+                       *(_mat(pre) if pre is not None else (None, 0, 0)), ws_ptr, ws_bytes, self._stream(A))
+        return C, (pre if code else (C if want_pre else None))
+
+    def gemm_sdd_lists_actgrad(self, A, B, lists: KeptLists, block_size, scale, act, act_at: torch.Tensor,
+                               keep_hint: float | None = None):
+        """``scale * (A @ B.T) ⊙ keep ⊙ act'(act_at)``: the input gradient of a layer whose input was
+        ``act(act_at)``, carried through to ``act_at`` in the kernel's store.  ``act_at`` is [M, N] like the
+        result; for "relu" it may be the activated tensor itself."""
+        self._check_pair(A, B)
+        bs = _block_size(block_size)
+        code = _activation(act)
+        M, N, K = A.shape[0], B.shape[0], A.shape[1]
+        want = (ceil(M / bs), ceil(N / bs))
+        if tuple(lists.shape) != want:
+            raise ValueError(f"lists are for a {lists.shape} mask, operands need {want}")
+        if code:
+            _check_operand("act_at", act_at)
+            if tuple(act_at.shape) != (M, N) or act_at.dtype != A.dtype or act_at.device != A.device:
+                raise ValueError(f"act_at must be a [{M}, {N}] {A.dtype} tensor on {A.device}")
+        C = torch.empty((M, N), dtype=A.dtype, device=A.device)
+        if M == 0 or N == 0:
+            return C
+        with _guard(A.device):
+            self._call(self.lib.sd_gemm_sdd_lists_actgrad, *_mat(A), *_mat(B), *_mat(C), lists.row_ptr.data_ptr(),
+                       lists.col_idx.data_ptr(), M, N, K, bs, float(scale), _DTYPES[A.dtype], code,
+                       *(_mat(act_at) if code else (None, 0, 0)), -1.0 if keep_hint is None else float(keep_hint),
+                       self._stream(A))
         return C
 
     # ------------------------------------------------------------------ the autograd function's two calls

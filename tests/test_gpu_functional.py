@@ -277,3 +277,107 @@ def test_fused_forward_and_backward_calls_match_the_separate_ones(bs):
     _, m5, _, _ = ext.dropout_matmul_forward(x, w, bs, p)
     assert np.array_equal(m4.cpu().numpy(), O.random_mask(O.mask_shape(M, K, bs), p, 5, offset=0))
     assert np.array_equal(m5.cpu().numpy(), O.random_mask(O.mask_shape(M, K, bs), p, 5, offset=1))
+
+
+@pytest.mark.parametrize("act", ["relu", "gelu"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fused_activation_products_against_the_oracle(act, dtype):
+    """sd_gemm_dsd_lists_act (activation on the fp32 accumulator in the store, pre-activation kept on request) and
+    sd_gemm_sdd_lists_actgrad (derivative multiplied in the store, dropped tiles exactly zero) against the oracle's
+    closed forms, on a shape with ragged edges in every dimension."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(16)
+    M, K, N, p = 1000, 456, 328, 0.5
+    x = torch.randn(M, K, generator=gen).to(dtype)
+    w = (torch.randn(N, K, generator=gen) * K ** -0.5).to(dtype)
+    mk = cpu_mask(O.mask_shape(M, K, 64), p, gen)
+    lists = ext.build_lists(mk.cuda())
+    s = 1 / (1 - p)
+    y, pre = ext.gemm_dsd_lists_act(x.cuda(), w.cuda(), lists, 64, s, act, want_pre=True)
+    assert ext.last_kernel() == "specialised"
+    ry, rpre = O.dsd_forward_act(to_np(x), to_np(w), mk.numpy(), 64, p, act, np.float32)
+    assert max_tile_rel_fro(pre, rpre) <= REL_FRO_TOL
+    assert max_tile_rel_fro(y, ry) <= REL_FRO_TOL
+    if act == "relu":
+        assert (y >= 0).all()
+    # input gradient carried to the previous pre-activation: dX[M, K] * act'(at[M, K])
+    dy = torch.randn(M, N, generator=gen).to(dtype)
+    at = torch.randn(M, K, generator=gen).to(dtype)
+    dx = ext.gemm_sdd_lists_actgrad(dy.cuda(), w.cuda().t(), lists, 64, s, act, at.cuda(), keep_hint=1 - p)
+    assert ext.last_kernel() == "specialised"
+    rdx = O.sdd_dx_actgrad(to_np(dy), to_np(w), mk.numpy(), 64, p, act, to_np(at), np.float32)
+    assert max_tile_rel_fro(dx, rdx) <= REL_FRO_TOL
+    keep = O.expand_keep(mk.numpy(), 64, M, K)
+    assert (to_np(dx)[~keep] == 0).all()
+    # act = None is the plain product
+    y0, none = ext.gemm_dsd_lists_act(x.cuda(), w.cuda(), lists, 64, s, None)
+    assert none is None and torch.equal(y0, ext.gemm_dsd_lists(x.cuda(), w.cuda(), lists, 64, s))
+
+
+@pytest.mark.parametrize("act,dims,rows", [("relu", (784, 1024, 1024, 10), 4096), ("gelu", (384, 1536, 384), 16384),
+                                            (None, (192, 128, 72), 300)])
+def test_fused_mlp_against_the_oracle_and_the_unfused_layers(act, dims, rows):
+    """The MLP-on-images and transformer-FFN configurations as one autograd function with fused activation
+    epilogues: output, input gradient and every weight gradient against the oracle's chain rule under the same
+    masks, and against the unfused composition (separate layers + torch activations)."""
+    import flash_dropout.functional as F
+
+    gen = torch.Generator().manual_seed(17)
+    p = 0.5
+    x = (torch.rand(rows, dims[0], generator=gen) if act == "relu" else torch.randn(rows, dims[0], generator=gen)).half()
+    ws = [((torch.rand(dims[i + 1], dims[i], generator=gen) * 2 - 1) * dims[i] ** -0.5).half() for i in range(len(dims) - 1)]
+    masks = [cpu_mask(O.mask_shape(rows, dims[i], 64), p, gen) for i in range(len(ws))]
+    dy = torch.randn(rows, dims[-1], generator=gen).half()
+    xg = x.cuda().requires_grad_()
+    wg = [w.cuda().requires_grad_() for w in ws]
+    out = F.hip_blockwise_dropout_mlp(xg, wg, 64, p, act, masks=[m.cuda() for m in masks])
+    out.backward(dy.cuda())
+    # hidden tensors live in fp16 between the layers, in the oracle as on the device
+    rout, rdx, rdws = O.mlp_forward_backward(to_np(x), [to_np(w) for w in ws], [m.numpy() for m in masks], 64, p, act,
+                                             to_np(dy), np.float32, hidden_dtype=np.float16)
+    assert max_tile_rel_fro(out, rout) <= REL_FRO_TOL
+    assert max_tile_rel_fro(xg.grad, rdx) <= REL_FRO_TOL
+    for got, ref in zip(wg, rdws):
+        assert got.grad.shape == ref.shape
+        assert max_tile_rel_fro(got.grad, ref) <= REL_FRO_TOL
+    # the unfused composition (it rounds the hidden pre-activations to fp16 before activating them)
+    x2 = x.cuda().requires_grad_()
+    w2 = [w.cuda().requires_grad_() for w in ws]
+    f = {"relu": torch.relu, "gelu": torch.nn.functional.gelu, None: lambda t: t}[act]
+    h = x2
+    for i, w in enumerate(w2):
+        h = F.hip_blockwise_dropout_matmul_mask(h, masks[i].cuda(), 64, p, w)
+        if i + 1 < len(w2):
+            h = f(h)
+    h.backward(dy.cuda())
+    assert rel_fro(out, h.float()) <= 2e-3
+    assert rel_fro(xg.grad, x2.grad.float()) <= 4e-3
+    for a, b in zip(wg, w2):
+        assert rel_fro(a.grad, b.grad.float()) <= 4e-3
+
+
+@pytest.mark.parametrize("name", ["mlp", "mlp-784", "vit-ffn"])
+def test_model_harness_runs_every_variant(name):
+    """benchmark/model.py (the reference's benchmark/model.py:119-229 protocol): every variant of every model
+    steps forward and backward, eagerly and as a replayed graph, and the fused stack agrees with the layer-by-layer
+    model when both are given the same weights and no dropout."""
+    from benchmark import model as bm
+
+    cls, make_x = bm.MODELS[name]
+    torch.manual_seed(0)
+    x = make_x().cuda().half()
+    for variant in ("none", "vanilla", "blockwise[hip]", "blockwise[hip-fused]"):
+        net = (bm.fused_variant(name, 0.5, 64) if variant.endswith("fused]") else cls(variant, 0.5, 64)).cuda().half().train()
+        ts = bm.time_model(net, x, warmup=0.0, rep=0.0, graph=False)
+        assert len(ts) >= 5 and all(t > 0 for t in ts)
+    fused = bm.fused_variant(name, 0.5, 64).cuda().half().train()
+    assert len(bm.time_model(fused, x, warmup=0.0, rep=0.0, graph=True)) >= 5
+    # p = 0: the fused stack is the dense model
+    fused0 = bm.fused_variant(name, 0.0, 64).cuda().half().train()
+    plain = cls("none", 0.0, 64).cuda().half().train()
+    mods = list(plain.linears) if hasattr(plain, "linears") else [plain.up, plain.down]
+    for a, b in zip(fused0.linears, mods):
+        b.weight.data.copy_(a.weight.data)
+    assert rel_fro(fused0(x), plain(x).float()) <= 3e-3

@@ -293,3 +293,100 @@ def test_split_mask_expands_to_the_same_elements(m, k, bs, split):
     fine = O.split_mask(mask, split, O.mask_shape(m, k, bs // split))
     assert fine.shape == O.mask_shape(m, k, bs // split)
     assert np.array_equal(O.expand_keep(mask, bs, m, k), O.expand_keep(fine, bs // split, m, k))
+
+
+@pytest.mark.parametrize("act", ["relu", "gelu"])
+def test_activations_match_torch_and_its_autograd(act):
+    """act_apply / act_grad against the library routines (torch.relu, torch's erf-form gelu) and their autograd
+    derivatives, over a range that covers both tails and the origin."""
+    x = torch.linspace(-6, 6, 1201, dtype=torch.float64, requires_grad=True)
+    y = torch.relu(x) if act == "relu" else torch.nn.functional.gelu(x)
+    y.sum().backward()
+    np.testing.assert_allclose(O.act_apply(x.detach().numpy(), act), y.detach().numpy(), rtol=1e-12, atol=1e-14)
+    np.testing.assert_allclose(O.act_grad(x.detach().numpy(), act), x.grad.numpy(), rtol=1e-12, atol=1e-14)
+    # known values: gelu(0) = 0, gelu'(0) = 1/2, relu'(0) = 0 (torch's convention)
+    assert O.act_apply(np.zeros(1), act)[0] == 0.0
+    assert O.act_grad(np.zeros(1), act)[0] == (0.5 if act == "gelu" else 0.0)
+
+
+@pytest.mark.parametrize("act", ["relu", "gelu", None])
+def test_mlp_chain_rule_vs_autograd_of_the_naive_restatement(act):
+    """mlp_forward_backward, dsd_forward_act and sdd_dx_actgrad against torch autograd through the literal
+    restatement of the reference's naive layer with torch activations in between: the composition the
+    reference's models make (eval/mlp/model.py:31-40)."""
+    from oracle import naive_torch
+
+    gen = torch.Generator().manual_seed(31)
+    bs, p = 4, 0.4
+    dims = [16, 24, 12, 8]
+    m = 20
+    x = torch.randn(m, dims[0], generator=gen, dtype=torch.float64, requires_grad=True)
+    ws = [torch.randn(dims[i + 1], dims[i], generator=gen, dtype=torch.float64, requires_grad=True) for i in range(3)]
+    masks = [torch.rand(m // bs, dims[i] // bs, generator=gen) < p for i in range(3)]
+    dy = torch.randn(m, dims[-1], generator=gen, dtype=torch.float64)
+    f = {"relu": torch.relu, "gelu": torch.nn.functional.gelu, None: lambda t: t}[act]
+    h = x
+    pres = []
+    for i in range(3):
+        pre = naive_torch.forward(h, ws[i], masks[i], bs, p)
+        pres.append(pre)
+        h = f(pre) if i < 2 else pre
+    h.backward(dy)
+    out, dx, dws = O.mlp_forward_backward(x.detach().numpy(), [w.detach().numpy() for w in ws],
+                                          [mk.numpy() for mk in masks], bs, p, act, dy.numpy())
+    np.testing.assert_allclose(out, h.detach().numpy(), rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(dx, x.grad.numpy(), rtol=1e-10, atol=1e-12)
+    for got, w in zip(dws, ws):
+        np.testing.assert_allclose(got, w.grad.numpy(), rtol=1e-10, atol=1e-12)
+    # the two fused products on their own: layer 0's activated output, and layer 1's input gradient carried to
+    # layer 0's pre-activation
+    y0, pre0 = O.dsd_forward_act(x.detach().numpy(), ws[0].detach().numpy(), masks[0].numpy(), bs, p, act)
+    np.testing.assert_allclose(pre0, pres[0].detach().numpy(), rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(y0, f(pres[0]).detach().numpy(), rtol=1e-10, atol=1e-12)
+    dpre1 = torch.randn(m, dims[2], generator=gen, dtype=torch.float64)
+    x0 = pres[0].detach().clone().requires_grad_()
+    naive_torch.forward(f(x0), ws[1].detach(), masks[1], bs, p).backward(dpre1)
+    got = O.sdd_dx_actgrad(dpre1.numpy(), ws[1].detach().numpy(), masks[1].numpy(), bs, p, act, pres[0].detach().numpy())
+    np.testing.assert_allclose(got, x0.grad.numpy(), rtol=1e-10, atol=1e-12)
+
+
+@pytest.mark.parametrize("act", ["relu", "gelu"])
+def test_mlp_with_hidden_tensors_stored_in_fp16(act):
+    """mlp_forward_backward(hidden_dtype=float16) against torch autograd of the same computation: hidden tensors
+    rounded to fp16 in value, identity in gradient (a straight-through rounding), GELU's derivative evaluated at
+    the rounded pre-activation."""
+    from oracle import naive_torch
+
+    gen = torch.Generator().manual_seed(32)
+    bs, p, m = 4, 0.25, 24
+    dims = [16, 32, 8]
+    x = torch.randn(m, dims[0], generator=gen, dtype=torch.float64, requires_grad=True)
+    ws = [torch.randn(dims[i + 1], dims[i], generator=gen, dtype=torch.float64, requires_grad=True) for i in range(2)]
+    masks = [torch.rand(m // bs, dims[i] // bs, generator=gen) < p for i in range(2)]
+    dy = torch.randn(m, dims[-1], generator=gen, dtype=torch.float64)
+    st = lambda t: t + (t.half().double() - t).detach()  # rounded value, identity gradient
+    f = {"relu": torch.relu, "gelu": torch.nn.functional.gelu}[act]
+    pre = naive_torch.forward(x, ws[0], masks[0], bs, p)
+    # the activated tensor is act(exact pre) rounded; its derivative is taken at the rounded pre-activation (GELU)
+    # or read off the rounded activated tensor (ReLU): spelled out with a custom function
+    class Act(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, t):
+            ctx.save_for_backward(t)
+            return f(t).half().double()
+
+        @staticmethod
+        def backward(ctx, g):
+            (t,) = ctx.saved_tensors
+            at = t.half().double() if act == "gelu" else f(t).half().double()
+            return g * torch.from_numpy(O.act_grad(at.numpy(), act))
+    h = Act.apply(pre)
+    out = naive_torch.forward(h, ws[1], masks[1], bs, p)
+    out.backward(dy)
+    rout, rdx, rdws = O.mlp_forward_backward(x.detach().numpy(), [w.detach().numpy() for w in ws],
+                                             [mk.numpy() for mk in masks], bs, p, act, dy.numpy(),
+                                             hidden_dtype=np.float16)
+    np.testing.assert_allclose(rout, out.detach().numpy(), rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(rdx, x.grad.numpy(), rtol=1e-10, atol=1e-12)
+    for got, w in zip(rdws, ws):
+        np.testing.assert_allclose(got, w.grad.numpy(), rtol=1e-10, atol=1e-12)
