@@ -30,8 +30,12 @@
  *   - Return value: SD_OK, or an error code with the reason in sd_last_error() (thread-local).
  *     Shapes and strides are always validated on the host (the reference only has assert()s,
  *     matmul_dsd.cuh:79-95).  The library allocates no device memory; workspaces are the caller's.
- *   - Supported block sizes: multiples of 64.  M, N, K are arbitrary (edge tiles are predicated);
- *     the mask has ceil(M/block_size) x ceil(K/block_size) entries.
+ *   - Supported block sizes: multiples of 64, and 32.  M, N, K are arbitrary (edge tiles are predicated);
+ *     the mask has ceil(M/block_size) x ceil(K/block_size) entries.  The kernels work on 64 x 64 tiles: a larger
+ *     block size is listed with every mask entry repeated, and 32 with four mask entries merged into one list
+ *     entry that remembers which of its 32 x 32 quadrants are kept (the report's block splitting, report.pdf
+ *     section 3.3, in both directions; the reference's Triton path takes any block size divisible by its tile,
+ *     flash_dropout/triton/utils.py:6-19, its CUDA path only 128, matmul_dsd.cuh:92-93).
  */
 #ifndef SPARSEDROP_H_
 #define SPARSEDROP_H_
@@ -114,7 +118,12 @@ int sd_build_lists(const uint8_t* mask, int64_t mb, int64_t kb, int64_t mask_str
                    int64_t mask_stride_c, int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr,
                    int32_t* row_idx, void* stream);
 
-/* Block splitting: the same lists for the mask with every entry repeated split x split times, cropped
+/* Block splitting.  split == 0: the mask is at block size 32, HALF the 64 the lists are over: out_mb = ceil(mb / 2),
+ * out_kb = ceil(kb / 2), a list entry is kept when any of the (up to) four mask entries it covers is, and bits 28-31 of
+ * the entry say which: bit 2a + b = mask entry (2i + a, 2j + b) kept (row_idx, the list by columns, stores them as the
+ * list of the transposed mask needs them: halves swapped).  The *_lists entry points take such lists when called with
+ * block_size 32: the 64 x 64 tile of a kept entry is computed and its dropped quadrants contribute / come out as zeros.
+ * split >= 1: the same lists for the mask with every entry repeated split x split times, cropped
  * to out_mb x out_kb ((mb-1)*split < out_mb <= mb*split, likewise out_kb); capacities out_mb*out_kb.
  * A mask drawn at block size 64*split over an [M,K] operand is listed with out_mb = ceil(M/64),
  * out_kb = ceil(K/64) and then drives the 64-block kernels (block_size 64 in the *_lists calls), which
@@ -132,7 +141,7 @@ int sd_build_lists_split(const uint8_t* mask, int64_t mb, int64_t kb, int64_t ma
  * (w >> 8) * 2^-24 < p (compared in fp32), w = word e%4 of Philox4x32-10 with counter
  * (lo32(e/4), hi32(e/4), lo32(offset), hi32(offset)) and key (lo32(seed), hi32(seed)): a pure function
  * of (seed, offset, e), not torch's generator stream.  mask_out receives the mb x kb mask as row-major
- * bytes (the autograd context and parity tests keep it); split / out_mb / out_kb as above. */
+ * bytes (the autograd context and parity tests keep it); split / out_mb / out_kb as above (split 0 included). */
 int sd_random_lists(uint64_t seed, uint64_t offset, float p, int64_t mb, int64_t kb, uint8_t* mask_out,
                     int64_t split, int64_t out_mb, int64_t out_kb, int32_t* row_ptr, int32_t* col_idx,
                     int32_t* col_ptr, int32_t* row_idx, void* stream);

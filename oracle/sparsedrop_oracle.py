@@ -31,6 +31,8 @@ Parity status of each function (what pins it is in tests/test_oracle.py):
                                            random STREAM is not part of the contract (parity is defined for
                                            a given mask), only the distribution is
   split_mask                               pinned: expand_keep identity (same element mask at both sizes)
+  merge_mask_quads / compact_csr_quads     pinned: expand_keep identity (the 64-grid mask with its quadrant bits
+                                           expands to the same element mask as the block-size-32 mask), hand case
   act_apply / act_grad / dsd_forward_act /
   sdd_dx_actgrad / mlp_forward_backward    pinned: torch's relu / gelu (erf form) and their autograd derivatives;
                                            the MLP against torch autograd through the literal naive.py
@@ -54,6 +56,8 @@ __all__ = [
     "philox4x32_10",
     "random_mask",
     "split_mask",
+    "merge_mask_quads",
+    "compact_csr_quads",
     "gemm_dsd",
     "gemm_sdd",
     "dsd_forward",
@@ -128,6 +132,33 @@ def split_mask(mask: np.ndarray, split: int, grid: tuple[int, int] | None = None
         assert (mask.shape[1] - 1) * split < grid[1] <= mask.shape[1] * split, (mask.shape, split, grid)
         out = out[: grid[0], : grid[1]]
     return out
+
+def merge_mask_quads(mask: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
+    """A block-size-32 mask on the 64 grid: (mask64, quads).  mask64[i, j] is True (dropped) when all of the (up to)
+    four entries (2i + a, 2j + b) are; quads[i, j] has bit 2a + b set when entry (2i + a, 2j + b) exists and is
+    kept.  This is the report's block splitting read downwards (report.pdf section 3.3): the kernels' 64 x 64 tile
+    covers four logical blocks."""
+    mask = np.asarray(mask, dtype=bool)
+    mb, kb = mask.shape
+    ob, ok = (mb + 1) // 2, (kb + 1) // 2
+    padded = np.ones((2 * ob, 2 * ok), dtype=bool)
+    padded[:mb, :kb] = mask
+    quads = np.zeros((ob, ok), dtype=np.uint8)
+    for a in range(2):
+        for b in range(2):
+            quads |= (~padded[a::2, b::2]).astype(np.uint8) << (2 * a + b)
+    return quads == 0, quads
+
+
+def compact_csr_quads(mask: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
+    """CSR list of merge_mask_quads(mask) with each entry's quadrant bits in bits 28-31, as int32 (the encoding
+    of the library's lists for block size 32).  For the list by columns call it on mask.T."""
+    mask64, quads = merge_mask_quads(mask)
+    row_ptr, col_idx = compact_csr(mask64)
+    rows = np.repeat(np.arange(mask64.shape[0]), np.diff(row_ptr))
+    enc = col_idx.astype(np.uint32) | (quads[rows, col_idx].astype(np.uint32) << 28)
+    return row_ptr, enc.view(np.int32)
+
 
 def mask_shape(m: int, k: int, block_size: int) -> tuple[int, int]:
     """Shape of the block mask of an [m, k] matrix (utils.py:13-14: ceil on both axes)."""

@@ -17,7 +17,7 @@ char* kernel_detail_buf() {
   return buf;
 }
 
-int build_lists(const uint8_t* mask, int64_t msr, int64_t msc, int64_t stored_kb, int64_t split,
+int build_lists(const uint8_t* mask, int64_t msr, int64_t msc, int64_t stored_mb, int64_t stored_kb, int64_t split,
                 int64_t mb, int64_t kb, int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr,
                 int32_t* row_idx, hipStream_t stream);
 int random_lists(uint64_t seed, uint64_t offset, uint64_t* state, float p, int64_t stored_mb, int64_t stored_kb,
@@ -62,7 +62,8 @@ int check_common(const void* A, int64_t asr, int64_t asc, const void* B, int64_t
 
 int check_sparse(int64_t bs, float scale) {
   SD_REQUIRE(bs > 0, "block_size must be positive");
-  if (bs % 64 != 0) return fail(SD_ERR_UNSUPPORTED, "block_size %lld: only multiples of 64 are supported", (long long)bs);
+  if (bs % 64 != 0 && bs != 32)
+    return fail(SD_ERR_UNSUPPORTED, "block_size %lld: only 32 and multiples of 64 are supported", (long long)bs);
   SD_REQUIRE(scale == scale, "scale is NaN");
   return SD_OK;
 }
@@ -98,7 +99,9 @@ GemmArgs make_args(const void* A, int64_t asr, int64_t asc, const void* B, int64
   g.M = M;
   g.N = N;
   g.K = K;
-  g.bs = bs;
+  // block size 32: the lists are on the 64 grid and carry the keep bits of each entry's four 32-blocks
+  g.bs = bs == 32 ? 64 : bs;
+  g.quads = bs == 32;
   g.scale = scale;
   g.row_ptr = row_ptr;
   g.col_idx = col_idx;
@@ -202,11 +205,19 @@ static int check_list_grid(int64_t mb, int64_t kb, int64_t split, int64_t out_mb
                            const int32_t* row_ptr, const int32_t* col_idx, const int32_t* col_ptr,
                            const int32_t* row_idx) {
   SD_REQUIRE(mb > 0 && kb > 0, "build_lists: mask must be non-empty (got %lld x %lld)", (long long)mb, (long long)kb);
-  SD_REQUIRE(split >= 1 && split < (1 << 16), "build_lists: split must be >= 1 (got %lld)", (long long)split);
-  // the listed grid is the mask repeated split x split, cropped inside its last row / column of entries
-  SD_REQUIRE(out_mb > (mb - 1) * split && out_mb <= mb * split && out_kb > (kb - 1) * split && out_kb <= kb * split,
-             "build_lists: a %lld x %lld grid does not match a %lld x %lld mask split by %lld", (long long)out_mb,
-             (long long)out_kb, (long long)mb, (long long)kb, (long long)split);
+  SD_REQUIRE(split >= 0 && split < (1 << 16), "build_lists: split must be >= 0 (got %lld)", (long long)split);
+  if (split == 0) {
+    // a mask at half the listed granularity, merged two by two
+    SD_REQUIRE(out_mb == (mb + 1) / 2 && out_kb == (kb + 1) / 2,
+               "build_lists: a %lld x %lld grid does not match a %lld x %lld mask merged two by two", (long long)out_mb,
+               (long long)out_kb, (long long)mb, (long long)kb);
+    SD_REQUIRE(out_kb < (1 << 28), "build_lists: merged lists keep four bits of every entry for the quadrants");
+  } else {
+    // the listed grid is the mask repeated split x split, cropped inside its last row / column of entries
+    SD_REQUIRE(out_mb > (mb - 1) * split && out_mb <= mb * split && out_kb > (kb - 1) * split && out_kb <= kb * split,
+               "build_lists: a %lld x %lld grid does not match a %lld x %lld mask split by %lld", (long long)out_mb,
+               (long long)out_kb, (long long)mb, (long long)kb, (long long)split);
+  }
   SD_REQUIRE(out_mb * out_kb < kMaxDim, "build_lists: mask too large for 32-bit lists");
   SD_REQUIRE((row_ptr == nullptr) == (col_idx == nullptr), "build_lists: pass both CSR arrays or neither");
   SD_REQUIRE((col_ptr == nullptr) == (row_idx == nullptr), "build_lists: pass both CSC arrays or neither");
@@ -220,7 +231,7 @@ int sd_build_lists_split(const uint8_t* mask, int64_t mb, int64_t kb, int64_t ms
   SD_REQUIRE(mask != nullptr, "build_lists: null mask");
   if (int rc = check_list_grid(mb, kb, split, out_mb, out_kb, row_ptr, col_idx, col_ptr, row_idx)) return rc;
   SD_REQUIRE(msr >= 1 && msc >= 1 && (msr == 1 || msc == 1), "build_lists: mask must be row or column major");
-  return build_lists(mask, msr, msc, kb, split, out_mb, out_kb, row_ptr, col_idx, col_ptr, row_idx,
+  return build_lists(mask, msr, msc, mb, kb, split, out_mb, out_kb, row_ptr, col_idx, col_ptr, row_idx,
                      (hipStream_t)stream);
 }
 
@@ -379,8 +390,12 @@ static int lists_in_workspace(const uint8_t* mask, int64_t msr, int64_t msc, int
   const int64_t mb = ceil_div(rows, *bs), kb = ceil_div(cols, *bs);
   SD_REQUIRE(mb > 0 && kb > 0, "empty mask");
   int64_t split = 1, out_mb = mb, out_kb = kb;
-  if (*bs > 64 && *bs % 64 == 0 && ceil_div(rows, 64) * ceil_div(cols, 64) < kMaxDim &&
-      workspace_bytes >= sd_workspace_bytes(ceil_div(rows, 64), ceil_div(cols, 64))) {
+  if (*bs == 32) {  // listed on the 64 grid with quadrant bits; the *_lists calls are told so by block size 32
+    split = 0;
+    out_mb = ceil_div(rows, 64);
+    out_kb = ceil_div(cols, 64);
+  } else if (*bs > 64 && *bs % 64 == 0 && ceil_div(rows, 64) * ceil_div(cols, 64) < kMaxDim &&
+             workspace_bytes >= sd_workspace_bytes(ceil_div(rows, 64), ceil_div(cols, 64))) {
     split = *bs / 64;
     out_mb = ceil_div(rows, 64);
     out_kb = ceil_div(cols, 64);
@@ -433,7 +448,7 @@ int sd_gemm_sdd(const void* A, int64_t asr, int64_t asc, const void* B, int64_t 
 }
 
 // granularity of the lists the fused calls build and take: 64 for block sizes that are multiples of 64
-static int64_t list_granule(int64_t bs) { return bs % 64 == 0 ? 64 : bs; }
+static int64_t list_granule(int64_t bs) { return (bs % 64 == 0 || bs == 32) ? 64 : bs; }
 
 int sd_dropout_matmul_forward(const void* X, int64_t xsr, int64_t xsc, const void* W, int64_t wsr, int64_t wsc,
                               void* Y, int64_t ysr, int64_t ysc, const uint8_t* mask, int64_t msr, int64_t msc,
@@ -446,7 +461,7 @@ int sd_dropout_matmul_forward(const void* X, int64_t xsr, int64_t xsc, const voi
   if (int rc = check_sparse(bs, 1.f)) return rc;
   SD_REQUIRE(M > 0 && K > 0, "dropout_matmul_forward: empty operand");
   SD_REQUIRE(row_ptr && col_idx, "dropout_matmul_forward: the CSR list arrays are required");
-  const int64_t g = list_granule(bs), split = bs / g;
+  const int64_t g = list_granule(bs), split = bs / g;  // 0 for block size 32: merged two by two
   const int64_t mb = ceil_div(M, bs), kb = ceil_div(K, bs), out_mb = ceil_div(M, g), out_kb = ceil_div(K, g);
   if (mask) {
     if (int rc = sd_build_lists_split(mask, mb, kb, msr, msc, split, out_mb, out_kb, row_ptr, col_idx, col_ptr, row_idx,
@@ -462,8 +477,8 @@ int sd_dropout_matmul_forward(const void* X, int64_t xsr, int64_t xsc, const voi
       return rc;
   }
   if (N == 0) return SD_OK;
-  return sd_gemm_dsd_lists(X, xsr, xsc, W, wsr, wsc, Y, ysr, ysc, row_ptr, col_idx, M, N, K, g, 1.f / (1.f - p), dtype,
-                           workspace, workspace_bytes, stream);
+  return sd_gemm_dsd_lists(X, xsr, xsc, W, wsr, wsc, Y, ysr, ysc, row_ptr, col_idx, M, N, K, bs == 32 ? 32 : g,
+                           1.f / (1.f - p), dtype, workspace, workspace_bytes, stream);
 }
 
 int sd_dropout_matmul_backward(const void* dY, int64_t gsr, int64_t gsc, const void* W, int64_t wsr, int64_t wsc,
@@ -474,7 +489,7 @@ int sd_dropout_matmul_backward(const void* dY, int64_t gsr, int64_t gsc, const v
   SD_REQUIRE(p >= 0.f && p < 1.f, "dropout_matmul_backward: p must be in [0, 1) (got %g)", (double)p);
   if (int rc = check_sparse(bs, 1.f)) return rc;
   SD_REQUIRE(dX || dW, "dropout_matmul_backward: nothing to compute");
-  const int64_t g = list_granule(bs);
+  const int64_t g = bs == 32 ? 32 : list_granule(bs);  // 32: lists on the 64 grid with quadrant bits
   const float scale = 1.f / (1.f - p);
   if (dX) {
     // dX[M,K] = scale * (dY[M,N] . W[N,K]) where kept: A = dY, B = W^T as the [K, N] view of W

@@ -110,6 +110,8 @@ struct GemmArgs {
   int64_t c_sr, c_sc;
   int64_t M, N, K;
   int64_t bs;     // mask block size (0 for dense)
+  bool quads;     // the lists are on the 64 grid of a block-size-32 mask: bits 28-31 of an entry say which of its four
+                  // 32 x 32 quadrants are kept (bit 2a + b: row half a, column half b); 0 in those bits = all four
   float scale;
   const int32_t* row_ptr;  // CSR of the mask (DSD: over A; SDD: over C); null for dense
   const int32_t* col_idx;
@@ -147,6 +149,13 @@ struct ImplicitConv {
 };
 
 enum Mode { kDense = 0, kDsd = 1, kSdd = 2 };
+
+// list entry -> block index / quadrant keep bits
+__device__ inline int32_t entry_block(int32_t e) { return (int32_t)((uint32_t)e & 0x0fffffffu); }
+__device__ inline uint32_t entry_quads(int32_t e) {
+  const uint32_t q = (uint32_t)e >> 28;
+  return q ? q : 0xfu;
+}
 
 // ---- fused epilogues --------------------------------------------------------------------------
 // GELU is the exact (erf) form, torch.nn.GELU's default: gelu(x) = x * Phi(x), gelu'(x) = Phi(x) + x * phi(x).

@@ -49,8 +49,9 @@ constexpr int BN = 256;       // output columns per workgroup
 constexpr int THREADS = 512;  // 8 waves
 constexpr int TILE = BS * BS * 2;              // bytes of one 64 x 64 tile (rows of 128 B)
 constexpr int MAX_STEPS = 1024;
-// step table: one uint32 per step of the union walk, reduction block | keep flags << 16, followed by
-// STEP_PAD zero entries so that look-ahead reads past the end are harmless
+// step table: one uint32 per step of the union walk, reduction block | keep bits << 16 (four bits per row block
+// of the workgroup: which 32 x 32 quadrants of its tile are kept; all four unless the mask has block size 32),
+// followed by STEP_PAD zero entries so that look-ahead reads past the end are harmless
 constexpr int STEP_PAD = 4;
 // Shape of a DSD workgroup: RH groups of RW row blocks x NS column slices of NT * 32 columns; wave
 // (rh, ns) multiplies its slice of the W tile with the kept X tiles of its RW row blocks.  Waves (rh, ns)
@@ -88,6 +89,7 @@ constexpr int CONV_PATCH_MAX = 163840 - DsdConv::SMEM_BYTES - 16;  // bytes left
 constexpr int CONV_T_PATCH_MAX = 24 * 1024;  // weight gradient: bytes of one step's copy of its input rows
 __device__ inline int step_block(uint32_t e) { return (int)(e & 0xffffu); }
 __device__ inline uint32_t step_flags(uint32_t e) { return e >> 16; }
+__device__ inline uint32_t row_quads(uint32_t flags, int r) { return (flags >> (4 * r)) & 0xfu; }  // of row block r
 __device__ inline uint32_t uniform(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane(v); }
 
 typedef __attribute__((address_space(3))) void lds_void;
@@ -147,6 +149,7 @@ template <typename T, bool TRANS, bool CM, bool RAGGED, typename S, int IMPLICIT
 __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m, int tiles_n,
                                                          int Mb, int Kb_all, ImplicitConv cg) {
   static_assert(!IMPLICIT || (S::R == 4 && S::THREADS == 512), "the gather assumes 512 threads x 4 row blocks");
+  static_assert(S::R <= 4, "a step's keep bits are four per row block in 16 bits");
   constexpr int R = S::R, BN = S::BN, THREADS = S::THREADS, NT = S::NT, STAGE = S::STAGE, A_OFF = S::A_OFF;
   constexpr int BL = S::BL, AL = S::AL, RW = S::RW;
   constexpr bool STEP_COPIES = IMPLICIT != 0 && (TRANS || IMPLICIT == 2);  // input rows copied per step
@@ -178,12 +181,14 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
       if (rb0 + r >= Mb) break;
       const int beg = g.row_ptr[rb0 + r], end = g.row_ptr[rb0 + r + 1];
       for (int i = beg + tid; i < end; i += THREADS) {
-        const int k = g.col_idx[i] - kb_lo;
-        if (k >= 0 && k < Kb) atomicOr(&scratch[k], 1u << r);
+        const int32_t e = g.col_idx[i];
+        const int k = entry_block(e) - kb_lo;
+        if (k >= 0 && k < Kb) atomicOr(&scratch[k], (IMPLICIT ? 0xfu : entry_quads(e)) << (4 * r));
       }
     }
   } else {
-    const uint32_t all = (rb0 + R <= Mb) ? ((1u << R) - 1u) : ((1u << (Mb - rb0)) - 1u);
+    const int rows = (rb0 + R <= Mb) ? R : Mb - rb0;
+    const uint32_t all = rows >= 4 ? 0xffffu : ((1u << (4 * rows)) - 1u);
     for (int i = tid; i < Kb; i += THREADS) scratch[i] = all;
   }
   __syncthreads();
@@ -524,7 +529,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
       }
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      if (fl & (1u << r)) {
+      if (row_quads(fl, r)) {
         if constexpr (IMPLICIT && !TRANS) {
           gather_tile(r, kb, st + A_OFF + r * TILE);
           continue;
@@ -594,8 +599,10 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   // (MINE = 1, 2 or 3).  The work is a chain of units (row block, kk); the LDS reads of unit u+1 are
   // issued before the MFMAs of unit u so that their latency hides behind 4 * NT16 MFMAs.  The W
   // fragments are read during the first row block's units and stay in registers for the second.
+  // quads: the keep bits of the wave's row blocks (four each); a quadrant that is not kept is zeroed in the X
+  // fragments, in the ragged-edge instance only (masks of block size 32 run on it)
   auto compute = [&](auto mine_c, const char* st, bool mid_loads, uint32_t mid_entry, int mid_stage,
-                     bool red_tail) {
+                     bool red_tail, uint32_t quads) {
     constexpr int MINE = decltype(mine_c)::value;
     constexpr int NR = (MINE == 3) ? 2 : 1;
     constexpr int R0 = (MINE == 2) ? 1 : 0;
@@ -613,6 +620,12 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
         read_a(at0 + ((u + 1) / 2) * TILE, kk1, af[(u + 1) & 1]);
       }
       __builtin_amdgcn_sched_barrier(0);
+      if (RAGGED && g.quads) {  // a mask of block size 32: zero the 32 x 32 quadrants of the tile that are dropped
+        const uint32_t q = row_quads(quads, rr);
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+          if (!((q >> (2 * (mt / 2) + kk)) & 1u)) af[u & 1][mt] = u32x4{0u, 0u, 0u, 0u};
+      }
       if (RAGGED && red_tail) {  // ragged reduction block: nothing past the end may reach the MFMAs
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt) mask_fragment(af[u & 1][mt], kk);
@@ -658,17 +671,19 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
       if (step + 2 < nsteps) tpatch_load(uniform(step_e[step + 2]));
       tcopy = ((step + 1) & 1) ? patch1 : patch;  // holds the rows of step + 1
     }
-    const uint32_t mine = (step_flags(e_cur) >> (RW * rh)) & ((1u << RW) - 1u);
+    // keep bits of this wave's row blocks (four per block); a block takes part when any of them is set
+    const uint32_t quads = (step_flags(e_cur) >> (4 * RW * rh)) & ((1u << (4 * RW)) - 1u);
+    const uint32_t mine = ((quads & 0xfu) ? 1u : 0u) | ((RW == 2 && (quads >> 4)) ? 2u : 0u);
     const bool mid = late && more && mine != 0u;
     if (more && !mid) issue_loads(e_next, stage ^ 1);
     const char* st = smem + stage * STAGE;
     const bool red_tail = RAGGED && step_block(e_cur) == kb_tail;
     if constexpr (RW == 2) {
-      if (mine == 3u) compute(std::integral_constant<int, 3>{}, st, mid, e_next, stage ^ 1, red_tail);
-      else if (mine == 1u) compute(std::integral_constant<int, 1>{}, st, mid, e_next, stage ^ 1, red_tail);
-      else if (mine == 2u) compute(std::integral_constant<int, 2>{}, st, mid, e_next, stage ^ 1, red_tail);
+      if (mine == 3u) compute(std::integral_constant<int, 3>{}, st, mid, e_next, stage ^ 1, red_tail, quads);
+      else if (mine == 1u) compute(std::integral_constant<int, 1>{}, st, mid, e_next, stage ^ 1, red_tail, quads);
+      else if (mine == 2u) compute(std::integral_constant<int, 2>{}, st, mid, e_next, stage ^ 1, red_tail, quads);
     } else {
-      if (mine) compute(std::integral_constant<int, 1>{}, st, mid, e_next, stage ^ 1, red_tail);
+      if (mine) compute(std::integral_constant<int, 1>{}, st, mid, e_next, stage ^ 1, red_tail, quads);
     }
     if constexpr (STEP_COPIES) {
       if (step + 2 < nsteps) tpatch_store((step & 1) ? patch1 : patch);  // last read for this step's tiles, a step ago
@@ -763,7 +778,9 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
                                                             int Cb) {
   constexpr int R = G::R, GW = G::GW, SLOTS = G::SLOTS, G_BOFF = G::BOFF, G_STAGE = G::STAGE;
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  uint32_t* flags = reinterpret_cast<uint32_t*>(smem);  // bit r: tile (row block rb0 + r, column block c) kept
+  // bit r: tile (row block rb0 + r, column block c) kept; bits 8 + 4r .. 11 + 4r: which of its four 32 x 32
+  // quadrants (all of them unless the mask has block size 32)
+  uint32_t* flags = reinterpret_cast<uint32_t*>(smem);
   int* rec = reinterpret_cast<int*>(smem + 4 * ((Cb + 3) & ~3));  // c_lo, c_hi, ncols, kept bits, cols[GW]
 
   int tm, gi;
@@ -775,17 +792,21 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
 
   // ---- per-column keep flags of this row quad -------------------------------------------------------
   {
-    const uint32_t all = (rb0 + R <= Mb) ? ((1u << R) - 1u) : ((1u << (Mb - rb0)) - 1u);
+    const int rows = (rb0 + R <= Mb) ? R : Mb - rb0;
+    const uint32_t all = ((1u << rows) - 1u) | (((1u << (4 * rows)) - 1u) << 8);
     const uint32_t init = g.row_ptr ? 0u : all;
     for (int i = tid; i < Cb; i += THREADS) flags[i] = init;
-    if (tid < 16) rec[tid] = 0;
+    if (tid < 32) rec[tid] = 0;
   }
   __syncthreads();
   if (g.row_ptr) {
     for (int r = 0; r < R; ++r) {
       if (rb0 + r >= Mb) break;
       const int beg = g.row_ptr[rb0 + r], end = g.row_ptr[rb0 + r + 1];
-      for (int i = beg + tid; i < end; i += THREADS) atomicOr(&flags[g.col_idx[i]], 1u << r);
+      for (int i = beg + tid; i < end; i += THREADS) {
+        const int32_t e = g.col_idx[i];
+        atomicOr(&flags[entry_block(e)], (1u << r) | (entry_quads(e) << (8 + 4 * r)));
+      }
     }
     __syncthreads();
   }
@@ -801,7 +822,7 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
     if (w_hi - w_lo <= 64) {
       const uint32_t fv = (w_lo + lane < w_hi) ? flags[w_lo + lane] : 0u;
       for (int i = 0; i < w_hi - w_lo; ++i) {
-        const uint32_t f = (uint32_t)__builtin_amdgcn_readlane((int)fv, i);
+        const uint32_t f = (uint32_t)__builtin_amdgcn_readlane((int)fv, i) & 0xfu;
         if (f == 0) continue;
         const int a = __builtin_popcount(f);
         if (width == GW || cnt + a > G::MAXT) {  // the group ends in front of this column block
@@ -826,9 +847,13 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
     int n = 0;
     uint32_t kept = 0;  // bit 4*j + r
     for (int c = lo; c < hi; ++c) {
-      const uint32_t f = (uint32_t)__builtin_amdgcn_readfirstlane((int)flags[c]);
+      const uint32_t fq = (uint32_t)__builtin_amdgcn_readfirstlane((int)flags[c]);
+      const uint32_t f = fq & 0xfu;
       if (f) {
-        if (lane == 0) rec[4 + n] = c;
+        if (lane == 0) {
+          rec[4 + n] = c;
+          rec[16 + n] = (int)(fq >> 8);  // quadrant keep bits of the column block's tiles, four per row block
+        }
         kept |= f << (4 * n);
         ++n;
       }
@@ -865,6 +890,10 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
     my_r[k] = b % 4;
     my_c[k] = __builtin_amdgcn_readfirstlane(rec[4 + my_j[k]]);
   }
+  uint32_t my_q[SLOTS];  // which quadrants of the wave's tiles are kept
+#pragma unroll
+  for (int k = 0; k < SLOTS; ++k)
+    my_q[k] = ((uint32_t)__builtin_amdgcn_readfirstlane(rec[16 + my_j[k]]) >> (4 * my_r[k])) & 0xfu;
   uint32_t rowmask = 0;
 #pragma unroll
   for (int j = 0; j < GW; ++j) rowmask |= (kept >> (4 * j)) & 0xfu;
@@ -1066,8 +1095,11 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
-        for (int v = 0; v < 4; ++v)  // register v of lane l is element (4*(l/16) + v, l%16) of the 16 x 16 tile
-          stg[(mt * 16 + 4 * (lane / 16) + v) * S_PITCH + nt * 16 + lane % 16] = acc[k][mt][nt][v];
+        for (int v = 0; v < 4; ++v) {  // register v of lane l is element (4*(l/16) + v, l%16) of the 16 x 16 tile
+          // a mask of block size 32 drops 32 x 32 quadrants of a kept tile: those are stored as zeros
+          const bool keep = !EDGE || ((my_q[k] >> (2 * (mt / 2) + nt / 2)) & 1u);
+          stg[(mt * 16 + 4 * (lane / 16) + v) * S_PITCH + nt * 16 + lane % 16] = keep ? acc[k][mt][nt][v] : 0.f;
+        }
     store_staged_tile<T, true, BS, BS>(g, stg, lane, true, (int64_t)(rb0 + my_r[k]) * BS, (int64_t)my_c[k] * BS,
                                        nullptr);
   }
@@ -1112,7 +1144,8 @@ int launch_dsd_s(const GemmArgs& g, int splits, hipStream_t stream) {
 
 template <typename T, bool TRANS, bool CM>
 int launch_dsd(const GemmArgs& g, bool mid, int splits, hipStream_t stream) {
-  const bool ragged = g.M % BS != 0 || g.N % BS != 0 || g.K % BS != 0;
+  // masks of block size 32 (quadrant keep bits in the lists) run on the ragged-edge instance, which masks fragments
+  const bool ragged = g.M % BS != 0 || g.N % BS != 0 || g.K % BS != 0 || g.quads;
   if (mid)
     return ragged ? launch_dsd_s<T, TRANS, CM, true, DsdMid>(g, splits, stream)
                   : launch_dsd_s<T, TRANS, CM, false, DsdMid>(g, splits, stream);
@@ -1193,7 +1226,7 @@ int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
   const int64_t tiles = (((g.M + BS - 1) / BS + 1) / 2) * ((Cb + 3) / 4);  // the larger of the two shapes' grids
   if (!layout_ok || !shape_ok || !align_ok || tiles > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
   if (Cb > G_MAX_CB) return SD_ERR_UNSUPPORTED;
-  const bool edge = g.N % BS != 0 || g.K % BS != 0;
+  const bool edge = g.N % BS != 0 || g.K % BS != 0 || g.quads;  // quadrant zeroing lives in the edge instance
   if (dtype == SD_BF16) return edge ? launch_sdd_group<BF16, true>(g, stream) : launch_sdd_group<BF16, false>(g, stream);
   return edge ? launch_sdd_group<F16, true>(g, stream) : launch_sdd_group<F16, false>(g, stream);
 }

@@ -101,9 +101,13 @@ struct KWalk {
   int64_t bs, K;
   int64_t k, kend;
   bool listed;
+  uint32_t quads;  // keep bits of the four 32 x 32 quadrants of the block being walked (0xf unless listed so)
+  int half;        // which 32-wide half of that block the last next() returned
   // split s of S takes an equal share of the BK-steps (dense) or of the list entries (listed)
   __device__ inline void init_dense(int64_t K_, int s, int S) {
     listed = false;
+    quads = 0xfu;
+    half = 0;
     K = K_;
     const int64_t steps = (K_ + BK - 1) / BK;
     k = steps * s / S * BK;
@@ -121,31 +125,37 @@ struct KWalk {
     K = K_;
     k = 0;
     kend = 0;
+    quads = 0xfu;
+    half = 0;
   }
   // next k offset or -1
   __device__ inline int64_t next() {
     if (k >= kend) {
       if (!listed || pos >= end) return -1;
-      const int64_t blk = idx[pos++];
+      const int32_t e = idx[pos++];
+      const int64_t blk = entry_block(e);
+      quads = entry_quads(e);
       k = blk * bs;
       kend = k + bs < K ? k + bs : K;
       if (k >= kend) return -1;
     }
     const int64_t r = k;
+    half = listed ? (int)(((k % bs) / BK) & 1) : 0;  // BK = 32: the half of a 64-block (only read for such lists)
     k += BK;
     return r;
   }
 };
 
-// true if `want` occurs in the ascending list idx[beg, end)
-__device__ inline bool list_contains(const int32_t* idx, int32_t beg, int32_t end, int32_t want) {
+// quadrant keep bits of block `want` if it occurs in the ascending list idx[beg, end) (0xf for a list without
+// such bits), else 0
+__device__ inline uint32_t list_lookup(const int32_t* idx, int32_t beg, int32_t end, int32_t want) {
   while (beg < end) {
     const int32_t mid = (beg + end) >> 1;
-    const int32_t v = idx[mid];
-    if (v == want) return true;
+    const int32_t v = entry_block(idx[mid]);
+    if (v == want) return entry_quads(idx[mid]);
     if (v < want) beg = mid + 1; else end = mid;
   }
-  return false;
+  return 0u;
 }
 
 template <typename T, int MODE, bool TRANS_OUT, bool SPLIT>
@@ -163,6 +173,7 @@ __global__ __launch_bounds__(THREADS) void gemm_generic_kernel(GemmArgs g, int t
   const int wm = wave / 2, wn = wave % 2;  // wave's 32x64 piece
 
   KWalk walk;
+  uint32_t sdd_quads = 0x3u;  // SDD: which 32-column halves of the wave's piece are kept
   bool wave_kept = true;
   bool any_kept = true;
   if (MODE == kDsd) {
@@ -174,11 +185,14 @@ __global__ __launch_bounds__(THREADS) void gemm_generic_kernel(GemmArgs g, int t
     if (MODE == kSdd) {
       const int64_t rb = m0 / g.bs;
       const int32_t beg = g.row_ptr[rb], end = g.row_ptr[rb + 1];
-      const bool kept0 = list_contains(g.col_idx, beg, end, (int32_t)(n0 / g.bs));
-      const bool kept1 =
-          (n0 + 64 < g.N) && list_contains(g.col_idx, beg, end, (int32_t)((n0 + 64) / g.bs));
-      wave_kept = wn ? kept1 : kept0;
-      any_kept = kept0 || kept1;
+      const uint32_t q0 = list_lookup(g.col_idx, beg, end, (int32_t)(n0 / g.bs));
+      const uint32_t q1 = (n0 + 64 < g.N) ? list_lookup(g.col_idx, beg, end, (int32_t)((n0 + 64) / g.bs)) : 0u;
+      // with quadrant bits (block size 32, g.bs == 64 == the wave grid): the wave's 32 x 64 piece is row half wm of
+      // one 64-block, its two 32-column halves are quadrants (wm, 0) and (wm, 1)
+      sdd_quads = ((wn ? q1 : q0) >> (2 * wm)) & 0x3u;
+      if (!g.quads) sdd_quads = (wn ? q1 : q0) ? 0x3u : 0u;
+      wave_kept = sdd_quads != 0u;
+      any_kept = (q0 | q1) != 0u;
     }
   }
 
@@ -196,6 +210,8 @@ __global__ __launch_bounds__(THREADS) void gemm_generic_kernel(GemmArgs g, int t
       load_tile<BN>(g.b, b_kc, b_vec, n0, g.N, k0, g.K, rb);
     }
     while (k0 >= 0) {
+      // DSD with quadrant bits: the wave's 32 rows are row half wm of the 64-block, this step its 32-wide half
+      const bool step_kept = !(MODE == kDsd && g.quads) || ((walk.quads >> (2 * wm + walk.half)) & 1u);
       store_tile<BM>(sA, a_kc, ra);
       store_tile<BN>(sB, b_kc, rb);
       __syncthreads();
@@ -204,7 +220,7 @@ __global__ __launch_bounds__(THREADS) void gemm_generic_kernel(GemmArgs g, int t
         load_tile<BM>(g.a, a_kc, a_vec, m0, g.M, k0, g.K, ra);
         load_tile<BN>(g.b, b_kc, b_vec, n0, g.N, k0, g.K, rb);
       }
-      if (wave_kept) {
+      if (wave_kept && step_kept) {
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
           const int kk = ks * 16 + (lane / 32) * 8;
@@ -236,6 +252,7 @@ __global__ __launch_bounds__(THREADS) void gemm_generic_kernel(GemmArgs g, int t
       const int64_t m = m0 + wm * 32 + (TRANS_OUT ? lane_i : reg_i);
       const int64_t n = n0 + wn * 64 + j * 32 + (TRANS_OUT ? reg_i : lane_i);
       if (m < g.M && n < g.N) {
+        if (MODE == kSdd && !((sdd_quads >> j) & 1u)) acc[j][v] = 0.f;  // a dropped 32-column quadrant of a kept block
         if (SPLIT) {
           // workspace layout follows C's contiguous index so that lanes stay coalesced
           const int64_t e = TRANS_OUT ? n * g.M + m : m * g.N + n;

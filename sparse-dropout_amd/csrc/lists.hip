@@ -43,11 +43,15 @@ struct Philox {
 // Where "is block (i, j) dropped" comes from: a stored bool mask, or a Bernoulli(p) draw that is a pure
 // function of (seed, offset, entry index), so every reader recomputes the same value and no pass over
 // a stored mask is needed.  Each stored / drawn entry covers split x split entries of the listed grid
-// (a logical block size that is a multiple of the 64 the kernels work in).
+// (a logical block size that is a multiple of the 64 the kernels work in), or, with merge == 2, a quarter of
+// one: a mask at block size 32 is listed on the 64 grid, an entry being kept when any of its four 32-blocks
+// is, with those four keep bits stored in the top bits of its list entry (quad_bits).
 struct MaskSrc {
   const uint8_t* mask;  // null: drawn
   int64_t st_row, st_col;
   int32_t split;
+  int32_t merge;  // 1, or 2: four stored / drawn entries per listed entry
+  int32_t mb;     // rows of the stored / drawn mask (only read when merge == 2)
   int32_t kb;  // entries per row of the stored / drawn mask
   uint32_t seed_lo, seed_hi, off_lo, off_hi;
   float p;
@@ -80,7 +84,20 @@ struct MaskSrc {
     for (int v = 0; v < 4; ++v) bits |= ((float)(c[v] >> 8) * 0x1p-24f < p ? 1u : 0u) << v;
     return bits;
   }
+  // merge == 2: keep bits of the four 32-blocks of listed entry (i, j); bit 2a + b = block (2i + a, 2j + b)
+  __device__ inline uint32_t kept_quads(int32_t i, int32_t j) const {
+    uint32_t q = 0;
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const int32_t si = 2 * i + a, sj = 2 * j + b;
+        if (si < mb && sj < kb && !dropped_entry(si, sj)) q |= 1u << (2 * a + b);
+      }
+    return q;
+  }
   __device__ inline bool dropped(int32_t i, int32_t j) const {
+    if (merge == 2) return kept_quads(i, j) == 0;
     return split == 1 ? dropped_entry(i, j) : dropped_entry(i / split, j / split);
   }
 };
@@ -94,6 +111,15 @@ struct ListJob {
   int32_t* idx;    // [capacity nlines * len]
   __device__ inline bool kept(int64_t line, int64_t e) const {
     return by_col ? !src.dropped((int32_t)e, (int32_t)line) : !src.dropped((int32_t)line, (int32_t)e);
+  }
+  // what goes into idx for kept entry e of `line`: e itself, with merge == 2 the four keep bits of its
+  // 32-blocks in bits 28-31 (bit 2a + b: row half a, column half b of the LIST's own orientation, i.e.
+  // transposed for a list by columns, which is the row list of the transposed mask)
+  __device__ inline int32_t entry(int64_t line, int64_t e) const {
+    if (src.merge != 2) return (int32_t)e;
+    uint32_t q = by_col ? src.kept_quads((int32_t)e, (int32_t)line) : src.kept_quads((int32_t)line, (int32_t)e);
+    if (by_col) q = (q & 0x9u) | ((q & 0x2u) << 1) | ((q & 0x4u) >> 1);
+    return (int32_t)((uint32_t)e | (q << 28));
   }
 };
 
@@ -116,7 +142,7 @@ __device__ inline void wave_fill_kept(const ListJob& job, int64_t line, int lane
     const int64_t i = base + lane;
     const bool kept = (i < job.len) && job.kept(line, i);
     const uint64_t bal = __ballot(kept);
-    if (kept) out[written + __popcll(bal & lt)] = (int32_t)i;
+    if (kept) out[written + __popcll(bal & lt)] = job.entry(line, i);
     written += __popcll(bal);
   }
 }
@@ -229,7 +255,7 @@ __global__ __launch_bounds__(kFlatThreads) void build_lists_flat(ListJob job0, L
 
   // kept entries in front of this block's chunk
   // a mask drawn at the listed granularity: entry index = row-major position, four entries share a generator call
-  const bool drawn4 = job.src.mask == nullptr && job.src.split == 1 && job.src.kb == (job.by_col ? (int)job.nlines : len);
+  const bool drawn4 = job.src.mask == nullptr && job.src.split == 1 && job.src.merge == 1 && job.src.kb == (job.by_col ? (int)job.nlines : len);
   int cnt = 0;
   if (drawn4 && !job.by_col) {
     for (int grp = tid; grp * 4 < f0; grp += kFlatThreads) cnt += __popc(~job.src.dropped4((uint64_t)grp) & 0xFu);
@@ -280,7 +306,7 @@ __global__ __launch_bounds__(kFlatThreads) void build_lists_flat(ListJob job0, L
   for (int v = 0; v < kFlatPer; ++v) {
     if (mine + v < total_entries) {
       if (e == 0) job.ptr[line] = pos;
-      if (bits & (1u << v)) job.idx[pos++] = e;
+      if (bits & (1u << v)) job.idx[pos++] = job.entry(line, e);
     }
     if (++e == len) { e = 0; ++line; }
   }
@@ -380,11 +406,13 @@ static int launch_lists(const MaskSrc& src, int64_t mb, int64_t kb, int32_t* row
   return check_launch("build_lists");
 }
 
-// Lists over an mb x kb grid in which every stored mask entry covers split x split grid entries.
-int build_lists(const uint8_t* mask, int64_t msr, int64_t msc, int64_t stored_kb, int64_t split,
+// Lists over an mb x kb grid in which every stored mask entry covers split x split grid entries; split == 0: the
+// stored mask is at half the granularity (stored_mb x stored_kb entries) and is merged two by two.
+int build_lists(const uint8_t* mask, int64_t msr, int64_t msc, int64_t stored_mb, int64_t stored_kb, int64_t split,
                 int64_t mb, int64_t kb, int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr,
                 int32_t* row_idx, hipStream_t stream) {
-  MaskSrc src{mask, msr, msc, (int32_t)split, (int32_t)stored_kb, 0, 0, 0, 0, 0.f, nullptr};
+  MaskSrc src{mask, msr, msc, (int32_t)(split ? split : 1), split ? 1 : 2, (int32_t)stored_mb, (int32_t)stored_kb,
+              0, 0, 0, 0, 0.f, nullptr};
   return launch_lists(src, mb, kb, row_ptr, col_idx, col_ptr, row_idx, nullptr, 0, stream);
 }
 
@@ -392,8 +420,8 @@ int build_lists(const uint8_t* mask, int64_t msr, int64_t msc, int64_t stored_kb
 int random_lists(uint64_t seed, uint64_t offset, uint64_t* state, float p, int64_t stored_mb, int64_t stored_kb,
                  uint8_t* mask_out, int64_t split, int64_t mb, int64_t kb, int32_t* row_ptr,
                  int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx, hipStream_t stream) {
-  MaskSrc src{nullptr, 0, 0, (int32_t)split, (int32_t)stored_kb, (uint32_t)seed, (uint32_t)(seed >> 32),
-              (uint32_t)offset, (uint32_t)(offset >> 32), p, state};
+  MaskSrc src{nullptr, 0, 0, (int32_t)(split ? split : 1), split ? 1 : 2, (int32_t)stored_mb, (int32_t)stored_kb,
+              (uint32_t)seed, (uint32_t)(seed >> 32), (uint32_t)offset, (uint32_t)(offset >> 32), p, state};
   bool advanced = false;
   if (int rc = launch_lists(src, mb, kb, row_ptr, col_idx, col_ptr, row_idx, mask_out, stored_mb, stream, &advanced))
     return rc;

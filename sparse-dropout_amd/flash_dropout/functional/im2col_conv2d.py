@@ -169,6 +169,8 @@ def blockwise_dropout_conv2d_mask(input, mask, block_size, p: float, kernel, pad
     if not 0 <= p < 1:
         raise ValueError("Dropout probability must be in [0, 1)")
     bs = _block_size(block_size)
+    if bs % 64:
+        raise NotImplementedError(f"block_size {bs}: the convolution takes multiples of 64 (the matmul also 32)")
     input, kernel = _prepare(input, kernel)
     return _apply_outside_autocast(_Im2colConv2d, input, kernel, mask, bs, float(p), _pair(padding), _pair(stride), _pair(dilation))
 
@@ -180,6 +182,8 @@ def blockwise_dropout_conv2d(input, kernel, block_size, p: float, padding=(0, 0)
     if not 0 <= p < 1:
         raise ValueError("Dropout probability must be in [0, 1)")
     bs = _block_size(block_size)
+    if bs % 64:
+        raise NotImplementedError(f"block_size {bs}: the convolution takes multiples of 64 (the matmul also 32)")
     input, kernel = _prepare(input, kernel)
     return _apply_outside_autocast(_Im2colConv2d, input, kernel, None, bs, float(p), _pair(padding), _pair(stride),
                                    _pair(dilation), seed)

@@ -92,6 +92,12 @@ def _block_size(block_size) -> int:
     return int(block_size)
 
 
+def _list_grid_size(bs: int) -> int:
+    """Edge of the blocks the kept-block lists are over: 64 for a block size of 32 (the lists then carry, in the
+    top four bits of every entry, which of the entry's four 32-blocks are kept), else the block size."""
+    return 64 if bs == 32 else bs
+
+
 def _check_operand(name: str, x: torch.Tensor) -> None:
     # same rules as the reference's check_operand + dtype checks (gemm_binding.cu:18-22, 87-89)
     if not isinstance(x, torch.Tensor):
@@ -246,7 +252,7 @@ class GEMM:
         C = self._out(A, B, out, transposed_out)
         if M == 0 or N == 0:
             return C
-        if bs > 64 and bs % 64 == 0:  # room for the 64-granular list: the library then splits the mask
+        if (bs > 64 and bs % 64 == 0) or bs == 32:  # the 64-granular list: the library splits / merges the mask
             ws_bytes = self.lib.sd_workspace_bytes(ceil(M / 64), ceil((K if mask_cols == "K" else N) / 64))
         else:
             ws_bytes = self.lib.sd_workspace_bytes(mb, cb)
@@ -288,8 +294,13 @@ class GEMM:
     @staticmethod
     def _list_grid(mb, kb, split, grid):
         split = int(split)
-        if split < 1:
-            raise ValueError(f"split must be >= 1, got {split}")
+        if split < 0:
+            raise ValueError(f"split must be >= 0, got {split}")
+        if split == 0:  # a mask of block size 32 merged two by two onto the 64 grid
+            out_mb, out_kb = ((mb + 1) // 2, (kb + 1) // 2) if grid is None else (int(grid[0]), int(grid[1]))
+            if (out_mb, out_kb) != ((mb + 1) // 2, (kb + 1) // 2):
+                raise ValueError(f"grid {(out_mb, out_kb)} does not match a {(mb, kb)} mask merged two by two")
+            return split, out_mb, out_kb
         out_mb, out_kb = (mb * split, kb * split) if grid is None else (int(grid[0]), int(grid[1]))
         if not ((mb - 1) * split < out_mb <= mb * split and (kb - 1) * split < out_kb <= kb * split):
             raise ValueError(f"grid {(out_mb, out_kb)} does not match a {(mb, kb)} mask split by {split}")
@@ -306,7 +317,10 @@ class GEMM:
 
         ``split`` > 1 lists the mask with every entry repeated split x split times, cropped to
         ``grid`` = (rows, cols) of the finer block grid (default: uncropped): a mask drawn at block
-        size 64*split then drives the 64-block kernels."""
+        size 64*split then drives the 64-block kernels.  ``split`` = 0 goes the other way for a mask at block
+        size 32: it is listed on the 64 grid, an entry kept when any of its four 32-blocks is, and bits 28-31 of
+        the entry say which (bit 2a + b: row half a, column half b; in ``row_idx`` with the halves swapped, as
+        the list of the transposed mask needs them); the ``*_lists`` calls take such lists with block size 32."""
         if mask.dim() != 2 or mask.dtype != torch.bool or not mask.is_cuda:
             raise ValueError("mask must be a 2D bool tensor on the GPU")
         mb, kb = mask.shape
@@ -395,6 +409,8 @@ class GEMM:
         split, grid, kernel_bs = 1, None, bs
         if bs > 64 and bs % 64 == 0:
             split, grid, kernel_bs = bs // 64, (ceil(rows / 64), ceil(cols / 64)), 64
+        elif bs == 32:  # merged two by two onto the 64 grid; the *_lists calls are told so by block size 32
+            split, grid = 0, (ceil(rows / 64), ceil(cols / 64))
         if mask is None:
             mask, lists = self.random_lists(shape, p, seed, 0, device, split, grid)
         else:
@@ -423,7 +439,8 @@ class GEMM:
         self._check_pair(A, B)
         bs = _block_size(block_size)
         M, N, K = A.shape[0], B.shape[0], A.shape[1]
-        want = (ceil(M / bs), ceil((K if mask_cols == "K" else N) / bs))
+        lg = _list_grid_size(bs)
+        want = (ceil(M / lg), ceil((K if mask_cols == "K" else N) / lg))
         if tuple(lists.shape) != want:
             raise ValueError(f"lists are for a {lists.shape} mask, operands need {want}")
         C = self._out(A, B, out, transposed_out)
@@ -451,7 +468,8 @@ class GEMM:
         self._check_pair(A, B)
         bs = _block_size(block_size)
         M, N, K = A.shape[0], B.shape[0], A.shape[1]
-        want = (ceil(M / bs), ceil(N / bs))
+        lg = _list_grid_size(bs)
+        want = (ceil(M / lg), ceil(N / lg))
         if tuple(lists.shape) != want:
             raise ValueError(f"lists are for a {lists.shape} mask, operands need {want}")
         C = self._out(A, B, out, transposed_out)
@@ -472,7 +490,8 @@ class GEMM:
         bs = _block_size(block_size)
         code = _activation(act)
         M, N, K = A.shape[0], B.shape[0], A.shape[1]
-        want = (ceil(M / bs), ceil(K / bs))
+        lg = _list_grid_size(bs)
+        want = (ceil(M / lg), ceil(K / lg))
         if tuple(lists.shape) != want:
             raise ValueError(f"lists are for a {lists.shape} mask, operands need {want}")
         C = torch.empty((M, N), dtype=A.dtype, device=A.device)
@@ -495,7 +514,8 @@ class GEMM:
         bs = _block_size(block_size)
         code = _activation(act)
         M, N, K = A.shape[0], B.shape[0], A.shape[1]
-        want = (ceil(M / bs), ceil(N / bs))
+        lg = _list_grid_size(bs)
+        want = (ceil(M / lg), ceil(N / lg))
         if tuple(lists.shape) != want:
             raise ValueError(f"lists are for a {lists.shape} mask, operands need {want}")
         if code:
@@ -524,7 +544,7 @@ class GEMM:
         if not 0.0 <= p < 1.0:
             raise ValueError(f"p must be in [0, 1), got {p}")
         M, K, N = x.shape[0], x.shape[1], w.shape[0]
-        g = 64 if bs % 64 == 0 else bs
+        g = 64 if (bs % 64 == 0 or bs == 32) else bs
         mb, kb, out_mb, out_kb = ceil(M / bs), ceil(K / bs), ceil(M / g), ceil(K / g)
         if mb == 0 or kb == 0:
             raise ValueError("mask must be non-empty")
@@ -546,7 +566,8 @@ class GEMM:
                        None if state is None else state.data_ptr(), (int(seed) & (2 ** 64 - 1)) if seed is not None else 0,
                        0, float(p), mask.data_ptr(), row_ptr.data_ptr(), col_idx.data_ptr(), col_ptr.data_ptr(),
                        row_idx.data_ptr(), M, N, K, bs, _DTYPES[x.dtype], ws_ptr, ws_bytes, self._stream(x))
-        return y, mask, KeptLists(row_ptr, col_idx, col_ptr, row_idx, (out_mb, out_kb)), g
+        # block size 32 stays 32 for the backward call: it says that the lists carry quadrant bits
+        return y, mask, KeptLists(row_ptr, col_idx, col_ptr, row_idx, (out_mb, out_kb)), (32 if bs == 32 else g)
 
     def dropout_matmul_backward(self, dy: torch.Tensor, w: torch.Tensor, x: torch.Tensor, lists: KeptLists,
                                 block_size, p: float, need_dx: bool = True, need_dw: bool = True):
@@ -558,7 +579,7 @@ class GEMM:
         M, K, N = x.shape[0], x.shape[1], w.shape[0]
         if tuple(dy.shape) != (M, N) or dy.dtype != x.dtype or dy.device != x.device:
             raise ValueError(f"dy must be a [{M}, {N}] {x.dtype} tensor on {x.device}")
-        g = 64 if bs % 64 == 0 else bs
+        g = 64 if (bs % 64 == 0 or bs == 32) else bs
         if tuple(lists.shape) != (ceil(M / g), ceil(K / g)):
             raise ValueError(f"lists are for a {lists.shape} mask, operands need {(ceil(M / g), ceil(K / g))}")
         if N % 8 and N > 0 and M > 0 and K > 0 and (need_dx or need_dw):

@@ -468,3 +468,57 @@ def test_sdd_kept_only_leaves_dropped_tiles_untouched(M, N, K):
     keep = torch.from_numpy(O.expand_keep(mk.numpy(), 64, M, K)).cuda()
     assert torch.equal(got[keep], full[keep])
     assert (got[~keep] == sentinel).all()
+
+
+# ---- block size 32: four mask blocks per 64 x 64 tile of the kernels -------------------------------------------
+@pytest.mark.parametrize("mnk,p", list(product(REF_MNKS, REF_PS)))
+def test_reference_grid_at_block_size_32(mnk, p):
+    """The reference's shape and drop-rate grid (test/test_cuda.py:12-20) at block size 32, which its Triton path
+    takes (flash_dropout/triton/utils.py:6-19): Y, dX and dW against the oracle, dropped 32-blocks of dX exactly
+    zero."""
+    M, N, K = mnk
+    bs = 32
+    gen = torch.Generator().manual_seed(20)
+    A = make_operand(M, K, torch.float16, "cuda", gen=gen)
+    # weights scaled as a layer's are: with N(0, 1) weights the kept blocks at p = 0.999 (scale 1000) overflow fp16
+    B = make_operand(N, K, torch.float16, "cuda", scale=K ** -0.5, gen=gen)
+    dC = make_operand(M, N, torch.float16, "cuda", gen=gen)
+    mask = cpu_mask((M // bs, K // bs), p, gen).cuda()
+    C, dA, dB = _three_products(A, B, dC, mask, bs, p)
+    rC, rdA, rdB = _oracle_products(A, B, dC, mask, bs, p)
+    atol = 0.2 * max(1.0, (1 / (1 - p)) / 10)
+    _check(C, rC, "C", atol)
+    _check(dB, rdB, "dB", atol)
+    _check(dA, rdA, "dA", atol)
+    keep = O.expand_keep(mask.cpu().numpy(), bs, M, K)
+    assert (dA.cpu().numpy()[~keep] == 0).all(), "dropped dX blocks must be exactly zero"
+
+
+@pytest.mark.parametrize("M,N,K", [(1000, 136, 200), (100, 70, 50), (4096, 10, 1024), (4096, 1024, 784), (96, 64, 160),
+                                   (16384, 384, 1536)])
+@pytest.mark.parametrize("p", [0.3, 0.75])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_block_size_32_on_ragged_and_model_shapes(M, N, K, p, dtype):
+    """Block size 32 where the 32-grid has an odd number of blocks, the shape is ragged against both grids, or
+    the operands force the generic kernel (K = 50): mask forms and list forms, all three products."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(M + K)
+    A = make_operand(M, K, dtype, "cuda", gen=gen)
+    B = make_operand(N, K, dtype, "cuda", scale=K ** -0.5, gen=gen)
+    dC = make_operand(M, N, dtype, "cuda", gen=gen)
+    mk = cpu_mask(O.mask_shape(M, K, 32), p, gen)
+    C, dA, dB = _three_products(A, B, dC, mk.cuda(), 32, p)
+    rC, rdA, rdB = _oracle_products(A, B, dC, mk, 32, p)
+    for got, ref, what in ((C, rC, "C"), (dA, rdA, "dA"), (dB, rdB, "dB")):
+        assert max_tile_rel_fro(got, ref, tile=32) <= REL_FRO_TOL, what
+    keep = O.expand_keep(mk.numpy(), 32, M, K)
+    assert (to_np(dA)[~keep] == 0).all()
+    # the list forms on lists built once (block size 32 tells them that the lists carry quadrant bits)
+    lists = ext.build_lists(mk.cuda(), split=0)
+    s = 1 / (1 - p)
+    assert torch.equal(ext.gemm_dsd_lists(A, B, lists, 32, s), C)
+    assert torch.equal(ext.gemm_sdd_lists(dC, B.T, lists, 32, s), dA)
+    dBl = ext.gemm_dsd_lists(A.T, dC.T, lists.transposed(), 32, s, transposed_out=True).T
+    assert max_tile_rel_fro(dBl, rdB, tile=32) <= REL_FRO_TOL

@@ -87,3 +87,31 @@ def test_increment_table_vs_oracle(shape, p, bk):
     assert np.array_equal(table.cpu().numpy(), et)
     assert np.array_equal(ri.cpu().numpy(), eri)
     assert np.array_equal(rw.cpu().numpy(), erw)
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (2, 2), (5, 7), (16, 24), (63, 33), (256, 256), (600, 500)])
+@pytest.mark.parametrize("p", [0.0, 0.5, 0.9])
+def test_merged_lists_of_a_block_size_32_mask_bit_exact(shape, p):
+    """split = 0: a mask at block size 32 listed on the 64 grid with the quadrant keep bits in bits 28-31 of every
+    entry, against the oracle's encoding, for the list by rows and (transposed bits) by columns; masks larger than
+    2^18 listed entries take the multi-launch builder."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(shape[0] * 1000 + shape[1])
+    mask = torch.rand(*shape, generator=gen) < p
+    lists = ext.build_lists(mask.cuda(), split=0)
+    assert lists.shape == ((shape[0] + 1) // 2, (shape[1] + 1) // 2)
+    rp, ci = O.compact_csr_quads(mask.numpy())
+    assert np.array_equal(lists.row_ptr.cpu().numpy(), rp)
+    assert np.array_equal(lists.col_idx[: lists.nnz()].cpu().numpy(), ci)
+    cp, ri = O.compact_csr_quads(mask.numpy().T)
+    assert np.array_equal(lists.col_ptr.cpu().numpy(), cp)
+    assert np.array_equal(lists.row_idx[: lists.nnz()].cpu().numpy(), ri)
+    # the same from a drawn mask
+    drawn, lists = ext.random_lists(shape, p, seed=9, split=0)
+    want = O.random_mask(shape, p, 9)
+    assert np.array_equal(drawn.cpu().numpy(), want)
+    rp, ci = O.compact_csr_quads(want)
+    assert np.array_equal(lists.row_ptr.cpu().numpy(), rp)
+    assert np.array_equal(lists.col_idx[: lists.nnz()].cpu().numpy(), ci)

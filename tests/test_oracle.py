@@ -390,3 +390,41 @@ def test_mlp_with_hidden_tensors_stored_in_fp16(act):
     np.testing.assert_allclose(rdx, x.grad.numpy(), rtol=1e-10, atol=1e-12)
     for got, w in zip(rdws, ws):
         np.testing.assert_allclose(got, w.grad.numpy(), rtol=1e-10, atol=1e-12)
+
+
+@pytest.mark.parametrize("shape", [(4, 6), (5, 7), (1, 1), (9, 2)])
+def test_merged_mask_expands_to_the_same_elements(shape):
+    """merge_mask_quads / compact_csr_quads: a block-size-32 mask and its 64-grid form with quadrant bits describe
+    the same element mask (expand_keep identity), and the encoded list decodes back to mask and bits."""
+    rng = np.random.default_rng(sum(shape))
+    mask = rng.random(shape) < 0.5
+    m, k = shape[0] * 32 - 5, shape[1] * 32 - 9  # ragged last blocks
+    mask64, quads = O.merge_mask_quads(mask)
+    assert mask64.shape == ((shape[0] + 1) // 2, (shape[1] + 1) // 2)
+    keep = O.expand_keep(mask, 32, m, k)
+    rebuilt = np.zeros_like(keep)
+    for i in range(mask64.shape[0]):
+        for j in range(mask64.shape[1]):
+            for a in range(2):
+                for b in range(2):
+                    if quads[i, j] >> (2 * a + b) & 1:
+                        rebuilt[64 * i + 32 * a: 64 * i + 32 * a + 32, 64 * j + 32 * b: 64 * j + 32 * b + 32] = True
+    assert np.array_equal(rebuilt, keep)
+    assert np.array_equal(mask64, quads == 0)
+    row_ptr, enc = O.compact_csr_quads(mask)
+    rp, ci = O.compact_csr(mask64)
+    assert np.array_equal(row_ptr, rp)
+    assert np.array_equal(enc.view(np.uint32) & 0x0FFFFFFF, ci)
+    rows = np.repeat(np.arange(mask64.shape[0]), np.diff(rp))
+    assert np.array_equal(enc.view(np.uint32) >> 28, quads[rows, ci])
+
+
+def test_merged_mask_hand_case():
+    # rows 0-1 x cols 0-1 -> entry (0, 0): kept are (0, 1) and (1, 0): bits 1 and 2; entry (0, 1) covers column 2 only
+    mask = np.array([[1, 0, 1], [0, 1, 0]], dtype=bool)
+    mask64, quads = O.merge_mask_quads(mask)
+    assert mask64.tolist() == [[False, False]]
+    assert quads.tolist() == [[0b0110, 0b0100]]
+    row_ptr, enc = O.compact_csr_quads(mask)
+    assert row_ptr.tolist() == [0, 2]
+    assert enc.view(np.uint32).tolist() == [0 | (0b0110 << 28), 1 | (0b0100 << 28)]
