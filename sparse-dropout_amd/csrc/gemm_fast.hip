@@ -13,7 +13,14 @@
 // looks like: dropped blocks cost neither loads nor MFMAs and no wave idles behind a barrier.
 //
 // Global->LDS goes through global_load_lds_dwordx4 (no VGPR staging), two stages, one barrier per
-// step.  A tile row is 128 B (64 halfs) and its 16-byte chunks are XOR-swizzled with (row>>1)&7,
+// step.  That barrier stands in front of the MFMAs of a step's last (row block, half of the K block) unit,
+// when every fragment of the current stage is in registers: the loads of the step after next and the
+// fragment reads of the next step's first unit are issued behind it and run under those MFMAs, so no wave
+// starts a step by waiting for LDS.  Timed with parts of the kernel switched off (8192^3, dense, all-zero
+// operands): MFMAs + barriers alone 530 us, + fragment reads 652, + tile loads 855, everything 939, and the
+// tile loads + fragment reads without the MFMAs 848 - the L2->LDS path at about 10 TB/s over the chip is the
+// floor, the MFMA work hides behind it incompletely.  Staging the tiles through registers instead
+// (global_load_dwordx4 + ds_write_b128) moves them no faster.  A tile row is 128 B (64 halfs) and its 16-byte chunks are XOR-swizzled with (row>>1)&7,
 // which makes the MFMA fragment reads (ds_read_b128, 16 rows x one chunk per 16-lane group) hit all
 // 64 LDS banks; the swizzle is applied on the global side (which chunk a lane fetches), because the
 // LDS side of a direct load is fixed at lane*16.
@@ -100,17 +107,22 @@ typedef __attribute__((address_space(3))) void lds_void;
 // lgkmcnt(0), and transpose reads get a vmcnt(0) in front), which serialises the fragment reads with
 // the MFMAs.  Written this way the loads are invisible to its counters; the kernels wait for them
 // themselves with s_waitcnt vmcnt(0) before the barrier that publishes a stage.
-__device__ inline void load16_to_lds(const void* g, char* lds_dst) {
-  const uint32_t a = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_void*)lds_dst);
+// lds_dst is the destination's LDS byte address (lds_address() of a pointer, plus wave-uniform offsets): kept as
+// an integer in scalar registers, so no pointer conversion is made per load.
+__device__ inline uint32_t lds_address(const void* p) {
+  return (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)(lds_void*)p);
+}
+__device__ inline void load16_to_lds(const void* g, uint32_t lds_dst) {
+  const uint32_t a = uniform(lds_dst);
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(a) : "memory");
 }
 // The same with the address split into a wave-uniform 64-bit base (SGPRs) and a 32-bit per-lane byte
 // offset: half the VGPR reads per load and no 64-bit VALU add to form the lane addresses.
-__device__ inline void load16_to_lds(const char* base, uint32_t lane_off, char* lds_dst) {
+__device__ inline void load16_to_lds(const char* base, uint32_t lane_off, uint32_t lds_dst) {
   const uint64_t b = (uint64_t)(uintptr_t)base;
   const uint64_t sb = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32)) << 32) |
                       (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
-  const uint32_t a = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_void*)lds_dst);
+  const uint32_t a = uniform(lds_dst);
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(sb), "s"(a)
                : "memory");
 }
@@ -154,6 +166,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   constexpr int BL = S::BL, AL = S::AL, RW = S::RW;
   constexpr bool STEP_COPIES = IMPLICIT != 0 && (TRANS || IMPLICIT == 2);  // input rows copied per step
   extern __shared__ __attribute__((aligned(16))) char smem[];
+  const uint32_t smem_a = lds_address(smem);
   uint32_t* step_e = reinterpret_cast<uint32_t*>(smem + S::SMEM_STEPS);
   uint32_t* scratch = reinterpret_cast<uint32_t*>(smem + S::SMEM_SCRATCH);
   int* nsteps_p = reinterpret_cast<int*>(smem + S::SMEM_SCRATCH + 4 * MAX_STEPS);
@@ -163,6 +176,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   const int tid = threadIdx.x;
   const int lane = tid % 64;
   const int wave = tid / 64;
+  const int wave_u = (int)uniform((uint32_t)wave);  // the same in a scalar register, for load addresses
   const int ns = wave % S::NS;  // column slice
   const int rh = wave / S::NS;  // row-block pair
   const int rb0 = tm * R;   // first row block
@@ -516,7 +530,8 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   auto issue_loads = [&](uint32_t entry, int stage) {  // entry: wave-uniform step table word
     const int kb = step_block(entry);
     const uint32_t fl = step_flags(entry);
-    char* st = smem + stage * STAGE;
+    [[maybe_unused]] char* st = smem + stage * STAGE;
+    const uint32_t st_a = smem_a + (uint32_t)(stage * STAGE);
     const char* bp = b_tile0 + kb * b_red_stride;
     const char* ap = a_tile0 + kb * red_stride;
     const bool red_tail = RAGGED && kb == kb_tail;  // wave-uniform
@@ -525,7 +540,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
       if (b_valid[jj]) {
         uint32_t off = b_lane[jj];
         if (RAGGED) off += red_tail ? b_delta_k[jj] : 0u;
-        load16_to_lds(bp, off, st + (wave * BL + jj) * 1024);
+        load16_to_lds(bp, off, st_a + (uint32_t)((wave_u * BL + jj) * 1024));
       }
 #pragma unroll
     for (int r = 0; r < R; ++r)
@@ -542,7 +557,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
         for (int i = 0; i < AL; ++i) {
           uint32_t off = a_lane[i];
           if (RAGGED) off += (r == r_tail ? a_delta_m[i] : 0u) + (red_tail ? a_delta_k[i] : 0u);
-          load16_to_lds(ap + r * a_rstride, off, st + A_OFF + r * TILE + (wave * AL + i) * 1024);
+          load16_to_lds(ap + r * a_rstride, off, st_a + (uint32_t)(A_OFF + r * TILE + (wave_u * AL + i) * 1024));
         }
       }
   };
@@ -648,6 +663,103 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   // long returned: a read-and-wait at the top of a step would put an LDS round trip in front of its MFMAs.
   const bool late = __builtin_amdgcn_readfirstlane(rh) != 0;
   uint32_t e_cur = uniform(step_e[0]), e_next = uniform(step_e[1]);
+
+  if constexpr (IMPLICIT == 0) {
+    // The products that read their operands from memory run the units of all steps as one chain: the barrier
+    // that publishes the next stage stands in front of the MFMAs of a step's LAST unit, not behind them.  By
+    // then the wave holds every fragment it needs from the current stage in registers (the barrier's own wait
+    // for outstanding LDS reads sees to that), so the one barrier also frees the current stage, and the wave
+    // issues, behind it, the loads of the step after next into that stage and the fragment reads of the next
+    // step's first unit - both run under the last unit's MFMAs instead of in front of the next step's first.
+    u32x4 bf[NT16][2];
+    u32x4 af[2][4];
+    auto wave_quads = [&](uint32_t e) { return (step_flags(e) >> (4 * RW * rh)) & ((1u << (4 * RW)) - 1u); };
+    auto wave_mine = [&](uint32_t q) { return ((q & 0xfu) ? 1u : 0u) | ((RW == 2 && (q >> 4)) ? 2u : 0u); };
+    // fragments of the first unit of the step with table word e, whose tiles are in `stage`
+    auto first_reads = [&](uint32_t e, int stage) {
+      const uint32_t m = wave_mine(wave_quads(e));
+      if (m != 0u) {
+        const char* st = smem + stage * STAGE;
+        read_b(st, 0, bf);
+        read_a(st + A_OFF + (RW * rh + (m == 2u ? 1 : 0)) * TILE, 0, af[0]);
+      }
+    };
+    // the step boundary, see above; e_nn: table word of the step after next (only read when there is one)
+    auto boundary = [&](int step, int stage, uint32_t e_nx, uint32_t e_nn, bool defer_loads = false) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's loads for the next step have landed
+      __syncthreads();
+      if (step + 2 < nsteps && !defer_loads) issue_loads(uniform(e_nn), stage);
+      if (step + 1 < nsteps) first_reads(e_nx, stage ^ 1);
+    };
+    auto units = [&](auto mine_c, int step, int stage, uint32_t e_nx, uint32_t e_nn, bool red_tail,
+                     uint32_t quads) {
+      constexpr int MINE = decltype(mine_c)::value;
+      constexpr int NR = (MINE == 3) ? 2 : 1;
+      constexpr int R0 = (MINE == 2) ? 1 : 0;
+      constexpr bool DEFER = MINE == 3;
+      const char* st = smem + stage * STAGE;
+      const char* at0 = st + A_OFF + (RW * rh + R0) * TILE;
+#pragma unroll
+      for (int u = 0; u < NR * 2; ++u) {
+        const int rr = R0 + u / 2, kk = u % 2;
+        if (u + 1 < NR * 2) {
+          const int kk1 = (u + 1) % 2;
+          if (u + 1 < 2) read_b(st, kk1, bf);
+          read_a(at0 + ((u + 1) / 2) * TILE, kk1, af[(u + 1) & 1]);
+        } else {
+          boundary(step, stage, e_nx, e_nn, DEFER && late);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (RAGGED && g.quads) {  // a mask of block size 32: zero the dropped 32 x 32 quadrants of the tile
+          const uint32_t q = row_quads(quads, rr);
+#pragma unroll
+          for (int mt = 0; mt < 4; ++mt)
+            if (!((q >> (2 * (mt / 2) + kk)) & 1u)) af[u & 1][mt] = u32x4{0u, 0u, 0u, 0u};
+        }
+        if (RAGGED && red_tail) {  // ragged reduction block: nothing past the end may reach the MFMAs
+#pragma unroll
+          for (int mt = 0; mt < 4; ++mt) mask_fragment(af[u & 1][mt], kk);
+          if (u < 2) {  // the W fragments stay masked for the second row block
+#pragma unroll
+            for (int nt = 0; nt < NT16; ++nt) mask_fragment(bf[nt][kk], kk);
+          }
+        }
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+          for (int nt = 0; nt < NT16; ++nt)
+            acc[rr][mt][nt] = T::mfma16(af[u & 1][mt], bf[nt][kk], acc[rr][mt][nt]);
+        __builtin_amdgcn_sched_barrier(0);
+        // with both row blocks at work the second wave of each SIMD issues its loads behind the last MFMAs: the two
+        // waves then run a little out of step, which the dense product gains 3-5 % from
+        if (DEFER && u + 1 == NR * 2 && late && step + 2 < nsteps) issue_loads(uniform(e_nn), stage);
+      }
+    };
+
+    if (nsteps > 0) issue_loads(e_cur, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (nsteps > 1) issue_loads(e_next, 1);
+    if (nsteps > 0) first_reads(e_cur, 0);
+    for (int step = 0; step < nsteps; ++step) {
+      const int stage = step & 1;
+      const uint32_t e_after = step_e[step + 2];  // a VGPR until the boundary makes it uniform
+      const uint32_t quads = wave_quads(e_cur);
+      const uint32_t mine = wave_mine(quads);
+      const bool red_tail = RAGGED && step_block(e_cur) == kb_tail;
+      if constexpr (RW == 2) {
+        if (mine == 3u) units(std::integral_constant<int, 3>{}, step, stage, e_next, e_after, red_tail, quads);
+        else if (mine == 1u) units(std::integral_constant<int, 1>{}, step, stage, e_next, e_after, red_tail, quads);
+        else if (mine == 2u) units(std::integral_constant<int, 2>{}, step, stage, e_next, e_after, red_tail, quads);
+        else boundary(step, stage, e_next, e_after);
+      } else {
+        if (mine) units(std::integral_constant<int, 1>{}, step, stage, e_next, e_after, red_tail, quads);
+        else boundary(step, stage, e_next, e_after);
+      }
+      e_cur = e_next;
+      e_next = uniform(e_after);
+    }
+  } else {
   if constexpr (STEP_COPIES) {
     if (nsteps > 0) {
       tpatch_load(e_cur);
@@ -692,6 +804,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
     __syncthreads();
     e_cur = e_next;
     e_next = uniform(e_after);
+  }
   }
 
   // ---- epilogue: scale, round once, store ---------------------------------------------------------
@@ -780,6 +893,7 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
   extern __shared__ __attribute__((aligned(16))) char smem[];
   // bit r: tile (row block rb0 + r, column block c) kept; bits 8 + 4r .. 11 + 4r: which of its four 32 x 32
   // quadrants (all of them unless the mask has block size 32)
+  const uint32_t smem_a = lds_address(smem);
   uint32_t* flags = reinterpret_cast<uint32_t*>(smem);
   int* rec = reinterpret_cast<int*>(smem + 4 * ((Cb + 3) & ~3));  // c_lo, c_hi, ncols, kept bits, cols[GW]
 
@@ -968,7 +1082,7 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
   const int64_t a_tile_stride = (int64_t)BS * g.a.sr * 2;
   const int64_t b_step_stride = (int64_t)BS * g.b.sc * 2;
   auto issue_loads = [&](int step, int stage) {
-    char* st = smem + stage * G_STAGE + wave * 1024;
+    const uint32_t st = smem_a + (uint32_t)(stage * G_STAGE + wave * 1024);
     const char* ap = a_base + step * (BS * 2);
     const char* bp = b_base + step * b_step_stride;
     const bool red_tail = EDGE && step == s_tail;
@@ -977,14 +1091,14 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
       if (rowmask & (1u << r)) {
         uint32_t off = r == r_tail ? a_lane_m : a_lane;
         if (EDGE) off += red_tail ? a_delta_k : 0u;
-        load16_to_lds(ap + r * a_tile_stride, off, st + r * TILE);
+        load16_to_lds(ap + r * a_tile_stride, off, st + (uint32_t)(r * TILE));
       }
 #pragma unroll
     for (int j = 0; j < GW; ++j)
       if (j < ncols) {
         uint32_t off = b_lane;
         if (EDGE) off += (cols[j] == c_tail ? b_delta_c : 0u) + (red_tail ? b_delta_k : 0u);
-        load16_to_lds(bp + (int64_t)cols[j] * (BS * 2), off, st + G_BOFF + j * TILE);
+        load16_to_lds(bp + (int64_t)cols[j] * (BS * 2), off, st + (uint32_t)(G_BOFF + j * TILE));
       }
   };
   // zeroes the elements of a fragment whose reduction index (32*kk + 8*(lane/16) + 0..7 inside the
@@ -996,7 +1110,8 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
     f.z &= n >= 6 ? ~0u : (n == 5 ? 0xffffu : 0u);
     f.w &= n >= 8 ? ~0u : (n == 7 ? 0xffffu : 0u);
   };
-  // the two waves of a SIMD (w and w + 4) issue their loads half a step apart
+  // the two waves of a SIMD (w and w + 4) issue their loads apart: the first right behind the barrier, the second
+  // behind the step's last MFMAs
   const bool late = wave >= 4;
 
   f32x4 acc[SLOTS][4][4];  // [slot][16-row tile][16-column tile]
@@ -1009,76 +1124,82 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
 #pragma unroll
         for (int v = 0; v < 4; ++v) acc[k][a][b][v] = 0.f;
 
+  // Units u = 2*slot + kk run as one chain over all steps: the fragments of unit u+1 are read before the MFMAs
+  // of unit u, and the barrier that publishes the next stage (and frees the current one: by then the wave holds
+  // all its fragments of it) stands in front of the MFMAs of the step's last unit.  Behind it the wave issues the
+  // loads of the step after next and reads the next step's first fragments, under those MFMAs.
+  u32x4 af[2][4], bf[2][4];
+  auto read_unit = [&](int stage, int u) {
+    const int k = u / 2, kk = u % 2;
+    const char* st = smem + stage * G_STAGE;
+    const char* at = st + my_r[k] * TILE;
+    const char* bt = st + G_BOFF + my_j[k] * TILE;
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+      af[u & 1][h] = *reinterpret_cast<const u32x4*>(at + a_off[kk] + h * 16 * 128);
+      const char* p = bt + (b_off[kk] ^ (h * 32));
+      const u32x2 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * 128);
+      bf[u & 1][h] = u32x4{lo.x, lo.y, hi.x, hi.y};
+    }
+  };
+  auto boundary = [&](int step, int stage, bool defer_loads) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's loads for the next step have landed
+    __syncthreads();
+    if (step + 2 < nsteps && !defer_loads) issue_loads(step + 2, stage);
+    if (step + 1 < nsteps && act[0]) read_unit(stage ^ 1, 0);
+  };
+  auto mfma_unit = [&](auto k_c, int u, bool red_tail) {
+    constexpr int k = decltype(k_c)::value;
+    if (EDGE && red_tail) {  // nothing past the end of the reduction may reach the MFMAs
+#pragma unroll
+      for (int h = 0; h < 4; ++h) {
+        mask_fragment(af[u & 1][h], u % 2);
+        mask_fragment(bf[u & 1][h], u % 2);
+      }
+    }
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) acc[k][mt][nt] = T::mfma16(af[u & 1][mt], bf[u & 1][nt], acc[k][mt][nt]);
+  };
+
   issue_loads(0, 0);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
+  if (nsteps > 1) issue_loads(1, 1);
+  if (act[0]) read_unit(0, 0);
 
   for (int step = 0; step < nsteps; ++step) {
     const int stage = step & 1;
-    const bool more = step + 1 < nsteps;
-    const bool mid = late && more && act[0];
-    if (more && !mid) issue_loads(step + 1, stage ^ 1);
+    const bool red_tail = EDGE && step == s_tail;
+    const bool two = SLOTS == 2 && act[SLOTS - 1];  // the wave's second tile slot is in use: four units, else two
+    const bool defer = late;  // measured: the later the second wave of a SIMD issues its loads, the better
     if (act[0]) {
-      const char* st = smem + stage * G_STAGE;
-      // units u = 2*slot + kk; the fragments of unit u+1 are read before the MFMAs of unit u.  Slot 1's
-      // first fragments are read whether it is active or not (its tile indices are valid either way).
-      u32x4 af[2][4], bf[2][4];
-      auto read_unit = [&](int u) {
-        const int k = u / 2, kk = u % 2;
-        const char* at = st + my_r[k] * TILE;
-        const char* bt = st + G_BOFF + my_j[k] * TILE;
-#pragma unroll
-        for (int h = 0; h < 4; ++h) {
-          af[u & 1][h] = *reinterpret_cast<const u32x4*>(at + a_off[kk] + h * 16 * 128);
-          const char* p = bt + (b_off[kk] ^ (h * 32));
-          const u32x2 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * 128);
-          bf[u & 1][h] = u32x4{lo.x, lo.y, hi.x, hi.y};
-        }
-      };
-      const bool red_tail = EDGE && step == s_tail;
-      // the late waves of slot 0's second unit issue the next step's loads half-way through its MFMAs
-      auto mfma_unit = [&](auto k_c, int u, bool loads_inside) {
-        constexpr int k = decltype(k_c)::value;
-        if (EDGE && red_tail) {  // nothing past the end of the reduction may reach the MFMAs
-#pragma unroll
-          for (int h = 0; h < 4; ++h) {
-            mask_fragment(af[u & 1][h], u % 2);
-            mask_fragment(bf[u & 1][h], u % 2);
-          }
-        }
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt) {
-#pragma unroll
-          for (int nt = 0; nt < 4; ++nt) acc[k][mt][nt] = T::mfma16(af[u & 1][mt], bf[u & 1][nt], acc[k][mt][nt]);
-          if (mt == 1) {
-            __builtin_amdgcn_sched_barrier(0);
-            if (loads_inside) issue_loads(step + 1, stage ^ 1);
-            __builtin_amdgcn_sched_barrier(0);
-          }
-        }
-      };
-      read_unit(0);
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        if (u + 1 < 2 * SLOTS) read_unit(u + 1);
+        if (u == 0) read_unit(stage, 1);
+        else if (two) read_unit(stage, 2);
+        else boundary(step, stage, defer);
         __builtin_amdgcn_sched_barrier(0);
-        mfma_unit(std::integral_constant<int, 0>{}, u, u == 1 && mid);
+        mfma_unit(std::integral_constant<int, 0>{}, u, red_tail);
         __builtin_amdgcn_sched_barrier(0);
       }
       if constexpr (SLOTS == 2) {
-        if (act[1]) {
+        if (two) {
 #pragma unroll
           for (int u = 2; u < 4; ++u) {
-            if (u + 1 < 4) read_unit(u + 1);
+            if (u == 2) read_unit(stage, 3);
+            else boundary(step, stage, defer);
             __builtin_amdgcn_sched_barrier(0);
-            mfma_unit(std::integral_constant<int, 1>{}, u, false);
+            mfma_unit(std::integral_constant<int, 1>{}, u, red_tail);
             __builtin_amdgcn_sched_barrier(0);
           }
         }
       }
+      if (defer && step + 2 < nsteps) issue_loads(step + 2, stage);
+    } else {
+      boundary(step, stage, false);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------------
