@@ -155,6 +155,49 @@ def time_kernel_events(fn, reps: int, flush=None) -> float:
     return statistics.fmean(a.elapsed_time(b) for a, b in ev)
 
 
+def looped_with_clock(fn, seconds: float = 2.5):
+    """fn launched back to back for `seconds`; rocm-smi polled from a thread meanwhile.  Returns microseconds per
+    launch, the median shader clock seen and, from the two, shader cycles per launch."""
+    import re
+    import subprocess
+    import threading
+    import time
+
+    import torch
+
+    clocks = []
+
+    def poll():
+        time.sleep(0.7)
+        for _ in range(3):
+            out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True).stdout
+            m = re.search(r"sclk clock level: \d+: \((\d+)Mhz\)", out)
+            if m:
+                clocks.append(int(m.group(1)))
+            time.sleep(0.3)
+
+    for _ in range(20):
+        fn()
+    torch.cuda.synchronize()
+    th = threading.Thread(target=poll)
+    th.start()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    n, t0 = 0, time.time()
+    a.record()
+    while time.time() - t0 < seconds or th.is_alive():
+        for _ in range(50):
+            fn()
+        n += 50
+        torch.cuda.synchronize()
+    b.record()
+    torch.cuda.synchronize()
+    th.join()
+    us = a.elapsed_time(b) * 1e3 / n
+    mhz = statistics.median(clocks) if clocks else None
+    return {"us_per_launch": round(us, 1), "sclk_mhz": mhz,
+            "kilocycles_per_launch": round(us * mhz / 1e3, 1) if mhz else None}
+
+
 def cpu_baseline(size: int, bs: int, p: float, reps: int):
     """The oracle's literal naive path (mask expand + dense linear + autograd backward) on the host
     cores, fp32, same kind of workload at a bounded size."""
@@ -303,12 +346,11 @@ def main() -> int:
     if not args.no_sweep:
         flush = torch.empty(512 << 20, dtype=torch.int8, device="cuda")  # > L2 + MALL
         t_by_p = {}
-        for p in (0.0, 0.25, 0.5, 0.75):
-            st = Step(*make_problem(size, p, bs), bs, p)
-            for _ in range(3):
-                st()
+        sweep_steps = {p: Step(*make_problem(size, p, bs), bs, p) for p in (0.0, 0.25, 0.5, 0.75)}
+
+        def flushed_median(st, n):
             ts = []
-            for _ in range(max(5, args.steps // 2)):
+            for _ in range(n):
                 flush.zero_()
                 a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 a.record()
@@ -316,7 +358,16 @@ def main() -> int:
                 b.record()
                 torch.cuda.synchronize()
                 ts.append(a.elapsed_time(b))
-            t = statistics.median(ts)
+            return statistics.median(ts)
+
+        # One untimed pass over every p first: under this flush-and-synchronise protocol the first second or so
+        # of measurements comes out 10-15 % slow whatever is measured, which would flatter whichever p goes later.
+        for st in sweep_steps.values():
+            for _ in range(3):
+                st()
+            flushed_median(st, 5)
+        for p, st in sweep_steps.items():
+            t = flushed_median(st, max(5, args.steps // 2))
             t_by_p[p] = t
             sweep.append({
                 "p": p,
@@ -326,9 +377,8 @@ def main() -> int:
                 "dense_equiv_tflops": round(st.flops_dense / (t * 1e-3) / 1e12, 2),
                 "pct_mfma_peak_kept_work": round(100 * st.flops_total / (t * 1e-3) / 1e12 / PEAK_FP16_TFLOPS, 2),
             })
-            del st
         ratio = round(t_by_p[0.5] / t_by_p[0.0], 4)
-        del flush
+        del flush, sweep_steps
 
     dense_reference = None
     if args.dense_reference:
@@ -346,6 +396,13 @@ def main() -> int:
             "torch_matmul_ms": round(time_kernel_events(lambda: torch.matmul(x, w.t(), out=y), reps, flush), 4),
             "sd_gemm_ms": round(time_kernel_events(lambda: step.ext.gemm(x, w, out=y), reps, flush), 4),
             "sd_gemm_dx_layout_ms": round(time_kernel_events(lambda: step.ext.gemm(dy, w.t(), out=step.dx), reps, flush), 4),
+            # the same three in a tight loop (no flush) with the shader clock read beside them: the products run the
+            # chip into its power limit to different degrees, so milliseconds alone do not compare the kernels
+            "looped": {
+                "torch_matmul": looped_with_clock(lambda: torch.matmul(x, w.t(), out=y)),
+                "sd_gemm": looped_with_clock(lambda: step.ext.gemm(x, w, out=y)),
+                "sd_forward_p": looped_with_clock(step.fwd),
+            },
         }
         del flush
 

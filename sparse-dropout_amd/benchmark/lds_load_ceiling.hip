@@ -1,0 +1,120 @@
+// What the global -> LDS path sustains when nothing else happens: every CU streams 64 KB steps into two LDS
+// stages with global_load_lds_dwordx4, one step in flight behind a barrier per step - the load side of the GEMM
+// kernels without their fragment reads and MFMAs - under four address patterns:
+//   private   each workgroup walks its own contiguous region (every byte fetched once per pass; regions small
+//             enough to stay in L2)
+//   rows      each workgroup's step is 512 rows of 128 bytes, 16 KB apart: the tile rows of an 8192-wide fp16
+//             operand, private to the workgroup
+//   shared    the 32 workgroups of an XCD walk the tile rows of 8 + 4 operand panels the way the GEMM's 8 x 4
+//             patch of 256 x 256 tiles does (each step's bytes wanted by 4 or 8 workgroups at the same time);
+//             the panels are `positions` steps long and walked round and round: with 64 positions all panels
+//             together are 192 MB (they stay in the 256 MB memory-side cache), with 128 they are 384 MB (the
+//             L2 misses, a fifth of the requests, go to HBM as 128-byte reads 16 KB apart)
+//   hbm       private regions far larger than the caches
+// It prints bytes into LDS per second over the chip; the GEMM kernels' own rate is to be read against these.
+//
+//   hipcc --offload-arch=gfx950 -O3 -w -Xclang -target-feature -Xclang -packed-fp32-ops \
+//         -o /tmp/lds_load_ceiling sparse-dropout_amd/benchmark/lds_load_ceiling.hip && /tmp/lds_load_ceiling
+#include <hip/hip_runtime.h>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+
+typedef __attribute__((address_space(3))) void lds_void;
+constexpr int STAGE = 65536, THREADS = 512, LOADS = 8;  // per wave and step: 8 loads of 1 KB
+
+__device__ inline void load16_to_lds(const char* base, uint32_t lane_off, uint32_t lds_dst) {
+  const uint64_t b = (uint64_t)(uintptr_t)base;
+  const uint64_t sb = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32)) << 32) |
+                      (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+  const uint32_t a = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_dst);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(sb), "s"(a)
+               : "memory");
+}
+
+// mode 0: private contiguous; 1: private tile rows; 2: shared panels of an XCD patch
+// reads: 1 KB ds_read_b128 per wave and step from the stage that has landed (the GEMM kernels read 24: 16 KB of X
+// fragments and 8 KB of W fragments per wave)
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(THREADS) void stream(const char* src, size_t region, int steps, int mode, int reads,
+                                                  int positions, int* sink) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const uint32_t smem_a = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)(lds_void*)smem);
+  const int lane = threadIdx.x % 64, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+  const int wg = blockIdx.x;
+  const size_t ROW = 16384;  // bytes between tile rows
+  // per-lane offset inside a 1 KB load: 8 rows x 128 B for the row patterns, 1 KB contiguous otherwise
+  const uint32_t lane_off = mode == 0 ? lane * 16 : (uint32_t)((lane / 8) * ROW + (lane % 8) * 16);
+  // panels of the shared pattern: workgroup (r, c) of the XCD's 8 x 4 patch reads row panel r and column panel c
+  const int xcd = wg % 8, slot = wg / 8;  // consecutive workgroups go to consecutive XCDs
+  const int pr = slot % 8, pc = slot / 8 % 4;
+  auto issue = [&](int step, int stage) {
+    const uint32_t st = smem_a + stage * STAGE + wave * (LOADS * 1024);
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const char* p;
+      if (mode == 0) {
+        p = src + (size_t)wg * region + ((size_t)step * STAGE + (wave * LOADS + i) * 1024) % region;
+      } else if (mode == 1) {
+        // 64 loads of 8 rows = 512 rows of this workgroup's own 512-row band; a step moves 128 bytes along the rows
+        p = src + (size_t)wg * 512 * ROW + (size_t)(wave * LOADS + i) * 8 * ROW + (size_t)(step % positions) * 128;
+      } else {
+        // loads 0-31: 256 rows of row panel pr; loads 32-63: 256 rows of column panel pc (panels of 256 rows)
+        const int l = wave * LOADS + i;
+        const int panel = l < 32 ? pr : 8 + pc;
+        p = src + ((size_t)xcd * 12 + panel) * 256 * ROW + (size_t)(l % 32) * 8 * ROW + (size_t)(step % positions) * 128;
+      }
+      load16_to_lds(p, lane_off, st + i * 1024);
+    }
+  };
+  u32x4 x = {0, 0, 0, 0};
+  issue(0, 0);
+  for (int step = 0; step < steps; ++step) {
+    if (step + 1 < steps) {
+      issue(step + 1, (step + 1) & 1);
+      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");  // the loads of this step have landed, the next 8 fly
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();
+    const char* st = smem + (step & 1) * STAGE + lane * 16;
+    for (int i = 0; i < reads; ++i) x ^= *reinterpret_cast<const u32x4*>(st + ((wave * 24 + i) % 64) * 1024);
+  }
+  if ((x.x ^ x.y ^ x.z ^ x.w) == 0x12345678u) sink[wg] = 1;
+  if (threadIdx.x == 0) sink[wg] = *reinterpret_cast<int*>(smem + (steps & 1) * 4);
+}
+
+int main() {
+  const int wgs = 256, steps = 2048;
+  const size_t bytes = (size_t)8 << 30;
+  char* d;
+  if (hipMalloc(&d, bytes) != hipSuccess) { printf("hipMalloc failed\n"); return 1; }
+  hipMemset(d, 1, bytes);
+  int* sink; hipMalloc(&sink, wgs * 4);
+  hipFuncSetAttribute((const void*)stream, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * STAGE);
+  struct { const char* name; int mode; size_t region; int reads; int positions; } cases[] = {
+      {"private, 64 KB regions (L2)", 0, (size_t)64 << 10, 0, 128},
+      {"private, 512 KB regions", 0, (size_t)512 << 10, 0, 128},
+      {"hbm: private, 16 MB regions", 0, (size_t)16 << 20, 0, 128},
+      {"rows: private tile rows", 1, 0, 0, 128},
+      {"shared, 192 MB of panels", 2, 0, 0, 64},
+      {"shared, 192 MB + 24 KB LDS reads / wave", 2, 0, 24, 64},
+      {"shared, 384 MB of panels", 2, 0, 0, 128},
+      {"shared, 384 MB + 24 KB LDS reads / wave", 2, 0, 24, 128},
+  };
+  for (auto& c : cases) {
+    for (int rep = 0; rep < 2; ++rep) {
+      hipEvent_t e0, e1; hipEventCreate(&e0); hipEventCreate(&e1);
+      stream<<<wgs, THREADS, 2 * STAGE>>>(d, c.region, 64, c.mode, c.reads, c.positions, sink);
+      hipDeviceSynchronize();
+      hipEventRecord(e0);
+      stream<<<wgs, THREADS, 2 * STAGE>>>(d, c.region, steps, c.mode, c.reads, c.positions, sink);
+      hipEventRecord(e1); hipEventSynchronize(e1);
+      float ms; hipEventElapsedTime(&ms, e0, e1);
+      if (hipGetLastError() != hipSuccess) { printf("launch failed\n"); return 1; }
+      const double tb = (double)wgs * steps * STAGE / (ms * 1e-3) / 1e12;
+      printf("%-40s %8.3f ms  %6.2f TB/s into LDS  (%.1f B/clk/CU at 2.4 GHz)\n", c.name, ms, tb, tb * 1e12 / 256 / 2.4e9);
+    }
+  }
+  return 0;
+}
