@@ -67,15 +67,20 @@ def _run(cmd: list[str]) -> None:
         raise RuntimeError(f"command failed: {' '.join(cmd)}\n{proc.stdout}\n{err}")
 
 
-def build(force: bool = False, verbose: bool = False) -> Path:
-    OUT_DIR.mkdir(parents=True, exist_ok=True)
+def write_source_hash() -> Path:
+    """(Re)writes the generated header api.hip includes; touched only when the hash changes."""
     OBJ_DIR.mkdir(parents=True, exist_ok=True)
-    headers = sorted(CSRC.glob("*.h")) + sorted((ROOT / "include").glob("*.h"))
     inc = OBJ_DIR / "source_hash.inc"
     line = f'#define SD_SOURCE_HASH "{source_hash()}"\n'
     if not inc.exists() or inc.read_text() != line:
-        inc.write_text(line)  # newer than api.o: api.hip, which includes it, is recompiled below
-    headers.append(inc)
+        inc.write_text(line)  # newer than api.o: api.hip, which includes it, is recompiled by build()
+    return inc
+
+
+def build(force: bool = False, verbose: bool = False) -> Path:
+    OUT_DIR.mkdir(parents=True, exist_ok=True)
+    headers = sorted(CSRC.glob("*.h")) + sorted((ROOT / "include").glob("*.h"))
+    headers.append(write_source_hash())
     jobs = []
     objs = []
     for src in sources():

@@ -16,11 +16,13 @@
 // step.  That barrier stands in front of the MFMAs of a step's last (row block, half of the K block) unit,
 // when every fragment of the current stage is in registers: the loads of the step after next and the
 // fragment reads of the next step's first unit are issued behind it and run under those MFMAs, so no wave
-// starts a step by waiting for LDS.  Timed with parts of the kernel switched off (8192^3, dense, all-zero
-// operands): MFMAs + barriers alone 530 us, + fragment reads 652, + tile loads 855, everything 939, and the
-// tile loads + fragment reads without the MFMAs 848 - the L2->LDS path at about 10 TB/s over the chip is the
-// floor, the MFMA work hides behind it incompletely.  Staging the tiles through registers instead
-// (global_load_dwordx4 + ds_write_b128) moves them no faster.  A tile row is 128 B (64 halfs) and its 16-byte chunks are XOR-swizzled with (row>>1)&7,
+// starts a step by waiting for LDS.  Timed with parts of the loop compiled out (benchmark/decompose.py; 8192^3,
+// dense, all-zero operands): MFMAs + barriers alone 527 us, + fragment reads 643, + tile loads 802, everything 831, and
+// the tile loads + fragment reads without the MFMAs 808 - the parts add up instead of overlapping, because a wave that
+// stands at a load or a fragment read (the texture path takes a 1 KB load every 25 clocks or so, the LDS a 1 KB read
+// every 8) issues no MFMA behind it, and the data side alone is the floor.  Staging the tiles through registers
+// (global_load_dwordx4 + ds_write_b128) moves them no faster, dealing loads and reads out between the MFMAs loses.
+// A tile row is 128 B (64 halfs) and its 16-byte chunks are XOR-swizzled with (row>>1)&7,
 // which makes the MFMA fragment reads (ds_read_b128, 16 rows x one chunk per 16-lane group) hit all
 // 64 LDS banks; the swizzle is applied on the global side (which chunk a lane fetches), because the
 // LDS side of a direct load is fixed at lane*16.
@@ -664,6 +666,9 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   const bool late = __builtin_amdgcn_readfirstlane(rh) != 0;
   uint32_t e_cur = uniform(step_e[0]), e_next = uniform(step_e[1]);
 
+  // SD_TIMING_NO_LOADS / SD_TIMING_NO_READS / SD_TIMING_NO_MFMA compile the tile loads / the fragment reads / the
+  // MFMAs out of the step loop below: builds for timing what the rest costs (benchmark/decompose.py), whose results
+  // are wrong by construction.  The library is never built with them.
   if constexpr (IMPLICIT == 0) {
     // The products that read their operands from memory run the units of all steps as one chain: the barrier
     // that publishes the next stage stands in front of the MFMAs of a step's LAST unit, not behind them.  By
@@ -688,8 +693,12 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
     auto boundary = [&](int step, int stage, uint32_t e_nx, uint32_t e_nn, bool defer_loads = false) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's loads for the next step have landed
       __syncthreads();
+#ifndef SD_TIMING_NO_LOADS
       if (step + 2 < nsteps && !defer_loads) issue_loads(uniform(e_nn), stage);
+#endif
+#ifndef SD_TIMING_NO_READS
       if (step + 1 < nsteps) first_reads(e_nx, stage ^ 1);
+#endif
     };
     auto units = [&](auto mine_c, int step, int stage, uint32_t e_nx, uint32_t e_nn, bool red_tail,
                      uint32_t quads) {
@@ -703,9 +712,11 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
       for (int u = 0; u < NR * 2; ++u) {
         const int rr = R0 + u / 2, kk = u % 2;
         if (u + 1 < NR * 2) {
+#ifndef SD_TIMING_NO_READS
           const int kk1 = (u + 1) % 2;
           if (u + 1 < 2) read_b(st, kk1, bf);
           read_a(at0 + ((u + 1) / 2) * TILE, kk1, af[(u + 1) & 1]);
+#endif
         } else {
           boundary(step, stage, e_nx, e_nn, DEFER && late);
         }
@@ -728,11 +739,17 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
         for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
           for (int nt = 0; nt < NT16; ++nt)
+#ifdef SD_TIMING_NO_MFMA
+            acc[rr][mt][nt][0] += __builtin_bit_cast(float, af[u & 1][mt].x ^ bf[nt][kk].x);
+#else
             acc[rr][mt][nt] = T::mfma16(af[u & 1][mt], bf[nt][kk], acc[rr][mt][nt]);
+#endif
         __builtin_amdgcn_sched_barrier(0);
         // with both row blocks at work the second wave of each SIMD issues its loads behind the last MFMAs: the two
         // waves then run a little out of step, which the dense product gains 3-5 % from
+#ifndef SD_TIMING_NO_LOADS
         if (DEFER && u + 1 == NR * 2 && late && step + 2 < nsteps) issue_loads(uniform(e_nn), stage);
+#endif
       }
     };
 
@@ -741,6 +758,10 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
     __syncthreads();
     if (nsteps > 1) issue_loads(e_next, 1);
     if (nsteps > 0) first_reads(e_cur, 0);
+#ifdef SD_TIMING_NO_READS
+    read_b(smem, 1, bf);  // fragments are read once, here, and never again
+    read_a(smem + A_OFF, 1, af[1]);
+#endif
     for (int step = 0; step < nsteps; ++step) {
       const int stage = step & 1;
       const uint32_t e_after = step_e[step + 2];  // a VGPR until the boundary makes it uniform
