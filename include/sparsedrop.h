@@ -336,6 +336,25 @@ int sd_dropout_matmul_backward(const void* dY, int64_t dy_stride_r, int64_t dy_s
                                int64_t M, int64_t N, int64_t K, int64_t block_size, float p, int dtype,
                                void* workspace, int64_t workspace_bytes, void* stream);
 
+/* The same with the derivative of an activation multiplied into dX (sd_gemm_sdd_lists_actgrad's epilogue):
+ * dX = (dY . W) . keep / (1 - p) * act'(act_at[m, k]), for a layer whose input is act(previous layer's output);
+ * act = SD_ACT_NONE is the plain call.  No counterpart in the reference, whose layers run the activation gradient as a
+ * kernel of its own.
+ * Where both gradients are asked for and neither product would fill the chip by itself (at most 512 workgroups each,
+ * both on the same workgroup shape), the two run as ONE launch - the weight gradient's workgroups follow the input
+ * gradient's in the same grid - so small layers pay for one launch and run the two side by side.
+ * SPARSEDROP_SEPARATE_BACKWARD=1 in the environment keeps them apart (for comparing). */
+int sd_dropout_matmul_backward_act(const void* dY, int64_t dy_stride_r, int64_t dy_stride_c,
+                                   const void* W, int64_t w_stride_r, int64_t w_stride_c,
+                                   const void* X, int64_t x_stride_r, int64_t x_stride_c,
+                                   void* dX, int64_t dx_stride_r, int64_t dx_stride_c,
+                                   void* dW, int64_t dw_stride_r, int64_t dw_stride_c,
+                                   const int32_t* row_ptr, const int32_t* col_idx,
+                                   const int32_t* col_ptr, const int32_t* row_idx,
+                                   int64_t M, int64_t N, int64_t K, int64_t block_size, float p, int dtype,
+                                   int act, const void* act_at, int64_t at_stride_r, int64_t at_stride_c,
+                                   void* workspace, int64_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * (e) im2col gather feeding the same GEMMs for conv.
  *

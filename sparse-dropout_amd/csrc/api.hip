@@ -70,12 +70,26 @@ int check_sparse(int64_t bs, float scale) {
 
 thread_local const char* last_kernel = "";
 
-int run(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
+bool generic_forced() {
   static const bool force_generic = [] {
     const char* e = std::getenv("SPARSEDROP_FORCE_GENERIC");
     return e && e[0] == '1';
   }();
-  if (!force_generic) {
+  return force_generic;
+}
+
+// SPARSEDROP_SEPARATE_BACKWARD=1: sd_dropout_matmul_backward launches its two products one after the other even where
+// they qualify for the single launch (for comparing the two)
+bool separate_backward_forced() {
+  static const bool forced = [] {
+    const char* e = std::getenv("SPARSEDROP_SEPARATE_BACKWARD");
+    return e && e[0] == '1';
+  }();
+  return forced;
+}
+
+int run(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
+  if (!generic_forced()) {
     const int rc = launch_fast(g, mode, dtype, stream);
     if (rc != SD_ERR_UNSUPPORTED) {
       last_kernel = "specialised";
@@ -486,16 +500,49 @@ int sd_dropout_matmul_backward(const void* dY, int64_t gsr, int64_t gsc, const v
                                void* dW, int64_t dwsr, int64_t dwsc, const int32_t* row_ptr, const int32_t* col_idx,
                                const int32_t* col_ptr, const int32_t* row_idx, int64_t M, int64_t N, int64_t K,
                                int64_t bs, float p, int dtype, void* workspace, int64_t workspace_bytes, void* stream) {
+  return sd_dropout_matmul_backward_act(dY, gsr, gsc, W, wsr, wsc, X, xsr, xsc, dX, dxsr, dxsc, dW, dwsr, dwsc, row_ptr,
+                                        col_idx, col_ptr, row_idx, M, N, K, bs, p, dtype, SD_ACT_NONE, nullptr, 0, 0,
+                                        workspace, workspace_bytes, stream);
+}
+
+int sd_dropout_matmul_backward_act(const void* dY, int64_t gsr, int64_t gsc, const void* W, int64_t wsr, int64_t wsc,
+                                   const void* X, int64_t xsr, int64_t xsc, void* dX, int64_t dxsr, int64_t dxsc,
+                                   void* dW, int64_t dwsr, int64_t dwsc, const int32_t* row_ptr,
+                                   const int32_t* col_idx, const int32_t* col_ptr, const int32_t* row_idx, int64_t M,
+                                   int64_t N, int64_t K, int64_t bs, float p, int dtype, int act, const void* act_at,
+                                   int64_t at_stride_r, int64_t at_stride_c, void* workspace, int64_t workspace_bytes,
+                                   void* stream) {
   SD_REQUIRE(p >= 0.f && p < 1.f, "dropout_matmul_backward: p must be in [0, 1) (got %g)", (double)p);
+  if (dX) {
+    if (int rc = check_act(act, act_at, at_stride_r, at_stride_c, M, K, true)) return rc;
+  }
   if (int rc = check_sparse(bs, 1.f)) return rc;
   SD_REQUIRE(dX || dW, "dropout_matmul_backward: nothing to compute");
   const int64_t g = bs == 32 ? 32 : list_granule(bs);  // 32: lists on the 64 grid with quadrant bits
   const float scale = 1.f / (1.f - p);
+  if (dX && dW && row_ptr && col_idx && col_ptr && row_idx && !generic_forced() && !separate_backward_forced()) {
+    // both gradients in one launch where the pair qualifies (same operands and checks as the two calls below)
+    if (int rc = check_common(dY, gsr, gsc, W, wsc, wsr, dX, dxsr, dxsc, M, K, N, dtype)) return rc;
+    if (int rc = check_common(X, xsc, xsr, dY, gsc, gsr, dW, dwsc, dwsr, K, N, M, dtype)) return rc;
+    GemmArgs gx = make_args(dY, gsr, gsc, W, wsc, wsr, dX, dxsr, dxsc, M, K, N, g, scale, row_ptr, col_idx);
+    gx.keep_hint = 1.f - p;
+    gx.act = act;
+    gx.aux = act != SD_ACT_NONE ? const_cast<uint16_t*>(static_cast<const uint16_t*>(act_at)) : nullptr;
+    gx.aux_sr = at_stride_r;
+    gx.aux_sc = at_stride_c;
+    GemmArgs gw = make_args(X, xsc, xsr, dY, gsc, gsr, dW, dwsc, dwsr, K, N, M, g, scale, col_ptr, row_idx, workspace,
+                            workspace_bytes);
+    const int rc = launch_backward_pair(gx, gw, dtype, (hipStream_t)stream);
+    if (rc != SD_ERR_UNSUPPORTED) {
+      last_kernel = "specialised";
+      return rc;
+    }
+  }
   if (dX) {
     // dX[M,K] = scale * (dY[M,N] . W[N,K]) where kept: A = dY, B = W^T as the [K, N] view of W
     SD_REQUIRE(row_ptr && col_idx, "dropout_matmul_backward: dX needs the CSR lists");
-    if (int rc = sd_gemm_sdd_lists_ex(dY, gsr, gsc, W, wsc, wsr, dX, dxsr, dxsc, row_ptr, col_idx, M, K, N, g, scale,
-                                      dtype, 0, 1.f - p, stream))
+    if (int rc = sd_gemm_sdd_lists_actgrad(dY, gsr, gsc, W, wsc, wsr, dX, dxsr, dxsc, row_ptr, col_idx, M, K, N, g,
+                                           scale, dtype, act, act_at, at_stride_r, at_stride_c, 1.f - p, stream))
       return rc;
   }
   if (dW) {

@@ -285,6 +285,9 @@ int fast_splits(int64_t M, int64_t N, int64_t K);
 int launch_splitk_reduce(const GemmArgs& g, int splits, bool trans_out, int dtype, hipStream_t stream);
 // returns SD_ERR_UNSUPPORTED (without setting an error message) when the fast path does not apply
 int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream);
+// dX (SDD) and dW (DSD, reduction-strided operands, column-major C) of one layer in a single launch;
+// SD_ERR_UNSUPPORTED with nothing launched when the pair does not qualify
+int launch_backward_pair(const GemmArgs& gx, const GemmArgs& gw, int dtype, hipStream_t stream);
 // forward of the block-dropout convolution without the patch matrix: g.a is unused, g.b the [K_out, C*R*S]
 // weight matrix, g.c the [N*P*Q, K_out] output, the lists over the patch matrix's block grid.  Returns
 // SD_ERR_UNSUPPORTED (without an error message) for geometries it does not take.

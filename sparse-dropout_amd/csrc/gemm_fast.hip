@@ -44,6 +44,7 @@
 // (swizzled as in the forward), W tiles reduction-strided (read with ds_read_b64_tr_b16 as in dW).  See
 // sdd_group_kernel for how tiles are grouped into workgroups; dropped tiles are written as zeros.
 #include <atomic>
+#include <cstdlib>
 #include <type_traits>
 
 #include "common.h"
@@ -159,9 +160,11 @@ __device__ inline int swz_w(int row) { return ((row & 3) << 2) ^ (((row >> 3) & 
 // a tap falls outside the image never has to be asked: the copy carries a halo of zeros.
 // IMPLICIT = 2: the same with a copy per step that holds only the channels of the step's 64 columns (any number
 // of input channels fits); the reduction-strided instance (the weight gradient) always works that way.
+// bid: the workgroup's index in the launch order of this product; the reduction is split nsplit ways and this
+// workgroup takes part `split` (the kernels below pass their block indices; the fused backward launch its own)
 template <typename T, bool TRANS, bool CM, bool RAGGED, typename S, int IMPLICIT = 0>
-__global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m, int tiles_n,
-                                                         int Mb, int Kb_all, ImplicitConv cg) {
+__device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int tiles_n, int Mb, int Kb_all,
+                                         const ImplicitConv& cg, const int bid, const int nsplit, const int split) {
   static_assert(!IMPLICIT || (S::R == 4 && S::THREADS == 512), "the gather assumes 512 threads x 4 row blocks");
   static_assert(S::R <= 4, "a step's keep bits are four per row block in 16 bits");
   constexpr int R = S::R, BN = S::BN, THREADS = S::THREADS, NT = S::NT, STAGE = S::STAGE, A_OFF = S::A_OFF;
@@ -174,7 +177,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   int* nsteps_p = reinterpret_cast<int*>(smem + S::SMEM_SCRATCH + 4 * MAX_STEPS);
 
   int tm, tn;
-  tile_of_block<DSD_GROUP_M>(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  tile_of_block<DSD_GROUP_M>(bid, tiles_m, tiles_n, tm, tn);
   const int tid = threadIdx.x;
   const int lane = tid % 64;
   const int wave = tid / 64;
@@ -184,8 +187,7 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   const int rb0 = tm * R;   // first row block
   const int64_t n0 = (int64_t)tn * BN;
   const int nvalid = (int)((g.N - n0) < BN ? (g.N - n0) : BN);  // columns of this tile inside C
-  // split reduction: blockIdx.y takes the reduction blocks [kb_lo, kb_lo + Kb) and leaves an fp32 partial
-  const int nsplit = gridDim.y, split = blockIdx.y;
+  // split reduction: part `split` takes the reduction blocks [kb_lo, kb_lo + Kb) and leaves an fp32 partial
   const int kb_lo = (int)((int64_t)Kb_all * split / nsplit);
   const int Kb = (int)((int64_t)Kb_all * (split + 1) / nsplit) - kb_lo;
 
@@ -862,6 +864,13 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
   }
 }
 
+template <typename T, bool TRANS, bool CM, bool RAGGED, typename S, int IMPLICIT = 0>
+__global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m, int tiles_n,
+                                                         int Mb, int Kb_all, ImplicitConv cg) {
+  dsd_body<T, TRANS, CM, RAGGED, S, IMPLICIT>(g, tiles_m, tiles_n, Mb, Kb_all, cg, (int)blockIdx.x, (int)gridDim.y,
+                                              (int)blockIdx.y);
+}
+
 // ---- SDD with column groups ---------------------------------------------------------------------------
 // A = dY [M, red] reduction-contiguous; B = W^T [cols, red] given with the reduction index strided
 // (b.sr == 1); C row-major.  Mb x Cb is the block grid of the output (and of the mask); without a list
@@ -908,8 +917,7 @@ constexpr int G_MAX_CB = 8192;             // per-column flags share the first s
 // matrix instead, as in the DSD kernel, the fragments of the last reduction block are zeroed past the end,
 // and nothing is stored past the last column.  (A ragged M costs nothing worth a separate instance.)
 template <typename T, bool EDGE, typename G>
-__global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tiles_m, int gmax, int Mb,
-                                                            int Cb) {
+__device__ __forceinline__ void sdd_body(const GemmArgs& g, int tiles_m, int gmax, int Mb, int Cb, const int bid) {
   constexpr int R = G::R, GW = G::GW, SLOTS = G::SLOTS, G_BOFF = G::BOFF, G_STAGE = G::STAGE;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   // bit r: tile (row block rb0 + r, column block c) kept; bits 8 + 4r .. 11 + 4r: which of its four 32 x 32
@@ -919,7 +927,7 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
   int* rec = reinterpret_cast<int*>(smem + 4 * ((Cb + 3) & ~3));  // c_lo, c_hi, ncols, kept bits, cols[GW]
 
   int tm, gi;
-  tile_of_block<SDD_GROUP_M>(blockIdx.x, tiles_m, gmax, tm, gi);
+  tile_of_block<SDD_GROUP_M>(bid, tiles_m, gmax, tm, gi);
   const int tid = threadIdx.x;
   const int lane = tid % 64;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
@@ -1247,6 +1255,33 @@ __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tile
   }
 }
 
+template <typename T, bool EDGE, typename G>
+__global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tiles_m, int gmax, int Mb, int Cb) {
+  sdd_body<T, EDGE, G>(g, tiles_m, gmax, Mb, Cb, (int)blockIdx.x);
+}
+
+// Both gradients of one layer in one launch: workgroups [0, n_dx) are the SDD product's (dX; those past its own
+// grid exit: n_dx is rounded up to the 8 XCDs so that the second product's tile map keeps its XCD assignment), the
+// rest the weight gradient's (DSD on reduction-strided operands, column-major C; a split reduction leaves fp32
+// partials for the reduce pass as in the kernel of its own).  One launch instead of
+// two, and the second product's workgroups fill the CUs the first one's last round leaves idle - for small layers,
+// whose grids cover a fraction of the chip each, the two simply run side by side.
+template <typename T, bool EDGE, typename G, typename S>
+__global__ __launch_bounds__(THREADS) void backward_pair_kernel(GemmArgs gx, int x_tiles_m, int x_gmax, int x_Mb,
+                                                                int x_Cb, int n_dx, GemmArgs gw, int w_tiles_m,
+                                                                int w_tiles_n, int w_Mb, int w_Kb, int w_splits) {
+  static_assert(S::THREADS == THREADS, "both products run on 512 threads");
+  const int bid = (int)blockIdx.x;
+  if (bid < n_dx) {
+    if (bid < x_tiles_m * x_gmax) sdd_body<T, EDGE, G>(gx, x_tiles_m, x_gmax, x_Mb, x_Cb, bid);
+  } else {
+    // the weight gradient's workgroups, tile index fastest, then the part of a split reduction
+    const int wb = bid - n_dx, w_tiles = w_tiles_m * w_tiles_n;
+    dsd_body<T, true, true, EDGE, S, 0>(gw, w_tiles_m, w_tiles_n, w_Mb, w_Kb, ImplicitConv{}, wb % w_tiles, w_splits,
+                                        wb / w_tiles);
+  }
+}
+
 bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
 
 // Raises a kernel's dynamic LDS limit once per device (the attribute belongs to the device's copy of the
@@ -1493,6 +1528,33 @@ int launch_conv_implicit(const GemmArgs& g, const ImplicitConv& cg, int64_t P, i
   return ragged ? launch_conv_t<F16, true, 1>(g, cg, smem, stream) : launch_conv_t<F16, false, 1>(g, cg, smem, stream);
 }
 
+// How many ways the DSD kernel splits the reduction of this product: the plan's count cut down to what the caller's
+// scratch holds; 0 = the specialised kernel should not take the product (its step table is per workgroup, and with
+// scratch too small for its own partials the generic kernel's split may still fit).
+int usable_splits(const GemmArgs& g, const DsdPlan& plan, int mode) {
+  const int64_t tiles = plan.mid ? dsd_tiles<DsdMid>(g.M, g.N) : dsd_tiles<DsdBig>(g.M, g.N);
+  int splits = plan.splits;
+  const int64_t part_bytes = g.M * g.N * 4;
+  if (splits > 1 && (g.ws == nullptr || g.ws_bytes < part_bytes * splits))
+    splits = g.ws ? (int)(g.ws_bytes / part_bytes) : 1;
+  if (splits < 1) splits = 1;
+  if (((g.K + BS - 1) / BS + splits - 1) / splits > MAX_STEPS) return 0;
+  if (splits == 1 && tiles < 128 && g.ws != nullptr) {
+    const int gs = generic_splits(g.M, g.N, g.K, g.bs, mode);
+    if (gs > 1 && g.ws_bytes >= (int64_t)gs * part_bytes) return 0;
+  }
+  return splits;
+}
+
+// most workgroups either product of a single-launch backward may have (SPARSEDROP_PAIR_LIMIT overrides, for measuring)
+int64_t pair_limit() {
+  static const int64_t limit = [] {
+    const char* e = std::getenv("SPARSEDROP_PAIR_LIMIT");
+    return e ? (int64_t)std::atoll(e) : (int64_t)512;
+  }();
+  return limit;
+}
+
 int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   if (mode == kSdd) return try_sdd(g, dtype, stream);
   // a dense product of a row-major A with a reduction-strided B (dX = dY.W without dropout) is the SDD
@@ -1514,17 +1576,8 @@ int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   if (!(nt || tn) || !shape_ok || !align_ok || tiles > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
   // few output tiles and a long reduction (the weight gradient of a tall matrix): split the reduction
   // over workgroups when the caller gave scratch for the fp32 partials
-  int splits = plan.splits;
-  const int64_t part_bytes = g.M * g.N * 4;
-  if (splits > 1 && (g.ws == nullptr || g.ws_bytes < part_bytes * splits))
-    splits = g.ws ? (int)(g.ws_bytes / part_bytes) : 1;
-  if (splits < 1) splits = 1;
-  if (((g.K + BS - 1) / BS + splits - 1) / splits > MAX_STEPS) return SD_ERR_UNSUPPORTED;  // step table is per workgroup
-  if (splits == 1 && tiles < 128 && g.ws != nullptr) {
-    // scratch too small for this kernel's partials: the generic kernel's split may still fit
-    const int gs = generic_splits(g.M, g.N, g.K, g.bs, mode);
-    if (gs > 1 && g.ws_bytes >= (int64_t)gs * part_bytes) return SD_ERR_UNSUPPORTED;
-  }
+  const int splits = usable_splits(g, plan, mode);
+  if (splits < 1) return SD_ERR_UNSUPPORTED;
   const bool mid = plan.mid;
   if (dtype == SD_BF16) {
     if (nt) return cm ? launch_dsd<BF16, false, true>(g, mid, splits, stream) : launch_dsd<BF16, false, false>(g, mid, splits, stream);
@@ -1532,6 +1585,78 @@ int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   }
   if (nt) return cm ? launch_dsd<F16, false, true>(g, mid, splits, stream) : launch_dsd<F16, false, false>(g, mid, splits, stream);
   return cm ? launch_dsd<F16, true, true>(g, mid, splits, stream) : launch_dsd<F16, true, false>(g, mid, splits, stream);
+}
+
+// ---- both gradients in one launch ------------------------------------------------------------------------
+// gx: the SDD product dX = s (dY . W) on the kept tiles; gw: the DSD product dW^T = s X^T(kept blocks) . dY with
+// reduction-strided operands and column-major C.  SD_ERR_UNSUPPORTED (nothing launched) unless each would run on its
+// specialised kernel by itself, unsplit, and both on the same size of workgroup shape; the caller then launches them
+// one after the other.
+template <typename T, bool EDGE, typename G, typename S>
+int launch_pair_t(const GemmArgs& gx, const GemmArgs& gw, int splits, hipStream_t stream) {
+  constexpr int SMEM = G::SMEM > S::SMEM_BYTES ? G::SMEM : S::SMEM_BYTES;
+  static std::atomic<bool> configured[kMaxDevices] = {};
+  if (int rc = allow_big_lds(reinterpret_cast<const void*>(&backward_pair_kernel<T, EDGE, G, S>), SMEM, configured))
+    return rc;
+  const int x_Mb = (int)((gx.M + BS - 1) / BS), x_Cb = (int)((gx.N + BS - 1) / BS);
+  const int x_tiles_m = (x_Mb + G::R - 1) / G::R, x_gmax = (x_Cb + G::MINCOLS - 1) / G::MINCOLS;
+  const int64_t n_dx = ((int64_t)x_tiles_m * x_gmax + 7) / 8 * 8;
+  const int w_Mb = (int)((gw.M + BS - 1) / BS), w_Kb = (int)((gw.K + BS - 1) / BS);
+  const int w_tiles_m = (w_Mb + S::R - 1) / S::R, w_tiles_n = (int)((gw.N + S::BN - 1) / S::BN);
+  const int64_t total = n_dx + (int64_t)w_tiles_m * w_tiles_n * splits;
+  if (total > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL((backward_pair_kernel<T, EDGE, G, S>), dim3((unsigned)total), dim3(THREADS), SMEM, stream, gx,
+                     x_tiles_m, x_gmax, x_Mb, x_Cb, (int)n_dx, gw, w_tiles_m, w_tiles_n, w_Mb, w_Kb, splits);
+  note_kernel("pair:sdd+dsd:%s%s splits=%d", G::R == 4 ? "big" : "mid", EDGE ? ":ragged" : "", splits);
+  if (int rc = check_launch("backward_pair_kernel")) return rc;
+  if (splits > 1) return launch_splitk_reduce(gw, splits, true, T::id, stream);
+  return SD_OK;
+}
+
+int launch_backward_pair(const GemmArgs& gx, const GemmArgs& gw, int dtype, hipStream_t stream) {
+  // the SDD product's conditions (try_sdd)
+  if (!gx.row_ptr || gx.bs != BS || gx.kept_only) return SD_ERR_UNSUPPORTED;
+  const int64_t x_Cb = (gx.N + BS - 1) / BS, x_Mb = (gx.M + BS - 1) / BS;
+  const bool x_ok = gx.a.sc == 1 && gx.b.sr == 1 && gx.b.sc != 1 && gx.c_sc == 1 && gx.M > 0 && gx.N > 0 &&
+                    gx.N % 8 == 0 && gx.K > 0 && gx.K % 8 == 0 && aligned16(gx.a.ptr) && aligned16(gx.b.ptr) &&
+                    aligned16(gx.c) && gx.a.sr % 8 == 0 && gx.b.sc % 8 == 0 && gx.c_sr % 8 == 0 &&
+                    gx.a.sr < (1 << 22) && gx.b.sc < (1 << 22) && x_Cb <= G_MAX_CB;
+  // the weight gradient's (launch_fast), in the one form the autograd step produces
+  if (!gw.row_ptr || gw.bs != BS || gw.act) return SD_ERR_UNSUPPORTED;
+  const bool w_ok = gw.a.sr == 1 && gw.b.sr == 1 && gw.a.sc != 1 && gw.b.sc != 1 && gw.c_sc != 1 && gw.c_sr == 1 &&
+                    gw.M > 0 && gw.M % 8 == 0 && gw.N > 0 && gw.N % 8 == 0 && gw.K > 0 && (gw.K + BS - 1) / BS < 65536 &&
+                    aligned16(gw.a.ptr) && aligned16(gw.b.ptr) && aligned16(gw.c) && gw.a.sc % 8 == 0 &&
+                    gw.b.sc % 8 == 0 && gw.c_sc % 8 == 0 && gw.a.sc < (1 << 22) && gw.b.sc < (1 << 22);
+  if (!x_ok || !w_ok) return SD_ERR_UNSUPPORTED;
+  const DsdPlan plan = plan_dsd(gw.M, gw.N, gw.K);
+  const int splits = usable_splits(gw, plan, kDsd);
+  if (splits < 1) return SD_ERR_UNSUPPORTED;
+  // the SDD shape as launch_sdd_group picks it; both products must want the same size
+  const float keep = (gx.keep_hint >= 0.f && gx.keep_hint <= 1.f) ? gx.keep_hint : 1.f;
+  const int64_t cols = keep <= 0.3f ? SddBig::GW : SddBig::MINCOLS;
+  const int64_t big = ((x_Mb + 3) / 4) * ((x_Cb + cols - 1) / cols);
+  const int policy = tile_policy.load(std::memory_order_relaxed);
+  const bool x_mid = policy == kTileMid || (policy == kTileAuto && big <= 128);
+  if (x_mid != plan.mid) return SD_ERR_UNSUPPORTED;
+  // Worth it only while neither product fills the chip by itself: side by side, two large products get in each
+  // other's way in the L2 (8192^3 at p = 0.5: 1.33 ms in one launch against 1.28 in two; 1024^3: 27 us against 46).
+  const int64_t x_wgs = x_mid ? ((x_Mb + 1) / 2) * ((x_Cb + 3) / 4) : big;
+  const int64_t w_wgs = (plan.mid ? dsd_tiles<DsdMid>(gw.M, gw.N) : dsd_tiles<DsdBig>(gw.M, gw.N)) * splits;
+  if (x_wgs > pair_limit() || w_wgs > pair_limit()) return SD_ERR_UNSUPPORTED;
+  if ((x_Mb + 1) / 2 * ((x_Cb + 3) / 4) + dsd_tiles<DsdMid>(gw.M, gw.N) > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
+  // either product ragged (or on a block-size-32 mask): the instances that handle edges, for both
+  const bool edge = gx.N % BS != 0 || gx.K % BS != 0 || gx.quads || gw.M % BS != 0 || gw.N % BS != 0 ||
+                    gw.K % BS != 0 || gw.quads;
+  if (dtype == SD_BF16) {
+    if (x_mid) return edge ? launch_pair_t<BF16, true, SddMid, DsdMid>(gx, gw, splits, stream)
+                           : launch_pair_t<BF16, false, SddMid, DsdMid>(gx, gw, splits, stream);
+    return edge ? launch_pair_t<BF16, true, SddBig, DsdBig>(gx, gw, splits, stream)
+                : launch_pair_t<BF16, false, SddBig, DsdBig>(gx, gw, splits, stream);
+  }
+  if (x_mid) return edge ? launch_pair_t<F16, true, SddMid, DsdMid>(gx, gw, splits, stream)
+                         : launch_pair_t<F16, false, SddMid, DsdMid>(gx, gw, splits, stream);
+  return edge ? launch_pair_t<F16, true, SddBig, DsdBig>(gx, gw, splits, stream)
+              : launch_pair_t<F16, false, SddBig, DsdBig>(gx, gw, splits, stream);
 }
 
 int set_tile_policy(int policy) {

@@ -70,27 +70,21 @@ class BlockwiseDropoutMLPHIP(torch.autograd.Function):
         grads_w = [None] * n
         for i in reversed(range(n)):
             w, lists, _ = layers[i]
-            scale = 1.0 / (1.0 - ctx.ps[i])
             need_w = ctx.needs_input_grad[6 + i]
             need_in = i > 0 or ctx.needs_input_grad[0]
-            if w.shape[0] % 8:  # a narrow head: zero-padded copies keep both products on the specialised kernels
-                n_pad = (w.shape[0] + 7) // 8 * 8
-                gp = g.new_zeros((g.shape[0], n_pad))
-                gp[:, : w.shape[0]] = g
-                wp = w.new_zeros((n_pad, w.shape[1]))
-                wp[: w.shape[0]] = w
-                g, w = gp, wp
-            if need_w:
-                dw = ext.gemm_dsd_lists(hs[i].t(), g.t(), lists.transposed(), ctx.kbs[i], scale, transposed_out=True).t()
-                grads_w[i] = dw[: layers[i][0].shape[0]]
-            if not need_in:
-                break
-            if i > 0:
+            at = None
+            if i > 0 and need_in and act is not None:
                 prev_pre = layers[i - 1][2]
                 at = prev_pre if prev_pre.numel() else hs[i]  # GELU: pre-activation; ReLU: the activated input
-                g = ext.gemm_sdd_lists_actgrad(g, w.t(), lists, ctx.kbs[i], scale, act, at, keep_hint=1.0 / scale)
-            else:
-                g = ext.gemm_sdd_lists(g, w.t(), lists, ctx.kbs[i], scale, keep_hint=1.0 / scale)
+            # both gradients of the layer in one library call (one launch for small layers), the activation's
+            # derivative riding on the dX store
+            dx, dw = ext.dropout_matmul_backward(g, w, hs[i], lists, ctx.kbs[i], ctx.ps[i], need_dx=need_in,
+                                                 need_dw=need_w, activation=act if at is not None else None, act_at=at)
+            if need_w:
+                grads_w[i] = dw
+            if not need_in:
+                break
+            g = dx
         grad_in = g if ctx.needs_input_grad[0] else None
         return (grad_in, None, None, None, None, None, *grads_w)
 

@@ -63,6 +63,9 @@ SIGNATURES = {
     "sd_dropout_matmul_backward": (c_int, [*_mat, *_mat, *_mat, *_mat, *_mat, c_void_p, c_void_p, c_void_p, c_void_p,
                                            c_int64, c_int64, c_int64, c_int64, c_float, c_int, c_void_p, c_int64,
                                            c_void_p]),
+    "sd_dropout_matmul_backward_act": (c_int, [*_mat, *_mat, *_mat, *_mat, *_mat, c_void_p, c_void_p, c_void_p,
+                                               c_void_p, c_int64, c_int64, c_int64, c_int64, c_float, c_int,
+                                               c_int, *_mat, c_void_p, c_int64, c_void_p]),
     "sd_conv2d_dsd_lists": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64,
                                     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,

@@ -570,9 +570,12 @@ class GEMM:
         return y, mask, KeptLists(row_ptr, col_idx, col_ptr, row_idx, (out_mb, out_kb)), (32 if bs == 32 else g)
 
     def dropout_matmul_backward(self, dy: torch.Tensor, w: torch.Tensor, x: torch.Tensor, lists: KeptLists,
-                                block_size, p: float, need_dx: bool = True, need_dw: bool = True):
+                                block_size, p: float, need_dx: bool = True, need_dw: bool = True,
+                                activation: str | None = None, act_at: torch.Tensor | None = None):
         """``dX = (dy @ w) ⊙ keep / (1-p)`` and ``dW = dy.T @ (keep ⊙ x) / (1-p)`` (a contiguous [N, K] tensor) in
-        one library call; either may be skipped -> (dx or None, dw or None)."""
+        one library call - and, for small layers, one launch; either may be skipped -> (dx or None, dw or None).
+        With ``activation`` dX is also multiplied by the activation's derivative at ``act_at`` ([M, K]: the
+        pre-activation, or for ReLU the activated tensor), as :meth:`gemm_sdd_lists_actgrad` does."""
         self._check_pair(x, w)
         _check_operand("dy", dy)
         bs = _block_size(block_size)
@@ -593,7 +596,7 @@ class GEMM:
             w_pad = w.new_zeros((n_pad, K))
             if need_dx:
                 w_pad[:N] = w
-            dx, dw = self.dropout_matmul_backward(dy_pad, w_pad, x, lists, bs, p, need_dx, need_dw)
+            dx, dw = self.dropout_matmul_backward(dy_pad, w_pad, x, lists, bs, p, need_dx, need_dw, activation, act_at)
             return dx, (dw[:N] if dw is not None else None)
         dx = torch.empty((M, K), dtype=x.dtype, device=x.device) if need_dx else None
         dw = torch.empty((N, K), dtype=x.dtype, device=x.device) if need_dw else None
@@ -604,12 +607,17 @@ class GEMM:
         ws_ptr, ws_bytes, ws = None, 0, None
         if need_dw:  # the weight gradient of a tall activation matrix splits its reduction over workgroups
             ws, ws_ptr, ws_bytes = self._splitk_scratch(x.t(), dy.t(), g, 1)
+        act = _activation(activation) if need_dx else 0
+        if act:
+            if act_at is None or tuple(act_at.shape) != (M, K) or act_at.dtype != x.dtype or act_at.device != x.device:
+                raise ValueError(f"act_at must be a [{M}, {K}] {x.dtype} tensor on {x.device}")
+            _check_operand("act_at", act_at)
         with _guard(x.device):
-            self._call(self.lib.sd_dropout_matmul_backward, *_mat(dy), *_mat(w), *_mat(x),
+            self._call(self.lib.sd_dropout_matmul_backward_act, *_mat(dy), *_mat(w), *_mat(x),
                        *(_mat(dx) if need_dx else (None, 0, 0)), *(_mat(dw) if need_dw else (None, 0, 0)),
                        lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(), lists.col_ptr.data_ptr(),
-                       lists.row_idx.data_ptr(), M, N, K, bs, float(p), _DTYPES[x.dtype], ws_ptr, ws_bytes,
-                       self._stream(x))
+                       lists.row_idx.data_ptr(), M, N, K, bs, float(p), _DTYPES[x.dtype],
+                       act, *(_mat(act_at) if act else (None, 0, 0)), ws_ptr, ws_bytes, self._stream(x))
         return dx, dw
 
     # ------------------------------------------------------------------ conv feed

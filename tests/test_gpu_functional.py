@@ -279,6 +279,38 @@ def test_fused_forward_and_backward_calls_match_the_separate_ones(bs):
     assert np.array_equal(m5.cpu().numpy(), O.random_mask(O.mask_shape(M, K, bs), p, 5, offset=1))
 
 
+@pytest.mark.parametrize("M,K,N,bs,dtype,paired", [
+    (1024, 1024, 1024, 64, torch.float16, True),      # aligned, both products on a fraction of the chip
+    (4096, 784, 1024, 64, torch.float16, True),       # ragged K, weight gradient with a split reduction
+    (2048, 512, 384, 128, torch.bfloat16, True),      # bf16, block size listed at 64
+    (1000, 520, 264, 32, torch.float16, True),        # ragged everywhere, block size 32 (quadrant keep bits)
+    (16384, 1536, 384, 64, torch.float16, False),     # dX wants the big workgroup shape, dW the small one: two launches
+])
+def test_both_gradients_in_one_launch_match_the_two_launches(M, K, N, bs, dtype, paired):
+    """sd_dropout_matmul_backward puts dX and dW of a small layer into a single launch (backward_pair_kernel): the
+    result must be what the two products give by themselves, bit for bit, and what the oracle gives, per tile."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(23)
+    p = 0.5
+    x = torch.randn(M, K, generator=gen).to(dtype).cuda()
+    w = (torch.randn(N, K, generator=gen) * K ** -0.5).to(dtype).cuda()
+    dy = torch.randn(M, N, generator=gen).to(dtype).cuda()
+    mask = cpu_mask(O.mask_shape(M, K, bs), p, gen)
+    g = 64 if bs % 64 == 0 else bs
+    lists = ext.build_lists(mask.cuda(), split=0 if bs == 32 else bs // 64) if bs != 64 else ext.build_lists(mask.cuda())
+    s = 1 / (1 - p)
+    dx, dw = ext.dropout_matmul_backward(dy, w, x, lists, g, p)
+    detail = ext.last_kernel_detail()
+    assert detail.startswith("pair:") == paired, detail
+    assert torch.equal(dx, ext.gemm_sdd(dy, w.t(), mask.cuda(), bs, s))
+    assert torch.equal(dw, ext.gemm_dsd(x.t(), dy.t(), mask.t().cuda(), bs, s, transposed_out=True).t())
+    if M * K * N <= 1 << 31:
+        assert max_tile_rel_fro(dx, O.sdd_dx(to_np(dy), to_np(w), mask.numpy(), bs, p, np.float32)) <= REL_FRO_TOL
+        assert max_tile_rel_fro(dw, O.dsd_dw(to_np(dy), to_np(x), mask.numpy(), bs, p, np.float32)) <= REL_FRO_TOL
+
+
 @pytest.mark.parametrize("act", ["relu", "gelu"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_fused_activation_products_against_the_oracle(act, dtype):
