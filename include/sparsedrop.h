@@ -279,6 +279,16 @@ int sd_gemm_dsd_lists_act(const void* A, int64_t a_stride_r, int64_t a_stride_c,
                           int act, void* pre_out, int64_t pre_stride_r, int64_t pre_stride_c,
                           void* workspace, int64_t workspace_bytes, void* stream);
 
+/* The dense product with the same fused store, C = act(A . B^T) (and the pre-activation to pre_out when given): a
+ * layer without dropout inside a stack that fuses its activations (the reference's first layer, eval/mlp/model.py:
+ * 31-33, has p = 0).  B must have a contiguous reduction index when act != SD_ACT_NONE. */
+int sd_gemm_act(const void* A, int64_t a_stride_r, int64_t a_stride_c,
+                const void* B, int64_t b_stride_r, int64_t b_stride_c,
+                void* C, int64_t c_stride_r, int64_t c_stride_c,
+                int64_t M, int64_t N, int64_t K, int dtype, int act,
+                void* pre_out, int64_t pre_stride_r, int64_t pre_stride_c,
+                void* workspace, int64_t workspace_bytes, void* stream);
+
 int sd_gemm_sdd_lists_actgrad(const void* A, int64_t a_stride_r, int64_t a_stride_c,
                               const void* B, int64_t b_stride_r, int64_t b_stride_c,
                               void* C, int64_t c_stride_r, int64_t c_stride_c,

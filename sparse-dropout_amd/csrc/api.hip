@@ -346,6 +346,24 @@ static int check_act(int act, const void* aux, int64_t xsr, int64_t xsc, int64_t
   return SD_OK;
 }
 
+int sd_gemm_act(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc, void* C,
+                int64_t csr, int64_t csc, int64_t M, int64_t N, int64_t K, int dtype, int act, void* pre_out,
+                int64_t pre_stride_r, int64_t pre_stride_c, void* workspace, int64_t workspace_bytes, void* stream) {
+  if (int rc = check_common(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, dtype)) return rc;
+  if (int rc = check_act(act, pre_out, pre_stride_r, pre_stride_c, M, N, false)) return rc;
+  // row-major A with a reduction-strided B is the operand layout of the input gradient: the kernel that takes it
+  // multiplies by an activation's derivative in its store, it does not apply one
+  SD_REQUIRE(act == SD_ACT_NONE || !(asc == 1 && bsr == 1 && bsc != 1 && csc == 1),
+             "gemm_act: an activation needs B with a contiguous reduction index (the forward layout)");
+  GemmArgs g = make_args(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, 0, 1.0f, nullptr, nullptr,
+                         workspace, workspace_bytes);
+  g.act = act;
+  g.aux = act != SD_ACT_NONE ? static_cast<uint16_t*>(pre_out) : nullptr;
+  g.aux_sr = pre_stride_r;
+  g.aux_sc = pre_stride_c;
+  return run(g, kDense, dtype, (hipStream_t)stream);
+}
+
 int sd_gemm_dsd_lists_act(const void* A, int64_t asr, int64_t asc, const void* B, int64_t bsr, int64_t bsc,
                           void* C, int64_t csr, int64_t csc, const int32_t* row_ptr, const int32_t* col_idx,
                           int64_t M, int64_t N, int64_t K, int64_t bs, float scale, int dtype, int act, void* pre_out,

@@ -32,10 +32,23 @@ class BlockwiseDropoutMLPHIP(torch.autograd.Function):
         saved, shapes, kbs = [input], [], []
         for i, w in enumerate(weights):
             p = ps[i]
+            last = i + 1 == n
+            if i == 0 and p == 0.0 and masks is None and not ctx.needs_input_grad[0]:
+                # a first layer without dropout whose input needs no gradient (the reference's models start with one,
+                # eval/mlp/model.py:31-33): the dense product with the same fused store, no mask and no lists
+                out, pre = ext.gemm_act(h, w, None if last else activation,
+                                        want_pre=(not last and activation == "gelu"))
+                empty = out.new_empty(0)
+                saved += [w, empty, empty, empty, empty, empty, pre if pre is not None else empty]
+                if not last:
+                    saved.append(out)
+                shapes.append(None)
+                kbs.append(0)
+                h = out
+                continue
             mask, lists, kernel_bs = ext.kept_lists(h.shape[0], h.shape[1], block_size,
                                                     None if masks is None else masks[i], p,
                                                     None if seed is None else seed + i, h.device)
-            last = i + 1 == n
             out, pre = ext.gemm_dsd_lists_act(h, w, lists, kernel_bs, 1.0 / (1.0 - p), None if last else activation,
                                               want_pre=(not last and activation == "gelu"))
             # per layer: weight, mask, the four list arrays, what the activation's derivative is evaluated at
@@ -61,7 +74,7 @@ class BlockwiseDropoutMLPHIP(torch.autograd.Function):
         for i in range(n):
             w, _, rp, ci, cp, ri, pre = t[pos:pos + 7]
             pos += 7
-            layers.append((w, KeptLists(rp, ci, cp, ri, ctx.shapes[i]), pre))
+            layers.append((w, KeptLists(rp, ci, cp, ri, ctx.shapes[i]) if ctx.shapes[i] is not None else None, pre))
             if i + 1 < n:
                 hs.append(t[pos])
                 pos += 1
@@ -72,6 +85,13 @@ class BlockwiseDropoutMLPHIP(torch.autograd.Function):
             w, lists, _ = layers[i]
             need_w = ctx.needs_input_grad[6 + i]
             need_in = i > 0 or ctx.needs_input_grad[0]
+            if lists is None:  # the dense first layer: only its weight gradient is wanted, dW = g^T . h
+                if need_w:
+                    if w.shape[0] % 8:
+                        grads_w[i] = g.t().mm(hs[i])
+                    else:
+                        grads_w[i] = ext.gemm(g.t(), hs[i].t())
+                break
             at = None
             if i > 0 and need_in and act is not None:
                 prev_pre = layers[i - 1][2]

@@ -505,6 +505,24 @@ class GEMM:
                        *(_mat(pre) if pre is not None else (None, 0, 0)), ws_ptr, ws_bytes, self._stream(A))
         return C, (pre if code else (C if want_pre else None))
 
+    def gemm_act(self, A, B, act, want_pre: bool = False):
+        """``act(A @ B.T)``, the dense product with the activation in the kernel's store -> (activated,
+        pre-activation or None): a layer without dropout inside a fused stack."""
+        self._check_pair(A, B)
+        code = _activation(act)
+        M, N, K = A.shape[0], B.shape[0], A.shape[1]
+        C = torch.empty((M, N), dtype=A.dtype, device=A.device)
+        pre = torch.empty((M, N), dtype=A.dtype, device=A.device) if (want_pre and code) else None
+        if M == 0 or N == 0:
+            return C, pre
+        if K == 0:
+            return C.zero_(), (pre.zero_() if pre is not None else None)
+        ws, ws_ptr, ws_bytes = self._splitk_scratch(A, B, 0, 0)
+        with _guard(A.device):
+            self._call(self.lib.sd_gemm_act, *_mat(A), *_mat(B), *_mat(C), M, N, K, _DTYPES[A.dtype], code,
+                       *(_mat(pre) if pre is not None else (None, 0, 0)), ws_ptr, ws_bytes, self._stream(A))
+        return C, (pre if code else (C if want_pre else None))
+
     def gemm_sdd_lists_actgrad(self, A, B, lists: KeptLists, block_size, scale, act, act_at: torch.Tensor,
                                keep_hint: float | None = None):
         """``scale * (A @ B.T) ⊙ keep ⊙ act'(act_at)``: the input gradient of a layer whose input was

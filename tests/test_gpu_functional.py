@@ -390,6 +390,40 @@ def test_fused_mlp_against_the_oracle_and_the_unfused_layers(act, dims, rows):
         assert rel_fro(a.grad, b.grad.float()) <= 4e-3
 
 
+@pytest.mark.parametrize("act", ["relu", "gelu"])
+def test_dense_product_with_fused_activation_and_the_stack_that_starts_with_one(act):
+    """sd_gemm_act against act(A . B^T) from the oracle, and the fused MLP whose first layer has p = 0 (the dense
+    fused product, no mask, no lists) against the same stack run with explicit masks (the list path the oracle
+    test above pins)."""
+    import flash_dropout.functional as F
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(29)
+    rows, dims = 520, [200, 320, 264, 72]
+    x = torch.randn(rows, dims[0], generator=gen).half()
+    ws = [(torch.randn(dims[i + 1], dims[i], generator=gen) * dims[i] ** -0.5).half() for i in range(3)]
+    y, pre = ext.gemm_act(x.cuda(), ws[0].cuda(), act, want_pre=True)
+    ref_pre = to_np(x).astype(np.float64) @ to_np(ws[0]).astype(np.float64).T
+    assert max_tile_rel_fro(pre, ref_pre.astype(np.float32)) <= REL_FRO_TOL
+    assert max_tile_rel_fro(y, O.act_apply(ref_pre, act).astype(np.float32)) <= REL_FRO_TOL
+    assert ext.last_kernel() == "specialised"
+    ps, seed = [0.0, 0.5, 0.5], 31
+    masks = [torch.zeros(O.mask_shape(rows, dims[0], 64), dtype=torch.bool)] + [
+        torch.from_numpy(O.random_mask(O.mask_shape(rows, dims[i], 64), 0.5, seed + i)) for i in (1, 2)]
+    dy = torch.randn(rows, dims[-1], generator=gen).half().cuda()
+    grads = []
+    for kw in ({"seed": seed}, {"masks": [m.cuda() for m in masks]}):
+        wg = [w.cuda().requires_grad_() for w in ws]
+        out = F.hip_blockwise_dropout_mlp(x.cuda(), wg, 64, ps, act, **kw)
+        out.backward(dy)
+        grads.append((out.detach(), [w.grad for w in wg]))
+    (o1, g1), (o2, g2) = grads
+    assert rel_fro(o1, o2.float()) <= 1e-3
+    for a, b in zip(g1, g2):
+        assert a.shape == b.shape and rel_fro(a, b.float()) <= 1e-3
+
+
 @pytest.mark.parametrize("name", ["mlp", "mlp-784", "vit-ffn"])
 def test_model_harness_runs_every_variant(name):
     """benchmark/model.py (the reference's benchmark/model.py:119-229 protocol): every variant of every model
