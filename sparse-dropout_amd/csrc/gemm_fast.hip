@@ -90,7 +90,7 @@ struct DsdShape {
   static constexpr int SMEM_BYTES = SMEM_SCRATCH + 4 * MAX_STEPS + 16;
   static_assert(BL >= 1 && AL >= 1 && BL * NW * 1024 == B_TILE && AL * NW * 1024 == TILE, "loads must divide evenly");
 };
-using DsdBig = DsdShape<2, 4, 2>;
+using DsdBig = DsdShape<2, 4, 2>;  // (8 waves of 1 row block x 128 columns, DsdShape<4, 2, 4, 1>, measured 2-4 % slower)
 using DsdMid = DsdShape<2, 4, 1, 1>;
 // 256 rows x 128 columns, 8 waves: the shape of the implicit-GEMM convolution, whose input patch has to
 // fit in LDS next to the stages
@@ -839,7 +839,8 @@ __device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int til
   // along C's contiguous index, and writes it out in 16-byte pieces.  The last step's barrier has passed, so
   // nobody reads the stages or the step table any more.
   constexpr int WN = 32 * NT;
-  constexpr int S_ROWS = CM ? WN : BS, S_COLS = CM ? BS : WN, S_PITCH = S_COLS + 4;
+  constexpr int WC = WN > 64 ? 64 : WN;  // columns staged at a time
+  constexpr int S_ROWS = CM ? WC : BS, S_COLS = CM ? BS : WC, S_PITCH = S_COLS + 4;
   static_assert(S::NW * S_ROWS * S_PITCH * 4 <= S::SMEM_BYTES, "the staging tiles must fit in the kernel's LDS");
   float* stg = reinterpret_cast<float*>(smem) + wave * (S_ROWS * S_PITCH);
 #pragma unroll
@@ -847,20 +848,24 @@ __device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int til
     const int rb = rb0 + RW * rh + rr;
     if (rb >= Mb) continue;
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int h = 0; h < WN / WC; ++h) {
 #pragma unroll
-      for (int nt = 0; nt < NT16; ++nt) {
-        if (CM) {  // staged as [n][m]: the lane's four registers are consecutive along m
-          *reinterpret_cast<f32x4*>(stg + (nt * 16 + lane % 16) * S_PITCH + mt * 16 + 4 * (lane / 16)) = acc[rr][mt][nt];
-        } else {  // staged as [m][n]: four rows, one column (16 lanes x 4 row groups hit 64 distinct banks)
+      for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
-          for (int v = 0; v < 4; ++v)
-            stg[(mt * 16 + 4 * (lane / 16) + v) * S_PITCH + nt * 16 + lane % 16] = acc[rr][mt][nt][v];
+        for (int nc = 0; nc < WC / 16; ++nc) {
+          const int nt = h * (WC / 16) + nc;
+          if (CM) {  // staged as [n][m]: the lane's four registers are consecutive along m
+            *reinterpret_cast<f32x4*>(stg + (nc * 16 + lane % 16) * S_PITCH + mt * 16 + 4 * (lane / 16)) = acc[rr][mt][nt];
+          } else {  // staged as [m][n]: four rows, one column (16 lanes x 4 row groups hit 64 distinct banks)
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+              stg[(mt * 16 + 4 * (lane / 16) + v) * S_PITCH + nc * 16 + lane % 16] = acc[rr][mt][nt][v];
+          }
         }
-      }
-    const int64_t m_first = (int64_t)rb * BS, n_first = n0 + ns * WN;
-    store_staged_tile<T, false, S_ROWS, S_COLS>(g, stg, lane, !CM, CM ? n_first : m_first, CM ? m_first : n_first,
-                                                part);
+      const int64_t m_first = (int64_t)rb * BS, n_first = n0 + ns * WN + h * WC;
+      store_staged_tile<T, false, S_ROWS, S_COLS>(g, stg, lane, !CM, CM ? n_first : m_first, CM ? m_first : n_first,
+                                                  part);
+    }
   }
 }
 
