@@ -365,6 +365,23 @@ int sd_dropout_matmul_backward_act(const void* dY, int64_t dy_stride_r, int64_t 
                                    int act, const void* act_at, int64_t at_stride_r, int64_t at_stride_c,
                                    void* workspace, int64_t workspace_bytes, void* stream);
 
+/* sd_dropout_matmul_forward with an activation in the product's store (sd_gemm_dsd_lists_act's epilogue):
+ * Y = act((keep . X) / (1 - p) . W^T), the value before the activation to pre_out when that is given; act = SD_ACT_NONE
+ * is the plain call.  No counterpart in the reference, whose layers run the activation as a kernel of its own.
+ * Where the product is small (at most 512 workgroups) and its mask has at most 2^18 entries on the 64 grid, the mask
+ * draw, both lists and the product run as ONE launch: the product's workgroups evaluate the keep bits of their own
+ * row blocks from the mask source, other workgroups of the same grid write the lists the backward reads.
+ * SPARSEDROP_SEPARATE_FORWARD=1 in the environment keeps the list build a launch of its own (for comparing). */
+int sd_dropout_matmul_forward_act(const void* X, int64_t x_stride_r, int64_t x_stride_c,
+                                  const void* W, int64_t w_stride_r, int64_t w_stride_c,
+                                  void* Y, int64_t y_stride_r, int64_t y_stride_c,
+                                  const uint8_t* mask, int64_t mask_stride_r, int64_t mask_stride_c,
+                                  uint64_t* rng_state, uint64_t seed, uint64_t offset, float p, uint8_t* mask_out,
+                                  int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx,
+                                  int64_t M, int64_t N, int64_t K, int64_t block_size, int dtype,
+                                  int act, void* pre_out, int64_t pre_stride_r, int64_t pre_stride_c,
+                                  void* workspace, int64_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * (e) im2col gather feeding the same GEMMs for conv.
  *

@@ -488,13 +488,63 @@ int sd_dropout_matmul_forward(const void* X, int64_t xsr, int64_t xsc, const voi
                               int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx, int64_t M,
                               int64_t N, int64_t K, int64_t bs, int dtype, void* workspace, int64_t workspace_bytes,
                               void* stream) {
+  return sd_dropout_matmul_forward_act(X, xsr, xsc, W, wsr, wsc, Y, ysr, ysc, mask, msr, msc, rng_state, seed, offset, p,
+                                       mask_out, row_ptr, col_idx, col_ptr, row_idx, M, N, K, bs, dtype, SD_ACT_NONE,
+                                       nullptr, 0, 0, workspace, workspace_bytes, stream);
+}
+
+// SPARSEDROP_SEPARATE_FORWARD=1: the lists and the product of the fused forward always in two launches (for measuring)
+static bool separate_forward_forced() {
+  static const bool forced = [] {
+    const char* e = std::getenv("SPARSEDROP_SEPARATE_FORWARD");
+    return e && e[0] == '1';
+  }();
+  return forced;
+}
+
+int sd_dropout_matmul_forward_act(const void* X, int64_t xsr, int64_t xsc, const void* W, int64_t wsr, int64_t wsc,
+                                  void* Y, int64_t ysr, int64_t ysc, const uint8_t* mask, int64_t msr, int64_t msc,
+                                  uint64_t* rng_state, uint64_t seed, uint64_t offset, float p, uint8_t* mask_out,
+                                  int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx, int64_t M,
+                                  int64_t N, int64_t K, int64_t bs, int dtype, int act, void* pre_out,
+                                  int64_t pre_stride_r, int64_t pre_stride_c, void* workspace, int64_t workspace_bytes,
+                                  void* stream) {
   if (int rc = check_common(X, xsr, xsc, W, wsr, wsc, Y, ysr, ysc, M, N, K, dtype)) return rc;
   SD_REQUIRE(p >= 0.f && p < 1.f, "dropout_matmul_forward: p must be in [0, 1) (got %g)", (double)p);
   if (int rc = check_sparse(bs, 1.f)) return rc;
   SD_REQUIRE(M > 0 && K > 0, "dropout_matmul_forward: empty operand");
   SD_REQUIRE(row_ptr && col_idx, "dropout_matmul_forward: the CSR list arrays are required");
+  if (int rc = check_act(act, pre_out, pre_stride_r, pre_stride_c, M, N, false)) return rc;
   const int64_t g = list_granule(bs), split = bs / g;  // 0 for block size 32: merged two by two
   const int64_t mb = ceil_div(M, bs), kb = ceil_div(K, bs), out_mb = ceil_div(M, g), out_kb = ceil_div(K, g);
+  const float scale = 1.f / (1.f - p);
+  // what the list calls below would check, up front: the single launch takes the same arguments
+  if (int rc = check_list_grid(mb, kb, split, out_mb, out_kb, row_ptr, col_idx, col_ptr, row_idx)) return rc;
+  if (mask) {
+    SD_REQUIRE(msr >= 1 && msc >= 1 && (msr == 1 || msc == 1), "build_lists: mask must be row or column major");
+  } else {
+    SD_REQUIRE(mask_out != nullptr, "random_lists: null mask_out");
+    SD_REQUIRE(rng_state == nullptr || reinterpret_cast<uintptr_t>(rng_state) % 8 == 0,
+               "random_lists: state must be an aligned device pointer");
+  }
+  auto with_act = [&](GemmArgs a) {
+    a.act = act;
+    a.aux = act != SD_ACT_NONE ? static_cast<uint16_t*>(pre_out) : nullptr;
+    a.aux_sr = pre_stride_r;
+    a.aux_sc = pre_stride_c;
+    return a;
+  };
+  if (N > 0 && !generic_forced() && !separate_forward_forced()) {
+    // lists and product in one launch where the pair qualifies (small products, where a launch is a large part)
+    const GemmArgs a = with_act(make_args(X, xsr, xsc, W, wsr, wsc, Y, ysr, ysc, M, N, K, bs == 32 ? 32 : g, scale,
+                                          row_ptr, col_idx, workspace, workspace_bytes));
+    const int rc = forward_with_lists(a, mask, msr, msc, seed, offset, rng_state, p, mb, kb, mask_out, split, out_mb,
+                                      out_kb, row_ptr, col_idx, col_ptr, row_idx, dtype, (hipStream_t)stream);
+    if (rc != SD_ERR_UNSUPPORTED) {
+      last_kernel = "specialised";
+      return rc;
+    }
+  }
   if (mask) {
     if (int rc = sd_build_lists_split(mask, mb, kb, msr, msc, split, out_mb, out_kb, row_ptr, col_idx, col_ptr, row_idx,
                                       stream))
@@ -509,8 +559,9 @@ int sd_dropout_matmul_forward(const void* X, int64_t xsr, int64_t xsc, const voi
       return rc;
   }
   if (N == 0) return SD_OK;
-  return sd_gemm_dsd_lists(X, xsr, xsc, W, wsr, wsc, Y, ysr, ysc, row_ptr, col_idx, M, N, K, bs == 32 ? 32 : g,
-                           1.f / (1.f - p), dtype, workspace, workspace_bytes, stream);
+  return sd_gemm_dsd_lists_act(X, xsr, xsc, W, wsr, wsc, Y, ysr, ysc, row_ptr, col_idx, M, N, K, bs == 32 ? 32 : g,
+                               scale, dtype, act, pre_out, pre_stride_r, pre_stride_c, workspace, workspace_bytes,
+                               stream);
 }
 
 int sd_dropout_matmul_backward(const void* dY, int64_t gsr, int64_t gsc, const void* W, int64_t wsr, int64_t wsc,

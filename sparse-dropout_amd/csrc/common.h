@@ -288,6 +288,17 @@ int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream);
 // dX (SDD) and dW (DSD, reduction-strided operands, column-major C) of one layer in a single launch;
 // SD_ERR_UNSUPPORTED with nothing launched when the pair does not qualify
 int launch_backward_pair(const GemmArgs& gx, const GemmArgs& gw, int dtype, hipStream_t stream);
+// The forward product on its specialised kernel and the kept lists of its mask (stored: mask / msr / msc; drawn when
+// mask is null: seed / offset or the device-resident state, p, stored to mask_out) in a single launch; arguments as
+// for build_lists / random_lists.  SD_ERR_UNSUPPORTED with nothing launched when the pair does not qualify.
+int forward_with_lists(const GemmArgs& g, const uint8_t* mask, int64_t msr, int64_t msc, uint64_t seed, uint64_t offset,
+                       uint64_t* state, float p, int64_t stored_mb, int64_t stored_kb, uint8_t* mask_out, int64_t split,
+                       int64_t mb, int64_t kb, int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx,
+                       int dtype, hipStream_t stream);
+struct MaskSrc;
+int launch_forward_with_lists(const GemmArgs& g, const MaskSrc& src, int64_t mb, int64_t kb, int32_t* row_ptr,
+                              int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx, uint8_t* mask_out,
+                              int64_t mask_rows, int dtype, hipStream_t stream);
 // forward of the block-dropout convolution without the patch matrix: g.a is unused, g.b the [K_out, C*R*S]
 // weight matrix, g.c the [N*P*Q, K_out] output, the lists over the patch matrix's block grid.  Returns
 // SD_ERR_UNSUPPORTED (without an error message) for geometries it does not take.

@@ -48,6 +48,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include "mask_source.h"
 #include "tile_map.h"
 
 namespace sd {
@@ -162,9 +163,12 @@ __device__ inline int swz_w(int row) { return ((row & 3) << 2) ^ (((row >> 3) & 
 // of input channels fits); the reduction-strided instance (the weight gradient) always works that way.
 // bid: the workgroup's index in the launch order of this product; the reduction is split nsplit ways and this
 // workgroup takes part `split` (the kernels below pass their block indices; the fused backward launch its own)
+// ms: where the mask comes from when the kept lists do not exist yet (the forward launch that also builds them);
+// the keep bits of the workgroup's row blocks are then evaluated from it directly, g.row_ptr is not read
 template <typename T, bool TRANS, bool CM, bool RAGGED, typename S, int IMPLICIT = 0>
 __device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int tiles_n, int Mb, int Kb_all,
-                                         const ImplicitConv& cg, const int bid, const int nsplit, const int split) {
+                                         const ImplicitConv& cg, const int bid, const int nsplit, const int split,
+                                         const MaskSrc* ms = nullptr) {
   static_assert(!IMPLICIT || (S::R == 4 && S::THREADS == 512), "the gather assumes 512 threads x 4 row blocks");
   static_assert(S::R <= 4, "a step's keep bits are four per row block in 16 bits");
   constexpr int R = S::R, BN = S::BN, THREADS = S::THREADS, NT = S::NT, STAGE = S::STAGE, A_OFF = S::A_OFF;
@@ -194,7 +198,14 @@ __device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int til
   // ---- union of the kept lists of the 4 row blocks: (K block, 4-bit keep flags) per step -------
   for (int i = tid; i < Kb; i += THREADS) scratch[i] = 0;
   __syncthreads();
-  if (g.row_ptr) {
+  if (ms) {
+    const int rows = (rb0 + R <= Mb) ? R : Mb - rb0;
+    for (int i = tid; i < rows * Kb; i += THREADS) {
+      const int r = i / Kb, k = i - r * Kb;
+      const uint32_t q = ms->merge == 2 ? ms->kept_quads(rb0 + r, kb_lo + k) : (ms->dropped(rb0 + r, kb_lo + k) ? 0u : 0xfu);
+      if (q) atomicOr(&scratch[k], q << (4 * r));
+    }
+  } else if (g.row_ptr) {
     for (int r = 0; r < R; ++r) {
       if (rb0 + r >= Mb) break;
       const int beg = g.row_ptr[rb0 + r], end = g.row_ptr[rb0 + r + 1];
@@ -874,6 +885,26 @@ __global__ __launch_bounds__(S::THREADS) void dsd_kernel(GemmArgs g, int tiles_m
                                                          int Mb, int Kb_all, ImplicitConv cg) {
   dsd_body<T, TRANS, CM, RAGGED, S, IMPLICIT>(g, tiles_m, tiles_n, Mb, Kb_all, cg, (int)blockIdx.x, (int)gridDim.y,
                                               (int)blockIdx.y);
+}
+
+// The forward product and the kept lists of its mask in ONE launch: workgroups [0, n_gemm) are the product's and take
+// their keep bits from the mask source itself (a handful of generator calls or mask bytes per workgroup), the others
+// build the lists the backward will read, and store a drawn mask.  Nothing in the launch waits for anything else.
+template <typename T, bool RAGGED, typename S>
+__global__ __launch_bounds__(S::THREADS) void forward_lists_kernel(GemmArgs g, int tiles_m, int tiles_n, int Mb,
+                                                                   int Kb_all, int nsplit, int n_gemm, FlatJobs f) {
+  const int bid = (int)blockIdx.x;
+  if (bid < n_gemm) {
+    MaskSrc ms = f.job0.src;
+    ms.resolve();
+    const int tiles = tiles_m * tiles_n;
+    dsd_body<T, false, false, RAGGED, S, 0>(g, tiles_m, tiles_n, Mb, Kb_all, ImplicitConv{}, bid % tiles, nsplit,
+                                            bid / tiles, &ms);
+  } else {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    flat_lists_block<S::THREADS>(f, bid - n_gemm, reinterpret_cast<int32_t*>(smem));
+  }
+  report_in(const_cast<uint64_t*>(f.job0.src.state), gridDim.x);
 }
 
 // ---- SDD with column groups ---------------------------------------------------------------------------
@@ -1590,6 +1621,68 @@ int launch_fast(const GemmArgs& g, int mode, int dtype, hipStream_t stream) {
   }
   if (nt) return cm ? launch_dsd<F16, false, true>(g, mid, splits, stream) : launch_dsd<F16, false, false>(g, mid, splits, stream);
   return cm ? launch_dsd<F16, true, true>(g, mid, splits, stream) : launch_dsd<F16, true, false>(g, mid, splits, stream);
+}
+
+// ---- the forward product and the kept lists of its mask in one launch -------------------------------------------
+// most workgroups the product may have for its lists to ride along (SPARSEDROP_FORWARD_LISTS_LIMIT overrides, for
+// measuring; 0 switches the single launch off)
+int64_t forward_lists_limit() {
+  static const int64_t limit = [] {
+    const char* e = std::getenv("SPARSEDROP_FORWARD_LISTS_LIMIT");
+    return e ? (int64_t)std::atoll(e) : (int64_t)512;
+  }();
+  return limit;
+}
+
+template <typename T, bool RAGGED, typename S>
+int launch_forward_lists_t(const GemmArgs& g, int splits, const FlatJobs& f, hipStream_t stream) {
+  static std::atomic<bool> configured[kMaxDevices] = {};
+  auto* kernel = &forward_lists_kernel<T, RAGGED, S>;
+  if (int rc = allow_big_lds(reinterpret_cast<const void*>(kernel), S::SMEM_BYTES, configured)) return rc;
+  const int Mb = (int)((g.M + BS - 1) / BS), Kb = (int)((g.K + BS - 1) / BS);
+  const int tiles_m = (Mb + S::R - 1) / S::R, tiles_n = (int)((g.N + S::BN - 1) / S::BN);
+  const int n_gemm = tiles_m * tiles_n * splits;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)(n_gemm + f.blocks())), dim3(S::THREADS), S::SMEM_BYTES, stream, g, tiles_m,
+                     tiles_n, Mb, Kb, splits, n_gemm, f);
+  if (int rc = check_launch("forward_lists_kernel")) return rc;
+  note_kernel("dsd+lists:%s%s splits=%d", S::R * BS == 256 && S::BN == 256 ? "big" : "mid", RAGGED ? ":ragged" : "",
+              splits);
+  if (splits > 1) return launch_splitk_reduce(g, splits, false, T::id, stream);
+  return SD_OK;
+}
+
+// g: the forward product (reduction-contiguous operands, row-major C) on the 64 grid; src: its mask, listed on an
+// mb x kb grid into the arrays given (either list may be absent), a drawn mask stored to mask_out.
+// SD_ERR_UNSUPPORTED (nothing launched, no message) unless the product runs on the specialised kernel, the mask is
+// small enough for the single-launch list build and the product small enough for the saved launch to matter.
+int launch_forward_with_lists(const GemmArgs& g, const MaskSrc& src, int64_t mb, int64_t kb, int32_t* row_ptr,
+                              int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx, uint8_t* mask_out,
+                              int64_t mask_rows, int dtype, hipStream_t stream) {
+  if (g.bs != BS || mb * kb > kFlatMaxEntries) return SD_ERR_UNSUPPORTED;
+  if (mb != (g.M + BS - 1) / BS || kb != (g.K + BS - 1) / BS) return SD_ERR_UNSUPPORTED;
+  // the forward's conditions (launch_fast)
+  const bool nt = g.a.sc == 1 && g.b.sc == 1 && g.c_sc == 1;
+  const bool shape_ok = g.M > 0 && g.N > 0 && g.K > 0 && g.K % 8 == 0 && (g.K + BS - 1) / BS < 65536;
+  const bool align_ok = aligned16(g.a.ptr) && aligned16(g.b.ptr) && g.a.sr % 8 == 0 && g.b.sr % 8 == 0 &&
+                        g.a.sr < (1 << 22) && g.b.sr < (1 << 22);
+  if (!nt || !shape_ok || !align_ok) return SD_ERR_UNSUPPORTED;
+  const DsdPlan plan = plan_dsd(g.M, g.N, g.K);
+  const int64_t tiles = plan.mid ? dsd_tiles<DsdMid>(g.M, g.N) : dsd_tiles<DsdBig>(g.M, g.N);
+  const int splits = usable_splits(g, plan, kDsd);
+  if (splits < 1 || tiles * splits > forward_lists_limit()) return SD_ERR_UNSUPPORTED;
+  const bool ragged = g.M % BS != 0 || g.N % BS != 0 || g.K % BS != 0 || g.quads;
+  const FlatJobs f = flat_jobs(src, mb, kb, row_ptr, col_idx, col_ptr, row_idx, mask_out, mask_rows,
+                               plan.mid ? DsdMid::THREADS : DsdBig::THREADS);
+  if (dtype == SD_BF16) {
+    if (plan.mid) return ragged ? launch_forward_lists_t<BF16, true, DsdMid>(g, splits, f, stream)
+                                : launch_forward_lists_t<BF16, false, DsdMid>(g, splits, f, stream);
+    return ragged ? launch_forward_lists_t<BF16, true, DsdBig>(g, splits, f, stream)
+                  : launch_forward_lists_t<BF16, false, DsdBig>(g, splits, f, stream);
+  }
+  if (plan.mid) return ragged ? launch_forward_lists_t<F16, true, DsdMid>(g, splits, f, stream)
+                              : launch_forward_lists_t<F16, false, DsdMid>(g, splits, f, stream);
+  return ragged ? launch_forward_lists_t<F16, true, DsdBig>(g, splits, f, stream)
+                : launch_forward_lists_t<F16, false, DsdBig>(g, splits, f, stream);
 }
 
 // ---- both gradients in one launch ------------------------------------------------------------------------

@@ -46,11 +46,12 @@ class BlockwiseDropoutMLPHIP(torch.autograd.Function):
                 kbs.append(0)
                 h = out
                 continue
-            mask, lists, kernel_bs = ext.kept_lists(h.shape[0], h.shape[1], block_size,
-                                                    None if masks is None else masks[i], p,
-                                                    None if seed is None else seed + i, h.device)
-            out, pre = ext.gemm_dsd_lists_act(h, w, lists, kernel_bs, 1.0 / (1.0 - p), None if last else activation,
-                                              want_pre=(not last and activation == "gelu"))
+            # mask, lists and product in one library call (one launch for small layers)
+            out, mask, lists, kernel_bs, pre = ext.dropout_matmul_forward_act(
+                h, w, block_size, p, None if masks is None else masks[i], None if seed is None else seed + i,
+                activation=None if last else activation, want_pre=(not last and activation == "gelu"))
+            if last or activation is None:
+                pre = None
             # per layer: weight, mask, the four list arrays, what the activation's derivative is evaluated at
             # (GELU: the pre-activation; ReLU: nothing extra, the activated output is the next layer's input)
             saved += [w, mask, lists.row_ptr, lists.col_idx, lists.col_ptr, lists.row_idx]

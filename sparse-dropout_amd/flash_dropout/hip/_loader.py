@@ -60,6 +60,9 @@ SIGNATURES = {
     "sd_dropout_matmul_forward": (c_int, [*_mat, *_mat, *_mat, *_mat, c_void_p, c_uint64, c_uint64, c_float, c_void_p,
                                           c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
                                           c_int, c_void_p, c_int64, c_void_p]),
+    "sd_dropout_matmul_forward_act": (c_int, [*_mat, *_mat, *_mat, *_mat, c_void_p, c_uint64, c_uint64, c_float,
+                                              c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                                              c_int64, c_int64, c_int, c_int, *_mat, c_void_p, c_int64, c_void_p]),
     "sd_gemm_act": (c_int, [*_mat, *_mat, *_mat, c_int64, c_int64, c_int64, c_int, c_int, *_mat, c_void_p, c_int64,
                             c_void_p]),
     "sd_dropout_matmul_backward": (c_int, [*_mat, *_mat, *_mat, *_mat, *_mat, c_void_p, c_void_p, c_void_p, c_void_p,

@@ -554,10 +554,18 @@ class GEMM:
     def dropout_matmul_forward(self, x: torch.Tensor, w: torch.Tensor, block_size, p: float,
                                mask: torch.Tensor | None = None, seed: int | None = None):
         """Mask (given, or drawn on the device: pinned by ``seed``, else from the device-resident generator),
-        kept-block lists and ``Y = (keep ⊙ x)/(1-p) @ w.T`` in one library call -> (y, mask, lists, kernel block
-        size).  The lists are at the granularity the kernels run at (64 for block sizes that are multiples of
-        64) and serve :meth:`dropout_matmul_backward`."""
+        kept-block lists and ``Y = (keep ⊙ x)/(1-p) @ w.T`` in one library call - and, for small layers, one
+        launch -> (y, mask, lists, kernel block size).  The lists are at the granularity the kernels run at (64
+        for block sizes that are multiples of 64) and serve :meth:`dropout_matmul_backward`."""
+        return self.dropout_matmul_forward_act(x, w, block_size, p, mask, seed)[:4]
+
+    def dropout_matmul_forward_act(self, x: torch.Tensor, w: torch.Tensor, block_size, p: float,
+                                   mask: torch.Tensor | None = None, seed: int | None = None,
+                                   activation: str | None = None, want_pre: bool = False):
+        """:meth:`dropout_matmul_forward` with the activation ("relu", "gelu" or None) applied in the product's
+        store -> (activated y, mask, lists, kernel block size, pre-activation or None)."""
         self._check_pair(x, w)
+        code = _activation(activation)
         bs = _block_size(block_size)
         if not 0.0 <= p < 1.0:
             raise ValueError(f"p must be in [0, 1), got {p}")
@@ -578,14 +586,17 @@ class GEMM:
             given = (mask.data_ptr(), *_mask_strides(mask))
         row_ptr, col_ptr, col_idx, row_idx = self._list_buffers(out_mb, out_kb, dev)
         y = torch.empty((M, N), dtype=x.dtype, device=dev)
+        pre = torch.empty((M, N), dtype=x.dtype, device=dev) if (want_pre and code) else None
         ws, ws_ptr, ws_bytes = self._splitk_scratch(x, w, g, 1)
         with _guard(dev):
-            self._call(self.lib.sd_dropout_matmul_forward, *_mat(x), *_mat(w), *_mat(y), *given,
+            self._call(self.lib.sd_dropout_matmul_forward_act, *_mat(x), *_mat(w), *_mat(y), *given,
                        None if state is None else state.data_ptr(), (int(seed) & (2 ** 64 - 1)) if seed is not None else 0,
                        0, float(p), mask.data_ptr(), row_ptr.data_ptr(), col_idx.data_ptr(), col_ptr.data_ptr(),
-                       row_idx.data_ptr(), M, N, K, bs, _DTYPES[x.dtype], ws_ptr, ws_bytes, self._stream(x))
+                       row_idx.data_ptr(), M, N, K, bs, _DTYPES[x.dtype], code,
+                       *(_mat(pre) if pre is not None else (None, 0, 0)), ws_ptr, ws_bytes, self._stream(x))
         # block size 32 stays 32 for the backward call: it says that the lists carry quadrant bits
-        return y, mask, KeptLists(row_ptr, col_idx, col_ptr, row_idx, (out_mb, out_kb)), (32 if bs == 32 else g)
+        return (y, mask, KeptLists(row_ptr, col_idx, col_ptr, row_idx, (out_mb, out_kb)), (32 if bs == 32 else g),
+                pre if code else (y if want_pre else None))
 
     def dropout_matmul_backward(self, dy: torch.Tensor, w: torch.Tensor, x: torch.Tensor, lists: KeptLists,
                                 block_size, p: float, need_dx: bool = True, need_dw: bool = True,

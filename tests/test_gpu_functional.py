@@ -279,6 +279,66 @@ def test_fused_forward_and_backward_calls_match_the_separate_ones(bs):
     assert np.array_equal(m5.cpu().numpy(), O.random_mask(O.mask_shape(M, K, bs), p, 5, offset=1))
 
 
+@pytest.mark.parametrize("M,K,N,bs,dtype,merged", [
+    (1024, 1024, 1024, 64, torch.float16, True),      # aligned
+    (4096, 784, 1024, 64, torch.float16, True),       # ragged K
+    (2048, 512, 384, 128, torch.bfloat16, True),      # bf16, a mask at block size 128 listed on the 64 grid
+    (1000, 520, 264, 32, torch.float16, True),        # ragged everywhere, block size 32 (quadrant keep bits)
+    (256, 4096, 256, 64, torch.float16, True),        # few output tiles, long reduction: split over workgroups
+    (8192, 2048, 4352, 64, torch.float16, False),     # 544 workgroups: the list build stays a launch of its own
+])
+def test_forward_that_builds_its_lists_in_the_same_launch(M, K, N, bs, dtype, merged):
+    """sd_dropout_matmul_forward_act on a small layer is ONE launch (forward_lists_kernel): the product's workgroups
+    take their keep bits from the mask source, other workgroups of the grid write the lists and the drawn mask.  Mask,
+    lists, product and pre-activation must be, bit for bit, what the list build and the list-driven product give as
+    launches of their own, for a stored mask, a seeded draw and the device-resident generator."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(29)
+    p = 0.5
+    x = torch.randn(M, K, generator=gen).to(dtype).cuda()
+    w = (torch.randn(N, K, generator=gen) * K ** -0.5).to(dtype).cuda()
+    s = 1 / (1 - p)
+    split = 0 if bs == 32 else max(bs // 64, 1)
+    grid = (-(-M // 64), -(-K // 64))
+
+    def same_lists(a, b):
+        nnz = b.nnz()
+        assert a.shape == b.shape and a.nnz() == nnz
+        assert torch.equal(a.row_ptr, b.row_ptr) and torch.equal(a.col_ptr, b.col_ptr)
+        assert torch.equal(a.col_idx[:nnz], b.col_idx[:nnz]) and torch.equal(a.row_idx[:nnz], b.row_idx[:nnz])
+
+    def check(y, pre, mask, lists, g, act):
+        assert ext.last_kernel_detail().startswith("dsd+lists:") == merged, ext.last_kernel_detail()
+        want_lists = ext.build_lists(mask, split, grid) if bs != 64 else ext.build_lists(mask)
+        same_lists(lists, want_lists)
+        want_y, want_pre = ext.gemm_dsd_lists_act(x, w, want_lists, g, s, act, want_pre=pre is not None)
+        assert not ext.last_kernel_detail().startswith("dsd+lists:")
+        assert torch.equal(y, want_y)
+        if pre is not None:
+            assert torch.equal(pre, want_pre)
+
+    # a stored mask, plain and with the activation in the store
+    mask = cpu_mask(O.mask_shape(M, K, bs), p, gen).cuda()
+    y, m, lists, g = ext.dropout_matmul_forward(x, w, bs, p, mask=mask)
+    check(y, None, mask, lists, g, None)
+    y, m, lists, g, pre = ext.dropout_matmul_forward_act(x, w, bs, p, mask=mask, activation="gelu", want_pre=True)
+    check(y, pre, mask, lists, g, "gelu")
+    if M * K * N <= 1 << 31:
+        assert max_tile_rel_fro(pre, O.dsd_forward(to_np(x), to_np(w), mask.cpu().numpy(), bs, p, np.float32)) <= REL_FRO_TOL
+    # a seeded draw: the oracle's mask, stored for the caller
+    y, m, lists, g, pre = ext.dropout_matmul_forward_act(x, w, bs, p, seed=91, activation="relu")
+    assert pre is None and np.array_equal(m.cpu().numpy(), O.random_mask(O.mask_shape(M, K, bs), p, 91))
+    check(y, None, m, lists, g, "relu")
+    # the device-resident generator: every workgroup of the launch reads the state before the last one moves it on
+    ext.manual_seed(12)
+    for offset in range(3):
+        y, m, lists, g = ext.dropout_matmul_forward(x, w, bs, p)
+        assert np.array_equal(m.cpu().numpy(), O.random_mask(O.mask_shape(M, K, bs), p, 12, offset=offset))
+        check(y, None, m, lists, g, None)
+
+
 @pytest.mark.parametrize("M,K,N,bs,dtype,paired", [
     (1024, 1024, 1024, 64, torch.float16, True),      # aligned, both products on a fraction of the chip
     (4096, 784, 1024, 64, torch.float16, True),       # ragged K, weight gradient with a split reduction
