@@ -249,7 +249,7 @@ def test_as_matrix_lays_out_expanded_and_strided_views():
     assert _mat(torch.zeros(1, 8))[1:] == (8, 1)
 
 
-@pytest.mark.parametrize("name", ["mfma_ceiling.hip", "lds_load_ceiling.hip"])
+@pytest.mark.parametrize("name", ["mfma_ceiling.hip", "lds_load_ceiling.hip", "dense_4wave_probe.hip"])
 def test_ceiling_probes_compile_for_gfx950(name, tmp_path):
     """The stand-alone measurement programs under benchmark/ are only ever run on a GPU box by hand: keep them
     compiling (device code for gfx950, no GPU needed)."""
