@@ -11,6 +11,8 @@
 //             together are 192 MB (they stay in the 256 MB memory-side cache), with 128 they are 384 MB (the
 //             L2 misses, a fifth of the requests, go to HBM as 128-byte reads 16 KB apart)
 //   hbm       private regions far larger than the caches
+//   staged    the shared pattern with the tiles going through registers instead: global_load_dwordx4 for the next
+//             step at the top of a step, ds_write_b128 into the other stage behind the step's fragment reads
 // It prints bytes into LDS per second over the chip; the GEMM kernels' own rate is to be read against these.
 //
 //   hipcc --offload-arch=gfx950 -O3 -w -Xclang -target-feature -Xclang -packed-fp32-ops \
@@ -35,7 +37,10 @@ __device__ inline void load16_to_lds(const char* base, uint32_t lane_off, uint32
 // mode 0: private contiguous; 1: private tile rows; 2: shared panels of an XCD patch
 // reads: 1 KB ds_read_b128 per wave and step from the stage that has landed (the GEMM kernels read 24: 16 KB of X
 // fragments and 8 KB of W fragments per wave)
+// NL: loads per wave and step (8 = the dense step's 64 KB; 6 = the 48 KB of a step at p = 0.5: the W tile and two of
+// the four X tiles)
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <int NL>
 __global__ __launch_bounds__(THREADS) void stream(const char* src, size_t region, int steps, int mode, int reads,
                                                   int positions, int* sink) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -51,7 +56,7 @@ __global__ __launch_bounds__(THREADS) void stream(const char* src, size_t region
   auto issue = [&](int step, int stage) {
     const uint32_t st = smem_a + stage * STAGE + wave * (LOADS * 1024);
 #pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
+    for (int i = 0; i < NL; ++i) {
       const char* p;
       if (mode == 0) {
         p = src + (size_t)wg * region + ((size_t)step * STAGE + (wave * LOADS + i) * 1024) % region;
@@ -68,11 +73,43 @@ __global__ __launch_bounds__(THREADS) void stream(const char* src, size_t region
     }
   };
   u32x4 x = {0, 0, 0, 0};
+  if (mode == 3) {  // through registers
+    u32x4 regs[NL];
+    auto fetch = [&](int step) {
+#pragma unroll
+      for (int i = 0; i < NL; ++i) {
+        const int l = wave * LOADS + i;
+        const int panel = l < 32 ? pr : 8 + pc;
+        const char* p = src + ((size_t)xcd * 12 + panel) * 256 * ROW + (size_t)(l % 32) * 8 * ROW +
+                        (size_t)(step % positions) * 128 + (size_t)((lane / 8) * ROW + (lane % 8) * 16);
+        regs[i] = *reinterpret_cast<const u32x4*>(p);
+      }
+    };
+    auto put = [&](int stage) {
+#pragma unroll
+      for (int i = 0; i < NL; ++i)
+        *reinterpret_cast<u32x4*>(smem + stage * STAGE + (wave * LOADS + i) * 1024 + lane * 16) = regs[i];
+    };
+    fetch(0);
+    put(0);
+    __syncthreads();
+    for (int step = 0; step < steps; ++step) {
+      if (step + 1 < steps) fetch(step + 1);
+      const char* st = smem + (step & 1) * STAGE + lane * 16;
+      for (int i = 0; i < reads; ++i) x ^= *reinterpret_cast<const u32x4*>(st + ((wave * 24 + i) % 64) * 1024);
+      if (step + 1 < steps) put((step + 1) & 1);
+      __syncthreads();
+    }
+    if ((x.x ^ x.y ^ x.z ^ x.w) == 0x12345678u) sink[wg] = 1;
+    return;
+  }
   issue(0, 0);
   for (int step = 0; step < steps; ++step) {
     if (step + 1 < steps) {
       issue(step + 1, (step + 1) & 1);
-      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");  // the loads of this step have landed, the next 8 fly
+      // the loads of this step have landed, the next NL fly
+      if (NL == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
@@ -91,8 +128,9 @@ int main() {
   if (hipMalloc(&d, bytes) != hipSuccess) { printf("hipMalloc failed\n"); return 1; }
   hipMemset(d, 1, bytes);
   int* sink; hipMalloc(&sink, wgs * 4);
-  hipFuncSetAttribute((const void*)stream, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * STAGE);
-  struct { const char* name; int mode; size_t region; int reads; int positions; } cases[] = {
+  hipFuncSetAttribute((const void*)stream<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * STAGE);
+  hipFuncSetAttribute((const void*)stream<6>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * STAGE);
+  struct { const char* name; int mode; size_t region; int reads; int positions; int nl = 8; } cases[] = {
       {"private, 64 KB regions (L2)", 0, (size_t)64 << 10, 0, 128},
       {"private, 512 KB regions", 0, (size_t)512 << 10, 0, 128},
       {"hbm: private, 16 MB regions", 0, (size_t)16 << 20, 0, 128},
@@ -101,18 +139,26 @@ int main() {
       {"shared, 192 MB + 24 KB LDS reads / wave", 2, 0, 24, 64},
       {"shared, 384 MB of panels", 2, 0, 0, 128},
       {"shared, 384 MB + 24 KB LDS reads / wave", 2, 0, 24, 128},
+      {"p=.5 step: 48 KB loads + 14 KB reads / wave", 2, 0, 14, 128, 6},
+      {"staged, 384 MB of panels", 3, 0, 0, 128},
+      {"staged, 384 MB + 24 KB LDS reads / wave", 3, 0, 24, 128},
+      {"staged, p=.5 step: 48 KB + 14 KB reads / wave", 3, 0, 14, 128, 6},
   };
   for (auto& c : cases) {
     for (int rep = 0; rep < 2; ++rep) {
       hipEvent_t e0, e1; hipEventCreate(&e0); hipEventCreate(&e1);
-      stream<<<wgs, THREADS, 2 * STAGE>>>(d, c.region, 64, c.mode, c.reads, c.positions, sink);
+      auto launch = [&](int n) {
+        if (c.nl == 8) stream<8><<<wgs, THREADS, 2 * STAGE>>>(d, c.region, n, c.mode, c.reads, c.positions, sink);
+        else stream<6><<<wgs, THREADS, 2 * STAGE>>>(d, c.region, n, c.mode, c.reads, c.positions, sink);
+      };
+      launch(64);
       hipDeviceSynchronize();
       hipEventRecord(e0);
-      stream<<<wgs, THREADS, 2 * STAGE>>>(d, c.region, steps, c.mode, c.reads, c.positions, sink);
+      launch(steps);
       hipEventRecord(e1); hipEventSynchronize(e1);
       float ms; hipEventElapsedTime(&ms, e0, e1);
       if (hipGetLastError() != hipSuccess) { printf("launch failed\n"); return 1; }
-      const double tb = (double)wgs * steps * STAGE / (ms * 1e-3) / 1e12;
+      const double tb = (double)wgs * steps * (c.nl * THREADS / 64 * 1024) / (ms * 1e-3) / 1e12;
       printf("%-40s %8.3f ms  %6.2f TB/s into LDS  (%.1f B/clk/CU at 2.4 GHz)\n", c.name, ms, tb, tb * 1e12 / 256 / 2.4e9);
     }
   }
