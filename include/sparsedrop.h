@@ -326,12 +326,16 @@ int sd_gemm_sdd_lists_kept(const void* A, int64_t a_stride_r, int64_t a_stride_c
  * (written in full, zeros where dropped) and dW = dY^T . (keep . X) / (1 - p), each skipped when its pointer is NULL.
  * dW is written through its own strides: pass a row-major [N, K] tensor to get what the reference returns as a
  * transposed view.  workspace: optional split-reduction scratch for dW (sd_splitk_workspace_bytes(K, N, M, g, 1)).
+ *
+ * p is a double in these calls: the products are scaled by (float)(1 / (1 - p)) evaluated in double precision, which
+ * is the number the reference's Python passes to its kernels (blockwise_dropout_matmul_cuda.py:29), and the draw
+ * compares against (float)p as sd_random_lists does.
  * ------------------------------------------------------------------------------------------- */
 int sd_dropout_matmul_forward(const void* X, int64_t x_stride_r, int64_t x_stride_c,
                               const void* W, int64_t w_stride_r, int64_t w_stride_c,
                               void* Y, int64_t y_stride_r, int64_t y_stride_c,
                               const uint8_t* mask, int64_t mask_stride_r, int64_t mask_stride_c,
-                              uint64_t* rng_state, uint64_t seed, uint64_t offset, float p, uint8_t* mask_out,
+                              uint64_t* rng_state, uint64_t seed, uint64_t offset, double p, uint8_t* mask_out,
                               int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx,
                               int64_t M, int64_t N, int64_t K, int64_t block_size, int dtype,
                               void* workspace, int64_t workspace_bytes, void* stream);
@@ -343,7 +347,7 @@ int sd_dropout_matmul_backward(const void* dY, int64_t dy_stride_r, int64_t dy_s
                                void* dW, int64_t dw_stride_r, int64_t dw_stride_c,
                                const int32_t* row_ptr, const int32_t* col_idx,
                                const int32_t* col_ptr, const int32_t* row_idx,
-                               int64_t M, int64_t N, int64_t K, int64_t block_size, float p, int dtype,
+                               int64_t M, int64_t N, int64_t K, int64_t block_size, double p, int dtype,
                                void* workspace, int64_t workspace_bytes, void* stream);
 
 /* The same with the derivative of an activation multiplied into dX (sd_gemm_sdd_lists_actgrad's epilogue):
@@ -361,7 +365,7 @@ int sd_dropout_matmul_backward_act(const void* dY, int64_t dy_stride_r, int64_t 
                                    void* dW, int64_t dw_stride_r, int64_t dw_stride_c,
                                    const int32_t* row_ptr, const int32_t* col_idx,
                                    const int32_t* col_ptr, const int32_t* row_idx,
-                                   int64_t M, int64_t N, int64_t K, int64_t block_size, float p, int dtype,
+                                   int64_t M, int64_t N, int64_t K, int64_t block_size, double p, int dtype,
                                    int act, const void* act_at, int64_t at_stride_r, int64_t at_stride_c,
                                    void* workspace, int64_t workspace_bytes, void* stream);
 
@@ -376,7 +380,7 @@ int sd_dropout_matmul_forward_act(const void* X, int64_t x_stride_r, int64_t x_s
                                   const void* W, int64_t w_stride_r, int64_t w_stride_c,
                                   void* Y, int64_t y_stride_r, int64_t y_stride_c,
                                   const uint8_t* mask, int64_t mask_stride_r, int64_t mask_stride_c,
-                                  uint64_t* rng_state, uint64_t seed, uint64_t offset, float p, uint8_t* mask_out,
+                                  uint64_t* rng_state, uint64_t seed, uint64_t offset, double p, uint8_t* mask_out,
                                   int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx,
                                   int64_t M, int64_t N, int64_t K, int64_t block_size, int dtype,
                                   int act, void* pre_out, int64_t pre_stride_r, int64_t pre_stride_c,

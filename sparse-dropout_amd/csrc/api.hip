@@ -484,7 +484,7 @@ static int64_t list_granule(int64_t bs) { return (bs % 64 == 0 || bs == 32) ? 64
 
 int sd_dropout_matmul_forward(const void* X, int64_t xsr, int64_t xsc, const void* W, int64_t wsr, int64_t wsc,
                               void* Y, int64_t ysr, int64_t ysc, const uint8_t* mask, int64_t msr, int64_t msc,
-                              uint64_t* rng_state, uint64_t seed, uint64_t offset, float p, uint8_t* mask_out,
+                              uint64_t* rng_state, uint64_t seed, uint64_t offset, double p, uint8_t* mask_out,
                               int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx, int64_t M,
                               int64_t N, int64_t K, int64_t bs, int dtype, void* workspace, int64_t workspace_bytes,
                               void* stream) {
@@ -504,7 +504,7 @@ static bool separate_forward_forced() {
 
 int sd_dropout_matmul_forward_act(const void* X, int64_t xsr, int64_t xsc, const void* W, int64_t wsr, int64_t wsc,
                                   void* Y, int64_t ysr, int64_t ysc, const uint8_t* mask, int64_t msr, int64_t msc,
-                                  uint64_t* rng_state, uint64_t seed, uint64_t offset, float p, uint8_t* mask_out,
+                                  uint64_t* rng_state, uint64_t seed, uint64_t offset, double p, uint8_t* mask_out,
                                   int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx, int64_t M,
                                   int64_t N, int64_t K, int64_t bs, int dtype, int act, void* pre_out,
                                   int64_t pre_stride_r, int64_t pre_stride_c, void* workspace, int64_t workspace_bytes,
@@ -517,7 +517,7 @@ int sd_dropout_matmul_forward_act(const void* X, int64_t xsr, int64_t xsc, const
   if (int rc = check_act(act, pre_out, pre_stride_r, pre_stride_c, M, N, false)) return rc;
   const int64_t g = list_granule(bs), split = bs / g;  // 0 for block size 32: merged two by two
   const int64_t mb = ceil_div(M, bs), kb = ceil_div(K, bs), out_mb = ceil_div(M, g), out_kb = ceil_div(K, g);
-  const float scale = 1.f / (1.f - p);
+  const float scale = (float)(1.0 / (1.0 - p));  // in double, as the reference's Python evaluates it
   // what the list calls below would check, up front: the single launch takes the same arguments
   if (int rc = check_list_grid(mb, kb, split, out_mb, out_kb, row_ptr, col_idx, col_ptr, row_idx)) return rc;
   if (mask) {
@@ -538,7 +538,7 @@ int sd_dropout_matmul_forward_act(const void* X, int64_t xsr, int64_t xsc, const
     // lists and product in one launch where the pair qualifies (small products, where a launch is a large part)
     const GemmArgs a = with_act(make_args(X, xsr, xsc, W, wsr, wsc, Y, ysr, ysc, M, N, K, bs == 32 ? 32 : g, scale,
                                           row_ptr, col_idx, workspace, workspace_bytes));
-    const int rc = forward_with_lists(a, mask, msr, msc, seed, offset, rng_state, p, mb, kb, mask_out, split, out_mb,
+    const int rc = forward_with_lists(a, mask, msr, msc, seed, offset, rng_state, (float)p, mb, kb, mask_out, split, out_mb,
                                       out_kb, row_ptr, col_idx, col_ptr, row_idx, dtype, (hipStream_t)stream);
     if (rc != SD_ERR_UNSUPPORTED) {
       last_kernel = "specialised";
@@ -550,11 +550,11 @@ int sd_dropout_matmul_forward_act(const void* X, int64_t xsr, int64_t xsc, const
                                       stream))
       return rc;
   } else if (rng_state) {
-    if (int rc = sd_random_lists_state(rng_state, p, mb, kb, mask_out, split, out_mb, out_kb, row_ptr, col_idx, col_ptr,
+    if (int rc = sd_random_lists_state(rng_state, (float)p, mb, kb, mask_out, split, out_mb, out_kb, row_ptr, col_idx, col_ptr,
                                        row_idx, stream))
       return rc;
   } else {
-    if (int rc = sd_random_lists(seed, offset, p, mb, kb, mask_out, split, out_mb, out_kb, row_ptr, col_idx, col_ptr,
+    if (int rc = sd_random_lists(seed, offset, (float)p, mb, kb, mask_out, split, out_mb, out_kb, row_ptr, col_idx, col_ptr,
                                  row_idx, stream))
       return rc;
   }
@@ -568,7 +568,7 @@ int sd_dropout_matmul_backward(const void* dY, int64_t gsr, int64_t gsc, const v
                                const void* X, int64_t xsr, int64_t xsc, void* dX, int64_t dxsr, int64_t dxsc,
                                void* dW, int64_t dwsr, int64_t dwsc, const int32_t* row_ptr, const int32_t* col_idx,
                                const int32_t* col_ptr, const int32_t* row_idx, int64_t M, int64_t N, int64_t K,
-                               int64_t bs, float p, int dtype, void* workspace, int64_t workspace_bytes, void* stream) {
+                               int64_t bs, double p, int dtype, void* workspace, int64_t workspace_bytes, void* stream) {
   return sd_dropout_matmul_backward_act(dY, gsr, gsc, W, wsr, wsc, X, xsr, xsc, dX, dxsr, dxsc, dW, dwsr, dwsc, row_ptr,
                                         col_idx, col_ptr, row_idx, M, N, K, bs, p, dtype, SD_ACT_NONE, nullptr, 0, 0,
                                         workspace, workspace_bytes, stream);
@@ -578,7 +578,7 @@ int sd_dropout_matmul_backward_act(const void* dY, int64_t gsr, int64_t gsc, con
                                    const void* X, int64_t xsr, int64_t xsc, void* dX, int64_t dxsr, int64_t dxsc,
                                    void* dW, int64_t dwsr, int64_t dwsc, const int32_t* row_ptr,
                                    const int32_t* col_idx, const int32_t* col_ptr, const int32_t* row_idx, int64_t M,
-                                   int64_t N, int64_t K, int64_t bs, float p, int dtype, int act, const void* act_at,
+                                   int64_t N, int64_t K, int64_t bs, double p, int dtype, int act, const void* act_at,
                                    int64_t at_stride_r, int64_t at_stride_c, void* workspace, int64_t workspace_bytes,
                                    void* stream) {
   SD_REQUIRE(p >= 0.f && p < 1.f, "dropout_matmul_backward: p must be in [0, 1) (got %g)", (double)p);
@@ -588,13 +588,13 @@ int sd_dropout_matmul_backward_act(const void* dY, int64_t gsr, int64_t gsc, con
   if (int rc = check_sparse(bs, 1.f)) return rc;
   SD_REQUIRE(dX || dW, "dropout_matmul_backward: nothing to compute");
   const int64_t g = bs == 32 ? 32 : list_granule(bs);  // 32: lists on the 64 grid with quadrant bits
-  const float scale = 1.f / (1.f - p);
+  const float scale = (float)(1.0 / (1.0 - p));  // in double, as the reference's Python evaluates it
   if (dX && dW && row_ptr && col_idx && col_ptr && row_idx && !generic_forced() && !separate_backward_forced()) {
     // both gradients in one launch where the pair qualifies (same operands and checks as the two calls below)
     if (int rc = check_common(dY, gsr, gsc, W, wsc, wsr, dX, dxsr, dxsc, M, K, N, dtype)) return rc;
     if (int rc = check_common(X, xsc, xsr, dY, gsc, gsr, dW, dwsc, dwsr, K, N, M, dtype)) return rc;
     GemmArgs gx = make_args(dY, gsr, gsc, W, wsc, wsr, dX, dxsr, dxsc, M, K, N, g, scale, row_ptr, col_idx);
-    gx.keep_hint = 1.f - p;
+    gx.keep_hint = (float)(1.0 - p);
     gx.act = act;
     gx.aux = act != SD_ACT_NONE ? const_cast<uint16_t*>(static_cast<const uint16_t*>(act_at)) : nullptr;
     gx.aux_sr = at_stride_r;
@@ -611,7 +611,7 @@ int sd_dropout_matmul_backward_act(const void* dY, int64_t gsr, int64_t gsc, con
     // dX[M,K] = scale * (dY[M,N] . W[N,K]) where kept: A = dY, B = W^T as the [K, N] view of W
     SD_REQUIRE(row_ptr && col_idx, "dropout_matmul_backward: dX needs the CSR lists");
     if (int rc = sd_gemm_sdd_lists_actgrad(dY, gsr, gsc, W, wsc, wsr, dX, dxsr, dxsc, row_ptr, col_idx, M, K, N, g,
-                                           scale, dtype, act, act_at, at_stride_r, at_stride_c, 1.f - p, stream))
+                                           scale, dtype, act, act_at, at_stride_r, at_stride_c, (float)(1.0 - p), stream))
       return rc;
   }
   if (dW) {

@@ -7,7 +7,7 @@ loading raises.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_float, c_int, c_int64, c_uint64, c_void_p
+from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_uint64, c_void_p
 import hashlib
 from functools import lru_cache
 from pathlib import Path
@@ -57,19 +57,19 @@ SIGNATURES = {
                                           c_float, c_int, c_int, *_mat, c_float, c_void_p]),
     "sd_gemm_sdd_lists_kept": (c_int, [*_mat, *_mat, *_mat, c_void_p, c_void_p, c_int64, c_int64,
                                   c_int64, c_int64, c_float, c_int, c_void_p]),
-    "sd_dropout_matmul_forward": (c_int, [*_mat, *_mat, *_mat, *_mat, c_void_p, c_uint64, c_uint64, c_float, c_void_p,
+    "sd_dropout_matmul_forward": (c_int, [*_mat, *_mat, *_mat, *_mat, c_void_p, c_uint64, c_uint64, c_double, c_void_p,
                                           c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
                                           c_int, c_void_p, c_int64, c_void_p]),
-    "sd_dropout_matmul_forward_act": (c_int, [*_mat, *_mat, *_mat, *_mat, c_void_p, c_uint64, c_uint64, c_float,
+    "sd_dropout_matmul_forward_act": (c_int, [*_mat, *_mat, *_mat, *_mat, c_void_p, c_uint64, c_uint64, c_double,
                                               c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
                                               c_int64, c_int64, c_int, c_int, *_mat, c_void_p, c_int64, c_void_p]),
     "sd_gemm_act": (c_int, [*_mat, *_mat, *_mat, c_int64, c_int64, c_int64, c_int, c_int, *_mat, c_void_p, c_int64,
                             c_void_p]),
     "sd_dropout_matmul_backward": (c_int, [*_mat, *_mat, *_mat, *_mat, *_mat, c_void_p, c_void_p, c_void_p, c_void_p,
-                                           c_int64, c_int64, c_int64, c_int64, c_float, c_int, c_void_p, c_int64,
+                                           c_int64, c_int64, c_int64, c_int64, c_double, c_int, c_void_p, c_int64,
                                            c_void_p]),
     "sd_dropout_matmul_backward_act": (c_int, [*_mat, *_mat, *_mat, *_mat, *_mat, c_void_p, c_void_p, c_void_p,
-                                               c_void_p, c_int64, c_int64, c_int64, c_int64, c_float, c_int,
+                                               c_void_p, c_int64, c_int64, c_int64, c_int64, c_double, c_int,
                                                c_int, *_mat, c_void_p, c_int64, c_void_p]),
     "sd_conv2d_dsd_lists": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64,
                                     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,

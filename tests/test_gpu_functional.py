@@ -339,6 +339,34 @@ def test_forward_that_builds_its_lists_in_the_same_launch(M, K, N, bs, dtype, me
         check(y, None, m, lists, g, None)
 
 
+@pytest.mark.parametrize("p", [0.0, 0.95])
+@pytest.mark.parametrize("bs", [32, 64])
+def test_forward_with_its_lists_at_the_ends_of_the_drop_range(p, bs):
+    """The single-launch forward with nothing dropped, with nearly everything dropped (row blocks without a kept block,
+    workgroups without a step) and with the mask stored column-major: bit for bit what the separate launches give."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(31)
+    M, K, N = 1000, 520, 264
+    x = torch.randn(M, K, generator=gen).half().cuda()
+    w = (torch.randn(N, K, generator=gen) * K ** -0.5).half().cuda()
+    s = 1 / (1 - p)
+    mask = cpu_mask(O.mask_shape(M, K, bs), p, gen).cuda()
+    for stored in (mask, mask.t().contiguous().t()):  # row-major, column-major
+        y, m, lists, g = ext.dropout_matmul_forward(x, w, bs, p, mask=stored)
+        assert ext.last_kernel_detail().startswith("dsd+lists:")
+        want = ext.build_lists(mask, 0, (-(-M // 64), -(-K // 64))) if bs == 32 else ext.build_lists(mask)
+        nnz = want.nnz()
+        assert lists.nnz() == nnz and torch.equal(lists.row_ptr, want.row_ptr) and torch.equal(lists.col_ptr, want.col_ptr)
+        assert torch.equal(lists.col_idx[:nnz], want.col_idx[:nnz]) and torch.equal(lists.row_idx[:nnz], want.row_idx[:nnz])
+        assert torch.equal(y, ext.gemm_dsd_lists(x, w, want, g, s))
+        assert max_tile_rel_fro(y, O.dsd_forward(to_np(x), to_np(w), mask.cpu().numpy(), bs, p, np.float32)) <= REL_FRO_TOL
+    y, m, lists, g = ext.dropout_matmul_forward(x, w, bs, p, seed=5)
+    assert np.array_equal(m.cpu().numpy(), O.random_mask(O.mask_shape(M, K, bs), p, 5))
+    assert max_tile_rel_fro(y, O.dsd_forward(to_np(x), to_np(w), m.cpu().numpy(), bs, p, np.float32)) <= REL_FRO_TOL
+
+
 @pytest.mark.parametrize("M,K,N,bs,dtype,paired", [
     (1024, 1024, 1024, 64, torch.float16, True),      # aligned, both products on a fraction of the chip
     (4096, 784, 1024, 64, torch.float16, True),       # ragged K, weight gradient with a split reduction
