@@ -542,7 +542,8 @@ __device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int til
   }
   const int64_t b_red_stride = TRANS ? (int64_t)BS * g.b.sc * 2 : (int64_t)BS * 2;
 
-  auto issue_loads = [&](uint32_t entry, int stage) {  // entry: wave-uniform step table word
+  // with_w: the W tile too; rowsel: bit r = the X tile of row block r may be loaded (if the step keeps it)
+  auto issue_loads = [&](uint32_t entry, int stage, bool with_w = true, uint32_t rowsel = 0xfu) {  // entry: wave-uniform step table word
     const int kb = step_block(entry);
     const uint32_t fl = step_flags(entry);
     [[maybe_unused]] char* st = smem + stage * STAGE;
@@ -552,14 +553,14 @@ __device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int til
     const bool red_tail = RAGGED && kb == kb_tail;  // wave-uniform
 #pragma unroll
     for (int jj = 0; jj < BL; ++jj)
-      if (b_valid[jj]) {
+      if (with_w && b_valid[jj]) {
         uint32_t off = b_lane[jj];
         if (RAGGED) off += red_tail ? b_delta_k[jj] : 0u;
         load16_to_lds(bp, off, st_a + (uint32_t)((wave_u * BL + jj) * 1024));
       }
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      if (row_quads(fl, r)) {
+      if (row_quads(fl, r) && ((rowsel >> r) & 1u)) {
         if constexpr (IMPLICIT && !TRANS) {
           gather_tile(r, kb, st + A_OFF + r * TILE);
           continue;
@@ -679,10 +680,141 @@ __device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int til
   const bool late = __builtin_amdgcn_readfirstlane(rh) != 0;
   uint32_t e_cur = uniform(step_e[0]), e_next = uniform(step_e[1]);
 
-  // SD_TIMING_NO_LOADS / SD_TIMING_NO_READS / SD_TIMING_NO_MFMA compile the tile loads / the fragment reads / the
-  // MFMAs out of the step loop below: builds for timing what the rest costs (benchmark/decompose.py), whose results
-  // are wrong by construction.  The library is never built with them.
-  if constexpr (IMPLICIT == 0) {
+  // ---- the step loop of the 256 x 256 shape on aligned operands: the two waves of a SIMD in opposite phases -------
+  // Waves w and w + 4 (the two row-block pairs of one column slice) share a SIMD.  A step of a wave is a MEMORY phase -
+  // every fragment of the step is read into registers, then the wave's share of the coming tiles is put on its way -
+  // followed by a COMPUTE phase that issues nothing but MFMAs.  A barrier ends each phase, and the second group of
+  // four waves starts one phase later than the first: whenever one wave of a SIMD stands at a fragment read or a load,
+  // the other one feeds the matrix cores.  (With both waves in the same phase the parts of a step add up, because a
+  // wave that stands at a memory instruction issues no MFMA behind it: 8192^3 dense forward 0.95 -> 0.82 ms.)
+  // Who loads what follows from who reads what first.  Group 0 (row blocks 0-1) reads the W tile of step c in phase
+  // 2c, group 1 (row blocks 2-3) in phase 2c + 1; X tiles are read by their own group only.  So, reading step c,
+  //   group 0 loads W(c+1) into the other stage          (last read in phase 2c - 1, needed in phase 2c + 2),
+  //   group 1 loads X[2-3](c+1) into the other stage     (last read in phase 2c - 1, needed in phase 2c + 3)
+  //           and X[0-1](c+2) into the stage it reads    (last read in phase 2c,     needed in phase 2c + 4),
+  // and each wave waits for its own loads at the end of the compute phase that follows: every load has a whole
+  // phase to land, and with everything kept the two groups issue the same number (8 per wave).
+  // Measured against this arrangement and slower: loads in front of or between the fragment reads; loads issued by
+  // the computing wave, between its MFMAs (+27 % on the dense product: a load holds its wave for 50-60 clocks) or
+  // behind them (+12 % dense, nothing gained at p = 0.5).  Every instruction of the memory phase costs its wave four
+  // clocks or more, so the loads are kept to one branch per group and six instructions each: the same loads issued
+  // from a per-load choice between the groups' code (a few branches and a dozen scalar instructions more per load)
+  // cost 20 % of the kernel.
+  constexpr bool PINGPONG = IMPLICIT == 0 && !RAGGED && RW == 2 && S::RH == 2 && S::NS == 4 && NT == 2;
+  if constexpr (PINGPONG) {
+    const bool grp1 = __builtin_amdgcn_readfirstlane(rh) != 0;
+    const int wg = wave_u & 3;  // the wave inside its group
+    // per-lane byte offsets of the wave's direct loads (group 0: W tile, group 1: X tiles).  A load fills 1 KB of LDS in
+    // lane order; which chunk of which tile row a lane fetches depends on the load's index only through the swizzle bits
+    // that index reaches, so a few variants serve all loads and the rest of the address is wave-uniform.
+    constexpr int NV = TRANS ? 4 : 2;
+    uint32_t ld_off[NV];
+    if (!TRANS) {
+      // 8 tile rows of 128 B per load; lane -> (row lane/8, physical chunk lane%8); bit 2 of the swizzle is the load's parity
+      const int lr = lane / 8, pch = lane % 8;
+      const int64_t ld = grp1 ? g.a.sr : g.b.sr;
+#pragma unroll
+      for (int v = 0; v < NV; ++v) ld_off[v] = (uint32_t)(lr * ld + ((pch ^ (((lr >> 1) & 3) | (v << 2))) * 8)) * 2u;
+    } else if (!grp1) {
+      // W tile rows are reduction rows of 2*BN bytes, two per load: row = 2i + lane/32; swz_w needs row&3 and bit 3
+      const int lr = lane / 32, pch = lane % 32;
+#pragma unroll
+      for (int v = 0; v < NV; ++v) {
+        int c = pch ^ swz_w(2 * (v & 1) + lr + 8 * (v >> 1));
+        if (c * 8 >= nvalid) c = 0;  // past N: fetch something readable, those columns are never stored
+        ld_off[v] = (uint32_t)(lr * g.b.sc + c * 8) * 2u;
+      }
+    } else {
+      // X tile rows are reduction rows of 128 B, eight per load: row = 8i + lane/8; swz_x needs bit 1 and bit 3
+      const int lr = lane / 8, pch = lane % 8;
+#pragma unroll
+      for (int v = 0; v < NV; ++v) ld_off[v] = (uint32_t)(lr * g.a.sc + ((pch ^ swz_x(lr + 8 * (v & 1))) * 8)) * 2u;
+    }
+    const int64_t w_step = (TRANS ? 2 * g.b.sc : 8 * g.b.sr) * 2;  // bytes between the rows of consecutive W loads
+    const int64_t x_step = (TRANS ? 8 * g.a.sc : 8 * g.a.sr) * 2;  // ... X loads
+    const char* b_wave0 = b_tile0 + wg * 8 * w_step;
+    const char* a_wave0 = a_tile0 + wg * 2 * x_step;
+    auto load_w = [&](uint32_t entry, int stage) {  // the W tile of a step: 32 loads, 8 per wave of group 0
+      const char* bp = b_wave0 + step_block(entry) * b_red_stride;
+      const uint32_t dst = smem_a + (uint32_t)(stage * STAGE + wg * 8 * 1024);
+#pragma unroll
+      for (int jj = 0; jj < 8; ++jj) {
+        if (!TRANS) {  // tile rows are columns of C: those past N are not fetched (whole loads, N is a multiple of 64)
+          if ((wg * 8 + jj) * 8 < nvalid) load16_to_lds(bp + jj * w_step, ld_off[jj & 1], dst + (uint32_t)(jj * 1024));
+        } else {
+          load16_to_lds(bp + jj * w_step, ld_off[(jj & 1) | (((jj >> 2) & 1) << 1)], dst + (uint32_t)(jj * 1024));
+        }
+      }
+    };
+    auto load_x = [&](uint32_t entry, int stage, int r0) {  // the kept X tiles of row blocks r0, r0 + 1: 2 loads per wave and tile
+      const uint32_t fl = step_flags(entry);
+      const char* ap = a_wave0 + step_block(entry) * red_stride;
+      const uint32_t dst = smem_a + (uint32_t)(stage * STAGE + A_OFF + wg * 2 * 1024);
+#pragma unroll
+      for (int rr = 0; rr < 2; ++rr)
+        if (row_quads(fl, r0 + rr)) {
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            load16_to_lds(ap + (r0 + rr) * a_rstride + j * x_step, ld_off[j], dst + (uint32_t)((r0 + rr) * TILE + j * 1024));
+        }
+    };
+    u32x4 af[2][2][4];  // [row block of the wave][kk][16-row tile]
+    u32x4 bf[NT16][2];
+    if (nsteps > 0) {
+      uint32_t e0 = uniform(step_e[0]), e1 = uniform(step_e[1]), e2 = uniform(step_e[2]);
+      issue_loads(e0, 0);
+      if (nsteps > 1) issue_loads(e1, 1, false, 0x3u);  // X[0-1](1): nobody's memory phase comes early enough for it
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if (grp1) __syncthreads();  // phase 0 belongs to group 0
+      for (int step = 0; step < nsteps; ++step) {
+        const int stage = step & 1;
+        const uint32_t e3 = step_e[step + 3];  // a VGPR until the end of the step
+        const uint32_t m = (row_quads(step_flags(e0), 2 * rh) ? 1u : 0u) | (row_quads(step_flags(e0), 2 * rh + 1) ? 2u : 0u);
+        // ---- memory phase.  The reads stay in code common to both groups (under a branch per group the compiler
+        // keeps two sets of fragment registers and spills); the loads, which define no registers, follow in one
+        // branch per group.
+        const char* st = smem + stage * STAGE;
+        if (m) {
+          read_b(st, 0, bf);
+          read_b(st, 1, bf);
+        }
+        if (m & 1u) {
+          read_a(st + A_OFF + (2 * rh) * TILE, 0, af[0][0]);
+          read_a(st + A_OFF + (2 * rh) * TILE, 1, af[0][1]);
+        }
+        if (m & 2u) {
+          read_a(st + A_OFF + (2 * rh + 1) * TILE, 0, af[1][0]);
+          read_a(st + A_OFF + (2 * rh + 1) * TILE, 1, af[1][1]);
+        }
+        if (!grp1) {
+          if (step + 1 < nsteps) load_w(e1, stage ^ 1);
+        } else {
+          if (step + 1 < nsteps) load_x(e1, stage ^ 1, 2);
+          if (step + 2 < nsteps) load_x(e2, stage, 0);
+        }
+        __syncthreads();
+        // ---- compute phase
+        __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+        for (int rr = 0; rr < 2; ++rr)
+          if (m & (1u << rr)) {
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+              for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < NT16; ++nt) acc[rr][mt][nt] = T::mfma16(af[rr][kk][mt], bf[nt][kk], acc[rr][mt][nt]);
+          }
+        __builtin_amdgcn_s_setprio(0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's loads have landed
+        if (!(grp1 && step + 1 == nsteps)) __syncthreads();  // (group 1's last compute phase is nobody's memory phase)
+        e0 = e1;
+        e1 = e2;
+        e2 = uniform(e3);
+      }
+    }
+  } else if constexpr (IMPLICIT == 0) {
     // The products that read their operands from memory run the units of all steps as one chain: the barrier
     // that publishes the next stage stands in front of the MFMAs of a step's LAST unit, not behind them.  By
     // then the wave holds every fragment it needs from the current stage in registers (the barrier's own wait
