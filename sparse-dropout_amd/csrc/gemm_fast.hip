@@ -1423,9 +1423,321 @@ __device__ __forceinline__ void sdd_body(const GemmArgs& g, int tiles_m, int gma
   }
 }
 
+// ---- SDD on aligned operands, 4 row blocks per workgroup: the two waves of a SIMD in opposite phases -----------------
+// The step loop of the DSD kernel (memory phase: the wave's loads, then every fragment of the step; compute phase:
+// MFMAs only; the second group of four waves one phase behind the first) carried over to the output-sparse product.
+// For a step's fragments to fit in registers the two tiles of a wave must share an operand, so a wave owns ONE column
+// block of the group and up to two of its kept tiles: the W fragments of the column (32 registers) serve both, the dY
+// fragments of its one or two row blocks take 32 each.  A column block with 3 or 4 kept tiles takes two waves, and all
+// waves of a column block are in one group of four (so that a W tile is read by one group only: the dY tiles are to
+// this kernel what the W tile is to the DSD kernel, and the W tiles what the X tiles are).  Groups of column blocks are
+// formed greedily along the row: a column block goes to the group of waves with more waves to spare, and the
+// workgroup's group ends in front of the column block that fits neither, or after 6 (the LDS holds 4 + 6 tiles per
+// stage).  Everything kept: 4 column blocks, 16 tiles, as before; at p = 0.5 about 6 column blocks and 12-13 tiles.
+// Group 0 loads the dY tiles of the next step; group 1 its own W tiles of the next step and group 0's of the step
+// after next (the DSD kernel's reasoning, see there).  Measured and slower at every drop rate but 0.5 (where it gains
+// 1 %): letting a column block's two waves sit in different groups (13 instead of 10.5 tiles per group at p = 0.5)
+// with the W loads shared out evenly between the groups - what a step costs is the instructions of its memory
+// phase, and the fuller groups need more of them per wave.
+template <typename T>
+__device__ __forceinline__ void sdd_pp_body(const GemmArgs& g, int tiles_m, int gmax, int Mb, int Cb, const int bid) {
+  using G = SddBig;
+  constexpr int R = G::R, GW = G::GW, G_BOFF = G::BOFF, G_STAGE = G::STAGE;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const uint32_t smem_a = lds_address(smem);
+  uint32_t* flags = reinterpret_cast<uint32_t*>(smem);                   // bit r: tile (row block rb0 + r, column block c) kept
+  int* rec = reinterpret_cast<int*>(smem + 4 * ((Cb + 3) & ~3));        // c_lo, c_hi, ncols, group-1 slots, cols[6], waves[8]
+
+  int tm, gi;
+  tile_of_block<SDD_GROUP_M>(bid, tiles_m, gmax, tm, gi);
+  const int tid = threadIdx.x;
+  const int lane = tid % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  const int rb0 = tm * R;
+
+  // ---- per-column keep flags of this row quad -------------------------------------------------------
+  {
+    const int rows = (rb0 + R <= Mb) ? R : Mb - rb0;
+    const uint32_t init = g.row_ptr ? 0u : ((1u << rows) - 1u);
+    for (int i = tid; i < Cb; i += THREADS) flags[i] = init;
+    if (tid < 32) rec[tid] = 0;
+  }
+  __syncthreads();
+  if (g.row_ptr) {
+    for (int r = 0; r < R; ++r) {
+      if (rb0 + r >= Mb) break;
+      const int beg = g.row_ptr[rb0 + r], end = g.row_ptr[rb0 + r + 1];
+      for (int i = beg + tid; i < end; i += THREADS) atomicOr(&flags[entry_block(g.col_idx[i])], 1u << r);
+    }
+    __syncthreads();
+  }
+
+  // ---- the group this workgroup was launched for: (window, index inside it), as in the other SDD kernel -----------
+  if (wave == 0) {
+    const int nwin = Cb / G::WINDOW > 1 ? Cb / G::WINDOW : 1;
+    const int win = gi / G::GPW < nwin - 1 ? gi / G::GPW : nwin - 1, want = gi - win * G::GPW;
+    const int w_lo = win * G::WINDOW, w_hi = win == nwin - 1 ? Cb : w_lo + G::WINDOW;
+    int lo = -1, hi = -1;
+    if (w_hi - w_lo <= 64) {
+      const uint32_t fv = (w_lo + lane < w_hi) ? flags[w_lo + lane] : 0u;
+      int grp = 0, start = w_lo, used0 = 0, used1 = 0, slots = 0;
+      for (int i = 0; i < w_hi - w_lo; ++i) {
+        const uint32_t f = (uint32_t)__builtin_amdgcn_readlane((int)fv, i) & 0xfu;
+        if (f == 0) continue;
+        const int w = (__builtin_popcount(f) + 1) / 2;  // waves the column block takes
+        int gsel = used0 <= used1 ? 0 : 1;
+        if (4 - (gsel ? used1 : used0) < w) gsel ^= 1;
+        if (slots == GW || 4 - (gsel ? used1 : used0) < w) {  // the group ends in front of this column block
+          if (grp == want) {
+            lo = start;
+            hi = w_lo + i;
+            break;
+          }
+          ++grp;
+          start = w_lo + i;
+          used0 = used1 = slots = 0;
+          gsel = 0;
+        }
+        if (gsel) used1 += w; else used0 += w;
+        ++slots;
+      }
+      if (hi < 0 && grp == want) {  // the window's last group runs to its end
+        lo = start;
+        hi = w_hi;
+      }
+    }
+    // slots, groups and waves of the group's column blocks (the same choices again)
+    int n = 0, used0 = 0, used1 = 0;
+    uint32_t g1_slots = 0, rowmask = 0;
+    for (int c = lo; c < hi; ++c) {
+      const uint32_t f = (uint32_t)__builtin_amdgcn_readfirstlane((int)flags[c]) & 0xfu;
+      if (!f) continue;
+      const int cnt = __builtin_popcount(f), w = (cnt + 1) / 2;
+      int gsel = used0 <= used1 ? 0 : 1;
+      if (4 - (gsel ? used1 : used0) < w) gsel ^= 1;
+      const int wv = 4 * gsel + (gsel ? used1 : used0);
+      uint32_t m = f;
+      const int r_a = __builtin_ctz(m); m &= m - 1u;
+      const int r_b = m ? __builtin_ctz(m) : 0; if (m) m &= m - 1u;
+      const int r_c = m ? __builtin_ctz(m) : 0; if (m) m &= m - 1u;
+      const int r_d = m ? __builtin_ctz(m) : 0;
+      if (lane == 0) {
+        rec[4 + n] = c;
+        rec[10 + wv] = n | (r_a << 4) | (r_b << 8) | ((cnt >= 2 ? 2 : 1) << 12);
+        if (w == 2) rec[10 + wv + 1] = n | (r_c << 4) | (r_d << 8) | ((cnt - 2) << 12);
+      }
+      if (gsel) { used1 += w; g1_slots |= 1u << n; } else used0 += w;
+      rowmask |= f;
+      ++n;
+    }
+    if (lane == 0) {
+      rec[0] = lo;
+      rec[1] = hi;
+      rec[2] = n;
+      rec[3] = (int)(g1_slots | (rowmask << 8));
+    }
+  }
+  __syncthreads();
+  const int c_lo = __builtin_amdgcn_readfirstlane(rec[0]);
+  const int c_hi = __builtin_amdgcn_readfirstlane(rec[1]);
+  if (c_lo < 0) return;  // fewer groups in this row quad than the grid provides for
+  const int ncols = __builtin_amdgcn_readfirstlane(rec[2]);
+  const uint32_t g1_slots = (uint32_t)__builtin_amdgcn_readfirstlane(rec[3]) & 0xffu;
+  const uint32_t rowmask = ((uint32_t)__builtin_amdgcn_readfirstlane(rec[3]) >> 8) & 0xfu;
+  int cols[GW];
+#pragma unroll
+  for (int j = 0; j < GW; ++j) cols[j] = __builtin_amdgcn_readfirstlane(rec[4 + j]);
+  const uint32_t mine = (uint32_t)__builtin_amdgcn_readfirstlane(rec[10 + wave]);
+  const int my_j = (int)(mine & 0xfu), n_mine = (int)((mine >> 12) & 3u);
+  const int my_r[2] = {(int)((mine >> 4) & 0xfu), (int)((mine >> 8) & 0xfu)};
+  const int my_c = __builtin_amdgcn_readfirstlane(rec[4 + my_j]);
+
+  // ---- zeros for the dropped tiles of the group's column range ----------------------------------------
+  if (!g.kept_only) {
+    const int row = tid / 8, ch = tid % 8;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    for (int c = c_lo; c < c_hi; ++c) {
+      const uint32_t f = (uint32_t)__builtin_amdgcn_readfirstlane((int)flags[c]);
+      for (int r = 0; r < R; ++r) {
+        if (rb0 + r >= Mb) break;
+        if (!((f >> r) & 1u) && (int64_t)(rb0 + r) * BS + row < g.M)
+          *reinterpret_cast<u32x4*>(g.c + ((int64_t)(rb0 + r) * BS + row) * g.c_sr + (int64_t)c * BS + ch * 8) = z;
+      }
+    }
+  }
+  if (ncols == 0) return;
+  __syncthreads();  // flags and rec are dead: the stages may be written
+
+  // ---- per-lane constants -----------------------------------------------------------------------------
+  int a_off[2], b_off[2];
+  {
+    const int fr_sw = (lane >> 1) & 7;
+    const int b4 = lane / 16, e = (lane % 16) / 4, j = lane % 4;
+    const int row = 8 * b4 + e;
+    const int b_ch = (j / 2) ^ swz_x(row);
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      a_off[kk] = (lane % 16) * 128 + ((4 * kk + lane / 16) ^ fr_sw) * 16;  // + 16*128 per 16-row tile
+      b_off[kk] = (32 * kk + row) * 128 + b_ch * 16 + (j % 2) * 8;           // ^ 32 per 16-column tile
+    }
+  }
+  const int nsteps = (int)(g.K / BS);
+  const bool grp1 = wave >= 4;
+  const int wg = wave & 3;
+  const int m_valid = (int)(g.M % BS);
+  const int r_tail = m_valid ? Mb - 1 - rb0 : -1;  // rows of the last row block past M are fetched from its last valid row
+  // per-lane offsets of the wave's loads: the two 8-row pieces (wg*2, wg*2 + 1) of a tile; group 0 loads dY tiles
+  // (rows of 128 B along the reduction), group 1 W tiles (reduction rows of 128 B along the columns)
+  uint32_t ld_off[2], ld_off_m[2];
+#pragma unroll
+  for (int v = 0; v < 2; ++v) {
+    const int lr = lane / 8, pch = lane % 8, row = (wg * 2 + v) * 8 + lr;
+    if (!grp1) {
+      const int c = pch ^ ((row >> 1) & 7);
+      const int rc = (r_tail >= 0 && row >= m_valid) ? m_valid - 1 : row;
+      ld_off[v] = (uint32_t)(row * g.a.sr + c * 8) * 2u;
+      ld_off_m[v] = (uint32_t)(rc * g.a.sr + c * 8) * 2u;
+    } else {
+      ld_off[v] = ld_off_m[v] = (uint32_t)(row * g.b.sc + (pch ^ swz_x(row)) * 8) * 2u;
+    }
+  }
+  const char* a_base = reinterpret_cast<const char*>(g.a.ptr + (int64_t)rb0 * BS * g.a.sr);
+  const char* b_base = reinterpret_cast<const char*>(g.b.ptr);
+  const int64_t a_tile_stride = (int64_t)BS * g.a.sr * 2;
+  const int64_t b_step_stride = (int64_t)BS * g.b.sc * 2;
+  const uint32_t my_dst = smem_a + (uint32_t)(wg * 2 * 1024);
+  auto load_dy = [&](int step, int stage) {  // group 0: its two loads of every dY tile in use
+    const char* ap = a_base + step * (BS * 2);
+    const uint32_t dst = my_dst + (uint32_t)(stage * G_STAGE);
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (rowmask & (1u << r)) {
+        load16_to_lds(ap + r * a_tile_stride, r == r_tail ? ld_off_m[0] : ld_off[0], dst + (uint32_t)(r * TILE));
+        load16_to_lds(ap + r * a_tile_stride, r == r_tail ? ld_off_m[1] : ld_off[1], dst + (uint32_t)(r * TILE) + 1024u);
+      }
+  };
+  auto load_w = [&](int step, int stage, uint32_t slots) {  // group 1: its two loads of the W tiles in `slots`
+    const char* bp = b_base + step * b_step_stride;
+    const uint32_t dst = my_dst + (uint32_t)(stage * G_STAGE + G_BOFF);
+#pragma unroll
+    for (int j = 0; j < GW; ++j)
+      if (slots & (1u << j)) {
+        load16_to_lds(bp + (int64_t)cols[j] * (BS * 2), ld_off[0], dst + (uint32_t)(j * TILE));
+        load16_to_lds(bp + (int64_t)cols[j] * (BS * 2), ld_off[1], dst + (uint32_t)(j * TILE) + 1024u);
+      }
+  };
+  const uint32_t all_slots = (1u << ncols) - 1u, g0_slots = all_slots & ~g1_slots;
+
+  f32x4 acc[2][4][4];  // [tile of the wave][16-row tile][16-column tile]
+#pragma unroll
+  for (int k = 0; k < 2; ++k)
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[k][a][b][v] = 0.f;
+  u32x4 af[2][2][4];  // [tile][kk][16-row tile]
+  u32x4 bf[2][4];     // [kk][16-column tile]
+
+  // prologue: step 0 whole, and group 0's W tiles of step 1 (nobody's memory phase comes early enough for them);
+  // here every wave loads its eighth of every tile
+  {
+    const int row = wave * 8 + lane / 8, pch = lane % 8;
+    const int rc = (r_tail >= 0 && row >= m_valid) ? m_valid - 1 : row;
+    const uint32_t a_lane = (uint32_t)(row * g.a.sr + (pch ^ ((row >> 1) & 7)) * 8) * 2u;
+    const uint32_t a_lane_m = (uint32_t)(rc * g.a.sr + (pch ^ ((row >> 1) & 7)) * 8) * 2u;
+    const uint32_t b_lane = (uint32_t)(row * g.b.sc + (pch ^ swz_x(row)) * 8) * 2u;
+    const uint32_t dst = smem_a + (uint32_t)(wave * 1024);
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (rowmask & (1u << r)) load16_to_lds(a_base + r * a_tile_stride, r == r_tail ? a_lane_m : a_lane, dst + (uint32_t)(r * TILE));
+#pragma unroll
+    for (int j = 0; j < GW; ++j) {
+      if (all_slots & (1u << j)) load16_to_lds(b_base + (int64_t)cols[j] * (BS * 2), b_lane, dst + (uint32_t)(G_BOFF + j * TILE));
+      if (nsteps > 1 && (g0_slots & (1u << j)))
+        load16_to_lds(b_base + b_step_stride + (int64_t)cols[j] * (BS * 2), b_lane, dst + (uint32_t)(G_STAGE + G_BOFF + j * TILE));
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (grp1) __syncthreads();  // phase 0 belongs to group 0
+  for (int step = 0; step < nsteps; ++step) {
+    const int stage = step & 1;
+    // ---- memory phase
+    if (!grp1) {
+      if (step + 1 < nsteps) load_dy(step + 1, stage ^ 1);
+    } else {
+      if (step + 1 < nsteps) load_w(step + 1, stage ^ 1, g1_slots);
+      if (step + 2 < nsteps) load_w(step + 2, stage, g0_slots);
+    }
+    const char* st = smem + stage * G_STAGE;
+    if (n_mine > 0) {
+      const char* bt = st + G_BOFF + my_j * TILE;
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+          const char* p = bt + (b_off[kk] ^ (h * 32));
+          const u32x2 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * 128);
+          bf[kk][h] = u32x4{lo.x, lo.y, hi.x, hi.y};
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 2; ++k)
+      if (k < n_mine) {
+        const char* at = st + my_r[k] * TILE;
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+          for (int h = 0; h < 4; ++h) af[k][kk][h] = *reinterpret_cast<const u32x4*>(at + a_off[kk] + h * 16 * 128);
+      }
+    __syncthreads();
+    // ---- compute phase
+    __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+    for (int k = 0; k < 2; ++k)
+      if (k < n_mine) {
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+          for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt) acc[k][mt][nt] = T::mfma16(af[k][kk][mt], bf[kk][nt], acc[k][mt][nt]);
+      }
+    __builtin_amdgcn_s_setprio(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's loads have landed
+    if (!(grp1 && step + 1 == nsteps)) __syncthreads();  // (group 1's last compute phase is nobody's memory phase)
+  }
+
+  // ---- epilogue: as in the other SDD kernel.  Group 0 gets here while group 1 still computes its last step, which
+  // reads no LDS any more.
+  constexpr int S_PITCH = BS + 4;
+  float* stg = reinterpret_cast<float*>(smem) + wave * (BS * S_PITCH);
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    if (k >= n_mine) continue;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int v = 0; v < 4; ++v)  // register v of lane l is element (4*(l/16) + v, l%16) of the 16 x 16 tile
+          stg[(mt * 16 + 4 * (lane / 16) + v) * S_PITCH + nt * 16 + lane % 16] = acc[k][mt][nt][v];
+    store_staged_tile<T, true, BS, BS>(g, stg, lane, true, (int64_t)(rb0 + my_r[k]) * BS, (int64_t)my_c * BS, nullptr);
+  }
+}
+
+template <typename T, bool EDGE, typename G>
+__device__ __forceinline__ void sdd_any_body(const GemmArgs& g, int tiles_m, int gmax, int Mb, int Cb, const int bid) {
+  // aligned operands on the 4-row-block shape: the kernel whose waves alternate between memory and compute phases
+  if constexpr (!EDGE && G::R == 4) sdd_pp_body<T>(g, tiles_m, gmax, Mb, Cb, bid);
+  else sdd_body<T, EDGE, G>(g, tiles_m, gmax, Mb, Cb, bid);
+}
+
 template <typename T, bool EDGE, typename G>
 __global__ __launch_bounds__(THREADS) void sdd_group_kernel(GemmArgs g, int tiles_m, int gmax, int Mb, int Cb) {
-  sdd_body<T, EDGE, G>(g, tiles_m, gmax, Mb, Cb, (int)blockIdx.x);
+  sdd_any_body<T, EDGE, G>(g, tiles_m, gmax, Mb, Cb, (int)blockIdx.x);
 }
 
 // Both gradients of one layer in one launch: workgroups [0, n_dx) are the SDD product's (dX; those past its own
@@ -1441,7 +1753,7 @@ __global__ __launch_bounds__(THREADS) void backward_pair_kernel(GemmArgs gx, int
   static_assert(S::THREADS == THREADS, "both products run on 512 threads");
   const int bid = (int)blockIdx.x;
   if (bid < n_dx) {
-    if (bid < x_tiles_m * x_gmax) sdd_body<T, EDGE, G>(gx, x_tiles_m, x_gmax, x_Mb, x_Cb, bid);
+    if (bid < x_tiles_m * x_gmax) sdd_any_body<T, EDGE, G>(gx, x_tiles_m, x_gmax, x_Mb, x_Cb, bid);
   } else {
     // the weight gradient's workgroups, tile index fastest, then the part of a split reduction
     const int wb = bid - n_dx, w_tiles = w_tiles_m * w_tiles_n;
