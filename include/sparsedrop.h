@@ -225,7 +225,11 @@ int sd_gemm_sdd(const void* A, int64_t a_stride_r, int64_t a_stride_c,
  * the 64-granular block grid must fit the array, i.e. about 2^18 mask blocks (a 32768 x 32768 operand at block
  * size 64); larger operands return SD_ERR_INVALID and launch nothing.  Nothing in the array has to start at
  * zero (the list builder writes every entry the product reads), but all calls on one GPU share it: calls that
- * overlap on one GPU (two streams, two host threads) race on the list and must be serialised by the caller. */
+ * overlap on one GPU (two streams, two host threads) race on the list and must be serialised by the caller.
+ * First use: the first call on a device looks the array's address up and raises the LDS limit of the kernels it
+ * launches (runtime calls that are not stream operations), so a caller that captures a graph makes one call with the
+ * same shapes and block size on that device BEFORE the capture begins; every later call, captured or not, issues
+ * nothing but kernel launches on `stream`. */
 #define SD_NOALLOC_SCRATCH_BYTES 1114112 /* 16-byte padded row_ptr of up to 16383 row blocks + 2^18 int32 */
 int64_t sd_noalloc_scratch_bytes(void);
 int sd_gemm_dsd_noalloc(const void* A, int64_t a_stride_r, int64_t a_stride_c,

@@ -333,11 +333,13 @@ def mlp_forward_backward(x, weights, masks, block_size: int, p: float, act: str 
     nothing is rounded.  (It matters for ReLU: a rounding upstream moves pre-activations near zero across the
     kink, which a comparison must not count as an error of the products.)"""
     rnd = (lambda a: a) if hidden_dtype is None else (lambda a: a.astype(hidden_dtype).astype(np.float64))
+    ps = [float(p)] * len(weights) if np.isscalar(p) else [float(v) for v in p]  # one drop rate, or one per layer
+    assert len(ps) == len(weights)
     h = np.asarray(x, dtype=np.float64)
     inputs, pres = [], []
     for i, (w, m) in enumerate(zip(weights, masks)):
         inputs.append(h)
-        pre = dsd_forward(h, np.asarray(w, dtype=np.float64), m, block_size, p, np.float64)
+        pre = dsd_forward(h, np.asarray(w, dtype=np.float64), m, block_size, ps[i], np.float64)
         if i + 1 < len(weights):
             pres.append(rnd(pre))
             h = rnd(act_apply(pre, act))
@@ -349,8 +351,8 @@ def mlp_forward_backward(x, weights, masks, block_size: int, p: float, act: str 
     dws = [None] * len(weights)
     for i in reversed(range(len(weights))):
         w = np.asarray(weights[i], dtype=np.float64)
-        dws[i] = dsd_dw(g, inputs[i], masks[i], block_size, p, np.float64).astype(dtype)
-        g = sdd_dx(g, w, masks[i], block_size, p, np.float64)
+        dws[i] = dsd_dw(g, inputs[i], masks[i], block_size, ps[i], np.float64).astype(dtype)
+        g = sdd_dx(g, w, masks[i], block_size, ps[i], np.float64)
         if i > 0:
             # ReLU's derivative can be read off either tensor (same sign); GELU's is evaluated at the stored
             # pre-activation

@@ -1,6 +1,6 @@
 """Whole-model forward + backward time as the drop rate varies (reference: benchmark/model.py:119-229).
 
-    python -m benchmark.model --model mlp mlp-784 vit-ffn --p 0 0.1 0.3 0.5 0.7
+    python -m benchmark.model --model mlp mlp-784 vit-ffn gpt-ffn --p 0 0.1 0.3 0.5 0.7
 
 Models are built from ``DropoutMM`` the way the reference's evaluation models are:
   mlp      flattened 32x32 images -> [hidden]*layers -> 10 classes padded to 128, ReLU between, dropout on
@@ -8,6 +8,8 @@ Models are built from ``DropoutMM`` the way the reference's evaluation models ar
   mlp-784  the same on 4096 unresized 28x28 images with 10 unpadded classes: 784 -> 1024 -> 1024 -> 10
   vit-ffn  one transformer feed-forward block on 64x256 tokens: 384 -> 1536 -> GELU -> 384, dropout on the
            inputs of both linears
+  gpt-ffn  the feed-forward block of the reference's GPT (benchmark/model.py:96-112: n_embed 1024, context 128,
+           batch 32; eval/llm/model.py:58-66: 1024 -> 4096 -> GELU -> 1024) on its 32x128 = 4096 tokens
 Each is timed with variant "none" (dense), "vanilla" (element dropout + dense), "blockwise[hip]" and
 "blockwise[hip-fused]": the same layers as one autograd function whose GEMM stores apply the activation and
 its derivative (no activation kernels in either direction)."""
@@ -73,6 +75,8 @@ def fused_variant(name, p, block_size):
         return FusedStack([1024, 1024, 1024, 128], [0.0, p, p], "relu", block_size)
     if name == "mlp-784":
         return FusedStack([784, 1024, 1024, 10], [0.0, p, p], "relu", block_size)
+    if name == "gpt-ffn":
+        return FusedStack([1024, 4096, 1024], [p, p], "gelu", block_size)
     return FusedStack([384, 1536, 384], [p, p], "gelu", block_size)
 
 
@@ -84,7 +88,15 @@ class Mlp784(Mlp):
         super().__init__(variant, p, block_size, in_dim=784, hidden=1024, layers=2, classes=10)
 
 
+class GptFfn(VitFfn):
+    """The feed-forward block of the reference's GPT configuration: 1024 -> 4096 -> GELU -> 1024."""
+
+    def __init__(self, variant, p, block_size):
+        super().__init__(variant, p, block_size, dim=1024, hidden=4096)
+
+
 MODELS = {
+    "gpt-ffn": (GptFfn, lambda: torch.randn(32, 128, 1024)),
     "mlp": (Mlp, lambda: torch.rand(1024, 1, 32, 32)),
     "mlp-784": (Mlp784, lambda: torch.rand(4096, 1, 28, 28)),
     "vit-ffn": (VitFfn, lambda: torch.randn(64, 256, 384)),

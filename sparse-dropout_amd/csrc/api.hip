@@ -351,16 +351,19 @@ int sd_gemm_act(const void* A, int64_t asr, int64_t asc, const void* B, int64_t 
                 int64_t pre_stride_r, int64_t pre_stride_c, void* workspace, int64_t workspace_bytes, void* stream) {
   if (int rc = check_common(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, dtype)) return rc;
   if (int rc = check_act(act, pre_out, pre_stride_r, pre_stride_c, M, N, false)) return rc;
-  // row-major A with a reduction-strided B is the operand layout of the input gradient: the kernel that takes it
-  // multiplies by an activation's derivative in its store, it does not apply one
-  SD_REQUIRE(act == SD_ACT_NONE || !(asc == 1 && bsr == 1 && bsc != 1 && csc == 1),
-             "gemm_act: an activation needs B with a contiguous reduction index (the forward layout)");
   GemmArgs g = make_args(A, asr, asc, B, bsr, bsc, C, csr, csc, M, N, K, 0, 1.0f, nullptr, nullptr,
                          workspace, workspace_bytes);
   g.act = act;
   g.aux = act != SD_ACT_NONE ? static_cast<uint16_t*>(pre_out) : nullptr;
   g.aux_sr = pre_stride_r;
   g.aux_sc = pre_stride_c;
+  // Row-major A with a reduction-strided B (a weight given as a transposed view) is the operand layout of the input
+  // gradient: the specialised kernel that takes it multiplies by an activation's derivative in its store, it does
+  // not apply one.  With an activation that layout runs on the generic kernel, whose store applies it.
+  if (act != SD_ACT_NONE && asc == 1 && bsr == 1 && bsc != 1 && csc == 1) {
+    last_kernel = "generic";
+    return launch_generic(g, kDense, dtype, (hipStream_t)stream);
+  }
   return run(g, kDense, dtype, (hipStream_t)stream);
 }
 

@@ -12,16 +12,18 @@
 // so every SIMD sees exactly (#kept row blocks) x 64x64x64 of MFMA work per step whatever the mask
 // looks like: dropped blocks cost neither loads nor MFMAs and no wave idles behind a barrier.
 //
-// Global->LDS goes through global_load_lds_dwordx4 (no VGPR staging), two stages, one barrier per
-// step.  That barrier stands in front of the MFMAs of a step's last (row block, half of the K block) unit,
-// when every fragment of the current stage is in registers: the loads of the step after next and the
-// fragment reads of the next step's first unit are issued behind it and run under those MFMAs, so no wave
-// starts a step by waiting for LDS.  Timed with parts of the loop compiled out (benchmark/decompose.py; 8192^3,
-// dense, all-zero operands): MFMAs + barriers alone 527 us, + fragment reads 643, + tile loads 802, everything 831, and
-// the tile loads + fragment reads without the MFMAs 808 - the parts add up instead of overlapping, because a wave that
-// stands at a load or a fragment read (the texture path takes a 1 KB load every 25 clocks or so, the LDS a 1 KB read
-// every 8) issues no MFMA behind it, and the data side alone is the floor.  Staging the tiles through registers
-// (global_load_dwordx4 + ds_write_b128) moves them no faster, dealing loads and reads out between the MFMAs loses.
+// Global->LDS goes through global_load_lds_dwordx4 (no VGPR staging), two stages.  Two step loops:
+//  * aligned operands on the 256 x 256 shape (what the large products run on): the two waves of a SIMD work in
+//    opposite phases - one reads fragments and issues loads while the other issues nothing but MFMAs - with a
+//    barrier per phase; see "the step loop of the 256 x 256 shape" in dsd_body.  A wave that stands at a load or a
+//    fragment read (the texture path takes a 1 KB load every 25 clocks or so) issues no MFMA behind it, so with both
+//    waves of a SIMD in the same phase the parts of a step add up instead of overlapping.
+//  * ragged operands, masks of block size 32 and the 128 x 128 shape: one barrier per step, in front of the MFMAs of
+//    the step's last (row block, half of the K block) unit, when every fragment of the current stage is in
+//    registers; the loads of the step after next and the fragment reads of the next step's first unit are issued
+//    behind it and run under those MFMAs.
+// Staging the tiles through registers (global_load_dwordx4 + ds_write_b128) moves them no faster; dealing loads and
+// reads out between the MFMAs of one wave loses.
 // A tile row is 128 B (64 halfs) and its 16-byte chunks are XOR-swizzled with (row>>1)&7,
 // which makes the MFMA fragment reads (ds_read_b128, 16 rows x one chunk per 16-lane group) hit all
 // 64 LDS banks; the swizzle is applied on the global side (which chunk a lane fetches), because the
@@ -699,10 +701,11 @@ __device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int til
   // behind them (+12 % dense, nothing gained at p = 0.5).  Every instruction of the memory phase costs its wave four
   // clocks or more, so the loads are kept to one branch per group and six instructions each: the same loads issued
   // from a per-load choice between the groups' code (a few branches and a dozen scalar instructions more per load)
-  // cost 20 % of the kernel.
+  // cost 20 % of the kernel; the same loads as buffer loads with a scalar offset (three instructions each) gain nothing.
   constexpr bool PINGPONG = IMPLICIT == 0 && !RAGGED && RW == 2 && S::RH == 2 && S::NS == 4 && NT == 2;
   if constexpr (PINGPONG) {
-    const bool grp1 = __builtin_amdgcn_readfirstlane(rh) != 0;
+    const int rh_u = __builtin_amdgcn_readfirstlane(rh);
+    const bool grp1 = rh_u != 0;
     const int wg = wave_u & 3;  // the wave inside its group
     // per-lane byte offsets of the wave's direct loads (group 0: W tile, group 1: X tiles).  A load fills 1 KB of LDS in
     // lane order; which chunk of which tile row a lane fetches depends on the load's index only through the swizzle bits
@@ -737,14 +740,12 @@ __device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int til
     auto load_w = [&](uint32_t entry, int stage) {  // the W tile of a step: 32 loads, 8 per wave of group 0
       const char* bp = b_wave0 + step_block(entry) * b_red_stride;
       const uint32_t dst = smem_a + (uint32_t)(stage * STAGE + wg * 8 * 1024);
+      // tile rows are columns of C: a wave's 64 are all inside the matrix or all past N (N is a multiple of 64).  One test
+      // for all eight loads: a test per load puts every load behind two taken branches (3 % of the kernel).
+      if (!TRANS && wg * 64 >= nvalid) return;
 #pragma unroll
-      for (int jj = 0; jj < 8; ++jj) {
-        if (!TRANS) {  // tile rows are columns of C: those past N are not fetched (whole loads, N is a multiple of 64)
-          if ((wg * 8 + jj) * 8 < nvalid) load16_to_lds(bp + jj * w_step, ld_off[jj & 1], dst + (uint32_t)(jj * 1024));
-        } else {
-          load16_to_lds(bp + jj * w_step, ld_off[(jj & 1) | (((jj >> 2) & 1) << 1)], dst + (uint32_t)(jj * 1024));
-        }
-      }
+      for (int jj = 0; jj < 8; ++jj)
+        load16_to_lds(bp + jj * w_step, ld_off[TRANS ? ((jj & 1) | (((jj >> 2) & 1) << 1)) : (jj & 1)], dst + (uint32_t)(jj * 1024));
     };
     auto load_x = [&](uint32_t entry, int stage, int r0) {  // the kept X tiles of row blocks r0, r0 + 1: 2 loads per wave and tile
       const uint32_t fl = step_flags(entry);
@@ -770,7 +771,9 @@ __device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int til
       for (int step = 0; step < nsteps; ++step) {
         const int stage = step & 1;
         const uint32_t e3 = step_e[step + 3];  // a VGPR until the end of the step
-        const uint32_t m = (row_quads(step_flags(e0), 2 * rh) ? 1u : 0u) | (row_quads(step_flags(e0), 2 * rh + 1) ? 2u : 0u);
+        // which of the wave's two row blocks keep this K block: wave-uniform, in a scalar register (2-3 % against
+        // per-lane conditions)
+        const uint32_t m = (row_quads(step_flags(e0), 2 * rh_u) ? 1u : 0u) | (row_quads(step_flags(e0), 2 * rh_u + 1) ? 2u : 0u);
         // ---- memory phase.  The loads go first (they then have the rest of this phase and the whole compute phase to
         // land: 3 % faster than behind the reads), in one branch per group; the reads stay in code common to both
         // groups (under a branch per group the compiler keeps two sets of fragment registers and spills).
@@ -838,12 +841,8 @@ __device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int til
     auto boundary = [&](int step, int stage, uint32_t e_nx, uint32_t e_nn, bool defer_loads = false) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's loads for the next step have landed
       __syncthreads();
-#ifndef SD_TIMING_NO_LOADS
       if (step + 2 < nsteps && !defer_loads) issue_loads(uniform(e_nn), stage);
-#endif
-#ifndef SD_TIMING_NO_READS
       if (step + 1 < nsteps) first_reads(e_nx, stage ^ 1);
-#endif
     };
     auto units = [&](auto mine_c, int step, int stage, uint32_t e_nx, uint32_t e_nn, bool red_tail,
                      uint32_t quads) {
@@ -857,11 +856,9 @@ __device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int til
       for (int u = 0; u < NR * 2; ++u) {
         const int rr = R0 + u / 2, kk = u % 2;
         if (u + 1 < NR * 2) {
-#ifndef SD_TIMING_NO_READS
           const int kk1 = (u + 1) % 2;
           if (u + 1 < 2) read_b(st, kk1, bf);
           read_a(at0 + ((u + 1) / 2) * TILE, kk1, af[(u + 1) & 1]);
-#endif
         } else {
           boundary(step, stage, e_nx, e_nn, DEFER && late);
         }
@@ -884,17 +881,11 @@ __device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int til
         for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
           for (int nt = 0; nt < NT16; ++nt)
-#ifdef SD_TIMING_NO_MFMA
-            acc[rr][mt][nt][0] += __builtin_bit_cast(float, af[u & 1][mt].x ^ bf[nt][kk].x);
-#else
             acc[rr][mt][nt] = T::mfma16(af[u & 1][mt], bf[nt][kk], acc[rr][mt][nt]);
-#endif
         __builtin_amdgcn_sched_barrier(0);
         // with both row blocks at work the second wave of each SIMD issues its loads behind the last MFMAs: the two
         // waves then run a little out of step, which the dense product gains 3-5 % from
-#ifndef SD_TIMING_NO_LOADS
         if (DEFER && u + 1 == NR * 2 && late && step + 2 < nsteps) issue_loads(uniform(e_nn), stage);
-#endif
       }
     };
 
@@ -903,10 +894,6 @@ __device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int til
     __syncthreads();
     if (nsteps > 1) issue_loads(e_next, 1);
     if (nsteps > 0) first_reads(e_cur, 0);
-#ifdef SD_TIMING_NO_READS
-    read_b(smem, 1, bf);  // fragments are read once, here, and never again
-    read_a(smem + A_OFF, 1, af[1]);
-#endif
     for (int step = 0; step < nsteps; ++step) {
       const int stage = step & 1;
       const uint32_t e_after = step_e[step + 2];  // a VGPR until the boundary makes it uniform

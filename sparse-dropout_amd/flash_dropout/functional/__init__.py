@@ -7,6 +7,7 @@ from .blockwise_dropout_mlp_hip import blockwise_dropout_mlp as hip_blockwise_dr
 from .im2col_conv2d import (
     blockwise_dropout_conv2d,
     blockwise_dropout_conv2d_mask,
+    conv_last_routes,
     conv_patch_matrix_shape,
     im2col_conv2d,
     naive_blockwise_dropout_conv2d,

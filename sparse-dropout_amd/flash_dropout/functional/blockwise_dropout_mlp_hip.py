@@ -89,7 +89,12 @@ class BlockwiseDropoutMLPHIP(torch.autograd.Function):
             if lists is None:  # the dense first layer: only its weight gradient is wanted, dW = g^T . h
                 if need_w:
                     if w.shape[0] % 8:
-                        grads_w[i] = g.t().mm(hs[i])
+                        # the library's kernels take gradients whose width is a multiple of 8 (the 16 bytes of a
+                        # lane's load): zero columns up to the next one, as the dropout layers' narrow heads do
+                        n8 = -(-w.shape[0] // 8) * 8
+                        gp = g.new_zeros(g.shape[0], n8)
+                        gp[:, : w.shape[0]] = g
+                        grads_w[i] = ext.gemm(gp.t(), hs[i].t())[: w.shape[0]]
                     else:
                         grads_w[i] = ext.gemm(g.t(), hs[i].t())
                 break
@@ -116,7 +121,12 @@ def blockwise_dropout_mlp(input: torch.Tensor, weights, block_size, p, activatio
     probability p (a number, or one per layer; 0 keeps everything) and scales by 1/(1-p), ``activation``
     ("relu", "gelu" or None) sits between consecutive layers, none after the last.  ``masks`` (one bool mask per
     layer, True = dropped) pins the masks, ``seed`` pins the draws (layer i uses seed + i); otherwise they come
-    from the device-resident generator.  ``input`` is [M, K], ``weights[i]`` is [out_i, in_i]."""
+    from the device-resident generator.  ``input`` is [M, K], ``weights[i]`` is [out_i, in_i].
+
+    With the device-resident generator a first layer with p = 0 whose input needs no gradient draws nothing (it runs as
+    a dense product): the following layers then use the generator's draws 0, 1, ...; when the input does require a
+    gradient that layer draws its (all kept) mask as well and the others use the draws 1, 2, ....  Results are valid
+    either way; pass ``seed`` or ``masks`` where a run must not depend on it."""
     weights = list(weights)
     if not weights:
         raise ValueError("at least one layer is needed")

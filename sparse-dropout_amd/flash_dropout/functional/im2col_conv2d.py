@@ -26,6 +26,28 @@ IMPLICIT_FORWARD = True
 # Use the one-launch input gradient (sd_conv2d_dx) where the library takes the geometry.
 FUSED_INPUT_GRADIENT = True
 
+# Which route each product of the calling process's last convolution took: "implicit" / "fused" (no patch matrix in
+# memory: sd_conv2d_dsd_lists, sd_conv2d_dw_lists, sd_conv2d_dx) or "explicit" (im2col / col2im around the GEMMs, taken
+# when the library does not take the geometry or a switch above is off).  Read it with conv_last_routes().
+_last_routes = {"forward": None, "dx": None, "dw": None}
+
+
+def conv_last_routes() -> dict:
+    """{"forward": ..., "dx": ..., "dw": ...} of the last convolution run through this module ("implicit", "fused" or
+    "explicit"; None for a product that was not computed): nothing falls back to the patch matrix unseen."""
+    return dict(_last_routes)
+
+
+def _mask_on_64_grid(mask: torch.Tensor, block_size: int, rows: int, cols: int) -> torch.Tensor:
+    """A mask at a block size that is a multiple of 64 as the mask of the same elements at block size 64 (every
+    entry repeated, cropped to the 64 grid of a rows x cols matrix)."""
+    f = block_size // 64
+    if f == 1:
+        return mask
+    m = mask.repeat_interleave(f, 0).repeat_interleave(f, 1)
+    return m[: ceil(rows / 64), : ceil(cols / 64)].contiguous()
+
+
 
 def _pair(v) -> tuple[int, int]:
     if isinstance(v, int):
@@ -60,6 +82,7 @@ class _Im2colConv2d(torch.autograd.Function):
             y2 = ext.conv2d_dsd_lists(input, w2, lists, kernel_bs, 1.0 / (1.0 - p), (r, s), padding, stride,
                                       dilation) if IMPLICIT_FORWARD else None
             ctx.implicit = y2 is not None
+            _last_routes.update(forward="implicit" if ctx.implicit else "explicit", dx=None, dw=None)
             if y2 is None:
                 cols = ext.im2col(input, (r, s), padding, stride, dilation, lists, kernel_bs)
                 y2 = ext.gemm_dsd_lists(cols, w2, lists, kernel_bs, 1.0 / (1.0 - p))
@@ -70,6 +93,7 @@ class _Im2colConv2d(torch.autograd.Function):
             y2 = ext.conv2d_dsd_lists(input, w2, None, 0, 1.0, (r, s), padding, stride,
                                       dilation) if IMPLICIT_FORWARD else None
             ctx.implicit = y2 is not None
+            _last_routes.update(forward="implicit" if ctx.implicit else "explicit", dx=None, dw=None)
             if y2 is None:
                 cols = ext.im2col(input, (r, s), padding, stride, dilation)
                 y2 = ext.gemm(cols, w2)
@@ -92,9 +116,11 @@ class _Im2colConv2d(torch.autograd.Function):
             lists = KeptLists(saved[3], saved[4], saved[5], saved[6], ctx.list_shape)
             scale = 1.0 / (1.0 - p)
             if ctx.needs_input_grad[0]:
-                if FUSED_INPUT_GRADIENT and block_size == 64:
-                    dx = ext.conv2d_dx(dy2, w2, x_shape, (r, s), padding, stride, dilation, mask, block_size, scale,
-                                       ch_last)
+                if FUSED_INPUT_GRADIENT and block_size % 64 == 0:
+                    # the kernel works on 64 x 64 blocks: a mask at a larger multiple of 64 is the same element mask
+                    m64 = _mask_on_64_grid(mask, block_size, dy2.shape[0], w2.shape[1])
+                    dx = ext.conv2d_dx(dy2, w2, x_shape, (r, s), padding, stride, dilation, m64, 64, scale, ch_last)
+                _last_routes["dx"] = "fused" if dx is not None else "explicit"
                 if dx is None:
                     # col2im skips the dropped blocks, so the SDD need not zero them
                     dcols = ext.gemm_sdd_lists(dy2, w2.t(), lists, kernel_bs, scale, kept_only=True,
@@ -105,6 +131,7 @@ class _Im2colConv2d(torch.autograd.Function):
                     dk = ext.conv2d_dw_lists(cols, dy2, lists, kernel_bs, scale, (r, s), padding, stride, dilation)
                     if dk is None:  # gather the kept blocks now
                         cols = ext.im2col(cols, (r, s), padding, stride, dilation, lists, kernel_bs)
+                _last_routes["dw"] = "implicit" if dk is not None else "explicit"
                 if dk is None:
                     dk = ext.gemm_dsd_lists(cols.t(), dy2.t(), lists.transposed(), kernel_bs, scale,
                                             transposed_out=True).t()
@@ -113,6 +140,7 @@ class _Im2colConv2d(torch.autograd.Function):
             if ctx.needs_input_grad[0]:
                 if FUSED_INPUT_GRADIENT:
                     dx = ext.conv2d_dx(dy2, w2, x_shape, (r, s), padding, stride, dilation, channels_last=ch_last)
+                _last_routes["dx"] = "fused" if dx is not None else "explicit"
                 if dx is None:
                     dcols = ext.gemm(dy2, w2.t())
                     dx = ext.col2im(dcols, x_shape, (r, s), padding, stride, dilation, channels_last=ch_last)
@@ -121,6 +149,7 @@ class _Im2colConv2d(torch.autograd.Function):
                     dk = ext.conv2d_dw_lists(cols, dy2, None, 0, 1.0, (r, s), padding, stride, dilation)
                     if dk is None:
                         cols = ext.im2col(cols, (r, s), padding, stride, dilation)
+                _last_routes["dw"] = "implicit" if dk is not None else "explicit"
                 if dk is None:
                     dk = ext.gemm(cols.t(), dy2.t(), transposed_out=True).t()
                 dk = dk.reshape(k_shape)

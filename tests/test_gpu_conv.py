@@ -412,6 +412,8 @@ def test_full_size_conv_config_against_the_full_oracle():
     xg, kg = x.cuda().requires_grad_(), k.cuda().requires_grad_()
     y = F.blockwise_dropout_conv2d_mask(xg, mask.cuda(), 64, 0.5, kg, **geo)
     y.backward(dy.cuda())
+    # none of the three products went through a patch matrix
+    assert F.conv_last_routes() == {"forward": "implicit", "dx": "fused", "dw": "implicit"}
     ry, rdx, rdk = O.conv2d_blockdrop(to_np(x), to_np(k), mask.numpy(), 64, 0.5, dy=to_np(dy), dtype=np.float32, **geo)
     # in the products' own layouts, so that a tile of the check is a tile of the kernels
     as_rows = lambda t: t.permute(0, 2, 3, 1).reshape(-1, t.shape[1])
@@ -424,3 +426,45 @@ def test_full_size_conv_config_against_the_full_oracle():
     lhs = (cols.double() * g.double()).sum().item()
     rhs = (xs.double() * ext.col2im(g, xs.shape, (3, 3), **geo).double()).sum().item()
     assert abs(lhs - rhs) <= 2e-3 * max(abs(lhs), (cols.double().norm() * g.double().norm()).item() * 1e-2)
+
+
+@pytest.mark.parametrize("bs,dx_route", [(64, "fused"), (128, "fused"), (192, "fused")])
+def test_conv_routes_are_reported_and_block_sizes_above_64_stay_fused(bs, dx_route):
+    """Which route a convolution's products took is visible (conv_last_routes), a geometry the fused kernels do not take
+    reports the patch-matrix route, and masks at block sizes 128 and 192 run the fused input gradient too (as the
+    mask of the same elements at block size 64): results against the oracle at that block size."""
+    import sys
+
+    import flash_dropout.functional as F
+
+    mod = sys.modules["flash_dropout.functional.im2col_conv2d"]  # the package re-exports a function of that name
+
+    gen = torch.Generator().manual_seed(12)
+    geo = dict(padding=(1, 1), stride=(1, 1), dilation=(1, 1))
+    x = torch.randn(8, 64, 32, 32, generator=gen).half()
+    k = ((torch.rand(128, 64, 3, 3, generator=gen) * 2 - 1) * 576 ** -0.5).half()
+    dy = torch.randn(8, 128, 32, 32, generator=gen).half()
+    mask = cpu_mask(O.mask_shape(8 * 32 * 32, 576, bs), 0.5, gen)
+    xg, kg = x.cuda().requires_grad_(), k.cuda().requires_grad_()
+    y = F.blockwise_dropout_conv2d_mask(xg, mask.cuda(), bs, 0.5, kg, **geo)
+    y.backward(dy.cuda())
+    assert F.conv_last_routes() == {"forward": "implicit", "dx": dx_route, "dw": "implicit"}
+    ry, rdx, rdk = O.conv2d_blockdrop(to_np(x), to_np(k), mask.numpy(), bs, 0.5, dy=to_np(dy), dtype=np.float32, **geo)
+    assert max_tile_rel_fro(y, ry) <= REL_FRO_TOL
+    assert max_tile_rel_fro(xg.grad, rdx) <= REL_FRO_TOL
+    assert max_tile_rel_fro(kg.grad, rdk) <= REL_FRO_TOL
+    if bs == 64:
+        # Q = 18 is a geometry none of the fused kernels takes; and the switches force the patch-matrix route
+        x2 = torch.randn(2, 16, 16, 16, generator=gen).half().cuda().requires_grad_()
+        k2 = (torch.randn(64, 16, 3, 3, generator=gen) * 144 ** -0.5).half().cuda().requires_grad_()
+        F.im2col_conv2d(x2, k2, padding=(2, 2)).sum().backward()
+        assert F.conv_last_routes() == {"forward": "explicit", "dx": "explicit", "dw": "explicit"}
+        old = mod.IMPLICIT_FORWARD, mod.FUSED_INPUT_GRADIENT
+        try:
+            mod.IMPLICIT_FORWARD = mod.FUSED_INPUT_GRADIENT = False
+            xg.grad = kg.grad = None
+            F.blockwise_dropout_conv2d_mask(xg, mask.cuda(), bs, 0.5, kg, **geo).backward(dy.cuda())
+            assert F.conv_last_routes() == {"forward": "explicit", "dx": "explicit", "dw": "explicit"}
+            assert max_tile_rel_fro(xg.grad, rdx) <= REL_FRO_TOL
+        finally:
+            mod.IMPLICIT_FORWARD, mod.FUSED_INPUT_GRADIENT = old

@@ -399,6 +399,35 @@ def test_both_gradients_in_one_launch_match_the_two_launches(M, K, N, bs, dtype,
         assert max_tile_rel_fro(dw, O.dsd_dw(to_np(dy), to_np(x), mask.numpy(), bs, p, np.float32)) <= REL_FRO_TOL
 
 
+@pytest.mark.parametrize("N,single", [(8192, True), (8448, False)])
+def test_single_launch_forward_and_backward_at_the_workgroup_limit_against_the_oracle(N, single):
+    """The forward that builds its lists in the same launch and the backward that runs both gradients in one are
+    taken up to 512 workgroups per product.  4096 x 4096 x 8192 is the largest square-ish layer under that limit
+    (16 x 32 = 512 tiles of 256 x 256 for the forward and for the weight gradient), N = 8448 the first over it: both
+    sides of the switch, every 64 x 64 tile of Y, dX and dW against the fp32 oracle."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(41)
+    M, K, bs, p = 4096, 4096, 64, 0.5
+    x = torch.randn(M, K, generator=gen).half().cuda()
+    w = (torch.randn(N, K, generator=gen) * K ** -0.5).half().cuda()
+    dy = torch.randn(M, N, generator=gen).half().cuda()
+    mask = cpu_mask(O.mask_shape(M, K, bs), p, gen)
+    y, m, lists, g = ext.dropout_matmul_forward(x, w, bs, p, mask=mask.cuda())
+    assert ext.last_kernel_detail().startswith("dsd+lists:") == single, ext.last_kernel_detail()
+    dx, dw = ext.dropout_matmul_backward(dy, w, x, lists, g, p)
+    assert ext.last_kernel_detail().startswith("pair:") == single, ext.last_kernel_detail()
+    xn, wn, dyn, mk = to_np(x), to_np(w), to_np(dy), mask.numpy()
+    for got, ref, what in ((y, O.dsd_forward(xn, wn, mk, bs, p, np.float32), "y"),
+                           (dx, O.sdd_dx(dyn, wn, mk, bs, p, np.float32), "dx"),
+                           (dw, O.dsd_dw(dyn, xn, mk, bs, p, np.float32), "dw")):
+        err = max_tile_rel_fro(got, ref)
+        assert err <= REL_FRO_TOL, f"{what}: largest per-tile relative Frobenius error {err:.3e}"
+    keep = O.expand_keep(mk, bs, M, K)
+    assert (dx.cpu().numpy()[~keep] == 0).all(), "dropped dX tiles must be exactly zero"
+
+
 @pytest.mark.parametrize("act", ["relu", "gelu"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_fused_activation_products_against_the_oracle(act, dtype):
@@ -512,7 +541,39 @@ def test_dense_product_with_fused_activation_and_the_stack_that_starts_with_one(
         assert a.shape == b.shape and rel_fro(a, b.float()) <= 1e-3
 
 
-@pytest.mark.parametrize("name", ["mlp", "mlp-784", "vit-ffn"])
+@pytest.mark.parametrize("act", ["relu", "gelu"])
+def test_dense_first_layer_takes_a_transposed_weight_view_and_a_narrow_output(act):
+    """The fused MLP's dense first layer (p = 0, input without gradient) with its weight given as a transposed view (the
+    operand layout of the input gradient: the activation then runs on the generic kernel's store), and a one-layer
+    stack whose output width is not a multiple of 8 (its weight gradient goes through zero-padded columns, inside
+    the library): both against the oracle."""
+    import flash_dropout.functional as F
+
+    gen = torch.Generator().manual_seed(37)
+    rows, dims = 384, [200, 320, 72]
+    x = torch.randn(rows, dims[0], generator=gen).half()
+    w0 = (torch.randn(dims[0], dims[1], generator=gen) * dims[0] ** -0.5).half()   # stored [in, out]: used as w0.t()
+    w1 = (torch.randn(dims[2], dims[1], generator=gen) * dims[1] ** -0.5).half()
+    dy = torch.randn(rows, dims[2], generator=gen).half()
+    seed = 5
+    w0g, w1g = w0.cuda().requires_grad_(), w1.cuda().requires_grad_()
+    out = F.hip_blockwise_dropout_mlp(x.cuda(), [w0g.t(), w1g], 64, [0.0, 0.5], act, seed=seed)
+    out.backward(dy.cuda())
+    masks = [np.zeros(O.mask_shape(rows, dims[0], 64), dtype=bool), O.random_mask(O.mask_shape(rows, dims[1], 64), 0.5, seed + 1)]
+    ry, _, rdw = O.mlp_forward_backward(to_np(x), [to_np(w0).T.copy(), to_np(w1)], masks, 64, [0.0, 0.5], act, to_np(dy),
+                                        hidden_dtype=np.float16)
+    assert max_tile_rel_fro(out, ry) <= REL_FRO_TOL
+    assert max_tile_rel_fro(w0g.grad.t(), rdw[0]) <= REL_FRO_TOL
+    assert max_tile_rel_fro(w1g.grad, rdw[1]) <= REL_FRO_TOL
+    # one dense layer, 10 outputs
+    w = (torch.randn(10, dims[0], generator=gen) * dims[0] ** -0.5).half().cuda().requires_grad_()
+    g10 = torch.randn(rows, 10, generator=gen).half()
+    F.hip_blockwise_dropout_mlp(x.cuda(), [w], 64, 0.0, act).backward(g10.cuda())
+    assert w.grad.shape == (10, dims[0])
+    assert max_tile_rel_fro(w.grad, to_np(g10).T @ to_np(x)) <= REL_FRO_TOL
+
+
+@pytest.mark.parametrize("name", ["mlp", "mlp-784", "vit-ffn", "gpt-ffn"])
 def test_model_harness_runs_every_variant(name):
     """benchmark/model.py (the reference's benchmark/model.py:119-229 protocol): every variant of every model
     steps forward and backward, eagerly and as a replayed graph, and the fused stack agrees with the layer-by-layer

@@ -278,11 +278,11 @@ def test_full_size_8192_sampled_against_oracle(p):
         assert rel_fro(dA, ext.gemm(dC, B.T).float()) <= 1e-3
 
 
-@pytest.mark.parametrize("size,p", [(4096, 0.0), (4096, 0.25), (4096, 0.5), (4096, 0.75), (8192, 0.25), (8192, 0.75)])
+@pytest.mark.parametrize("size,p", [(4096, 0.0), (4096, 0.25), (4096, 0.5), (4096, 0.75),
+                                    (8192, 0.0), (8192, 0.25), (8192, 0.5), (8192, 0.75)])
 def test_square_sweep_sizes_against_the_full_oracle(size, p, tile_policy):
-    """The square sweep's larger sizes, every 64 x 64 tile of Y, dX and dW against the fp32 oracle: 4096^3 sits
-    at the boundary between the two workgroup shapes, and at 8192^3 the drop rates 0.25 and 0.75 take the other
-    branch of the SDD group policy than 0 and 0.5 (checked on sampled blocks above)."""
+    """The square sweep's larger sizes at every drop rate of the benchmark, every 64 x 64 tile of Y, dX and dW against
+    the fp32 oracle: 4096^3 sits at the boundary between the two workgroup shapes, 8192^3 is the headline size."""
     if tile_policy != "auto":
         pytest.skip("full-size oracle runs once, under the shape policy the library picks itself")
     M = N = K = size
@@ -300,6 +300,31 @@ def test_square_sweep_sizes_against_the_full_oracle(size, p, tile_policy):
     for got, ref, what in ((C, rC, "C"), (dA, rdA, "dA"), (dB, rdB, "dB")):
         err = max_tile_rel_fro(got, ref)
         assert err <= REL_FRO_TOL, f"{what}: largest per-tile relative Frobenius error {err:.3e}"
+
+
+@pytest.mark.parametrize("dtype,bs", [(torch.bfloat16, 64), (torch.float16, 32), (torch.bfloat16, 32)])
+def test_4096_bf16_and_block_size_32_against_the_full_oracle(dtype, bs, tile_policy):
+    """bf16 and a mask of block size 32 at 4096^3, p = 0.5: every 64 x 64 tile of the three products against the
+    fp32 oracle on the same rounded inputs, dropped 32 x 32 blocks of dX exactly zero."""
+    if tile_policy != "auto":
+        pytest.skip("full-size oracle runs once, under the shape policy the library picks itself")
+    M = N = K = 4096
+    p = 0.5
+    gen = torch.Generator().manual_seed(10)
+    A = make_operand(M, K, dtype, "cuda", gen=gen)
+    B = make_operand(N, K, dtype, "cuda", scale=K ** -0.5, gen=gen)
+    dC = make_operand(M, N, dtype, "cuda", gen=gen)
+    mask = cpu_mask((M // bs, K // bs), p, gen).cuda()
+    C, dA, dB = _three_products(A, B, dC, mask, bs, p)
+    from flash_dropout.hip import GEMM
+
+    assert GEMM().last_kernel() == "specialised"
+    rC, rdA, rdB = _oracle_products(A, B, dC, mask, bs, p)
+    for got, ref, what in ((C, rC, "C"), (dA, rdA, "dA"), (dB, rdB, "dB")):
+        err = max_tile_rel_fro(got, ref, tile=bs)
+        assert err <= REL_FRO_TOL, f"{what}: largest per-tile relative Frobenius error {err:.3e}"
+    keep = O.expand_keep(mask.cpu().numpy(), bs, M, K)
+    assert (dA.float().cpu().numpy()[~keep] == 0).all(), "dropped dX blocks must be exactly zero"
 
 
 def _structured_masks(mb, cb, gen):

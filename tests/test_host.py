@@ -249,7 +249,7 @@ def test_as_matrix_lays_out_expanded_and_strided_views():
     assert _mat(torch.zeros(1, 8))[1:] == (8, 1)
 
 
-@pytest.mark.parametrize("name", ["mfma_ceiling.hip", "lds_load_ceiling.hip", "dense_4wave_probe.hip"])
+@pytest.mark.parametrize("name", ["mfma_ceiling.hip", "lds_load_ceiling.hip"])
 def test_ceiling_probes_compile_for_gfx950(name, tmp_path):
     """The stand-alone measurement programs under benchmark/ are only ever run on a GPU box by hand: keep them
     compiling (device code for gfx950, no GPU needed)."""
@@ -264,15 +264,3 @@ def test_ceiling_probes_compile_for_gfx950(name, tmp_path):
     assert proc.returncode == 0, proc.stderr[-2000:]
 
 
-def test_decompose_switches_exist_in_the_kernel_source():
-    """benchmark/decompose.py builds the GEMM kernels with SD_TIMING_* defined: each switch it passes must still be
-    one the source knows."""
-    import re
-
-    root = Path(__file__).resolve().parent.parent / "sparse-dropout_amd"
-    script = (root / "benchmark" / "decompose.py").read_text()
-    source = (root / "csrc" / "gemm_fast.hip").read_text()
-    switches = set(re.findall(r"-D(SD_TIMING_\w+)", script))
-    assert switches == {"SD_TIMING_NO_LOADS", "SD_TIMING_NO_READS", "SD_TIMING_NO_MFMA"}
-    for name in switches:
-        assert re.search(rf"#if(n?def)? {name}\b", source), name

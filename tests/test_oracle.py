@@ -348,6 +348,23 @@ def test_mlp_chain_rule_vs_autograd_of_the_naive_restatement(act):
     naive_torch.forward(f(x0), ws[1].detach(), masks[1], bs, p).backward(dpre1)
     got = O.sdd_dx_actgrad(dpre1.numpy(), ws[1].detach().numpy(), masks[1].numpy(), bs, p, act, pres[0].detach().numpy())
     np.testing.assert_allclose(got, x0.grad.numpy(), rtol=1e-10, atol=1e-12)
+    # a drop rate per layer (the reference's models start with a layer that drops nothing)
+    ps = [0.0, 0.4, 0.25]
+    pmasks = [torch.rand(m // bs, dims[i] // bs, generator=gen) < ps[i] for i in range(3)]
+    x.grad = None
+    for w in ws:
+        w.grad = None
+    h = x
+    for i in range(3):
+        h = naive_torch.forward(h, ws[i], pmasks[i], bs, ps[i])
+        h = f(h) if i < 2 else h
+    h.backward(dy)
+    out, dx, dws = O.mlp_forward_backward(x.detach().numpy(), [w.detach().numpy() for w in ws],
+                                          [mk.numpy() for mk in pmasks], bs, ps, act, dy.numpy())
+    np.testing.assert_allclose(out, h.detach().numpy(), rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(dx, x.grad.numpy(), rtol=1e-10, atol=1e-12)
+    for got, w in zip(dws, ws):
+        np.testing.assert_allclose(got, w.grad.numpy(), rtol=1e-10, atol=1e-12)
 
 
 @pytest.mark.parametrize("act", ["relu", "gelu"])

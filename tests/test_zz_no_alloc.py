@@ -76,3 +76,31 @@ def test_noalloc_rejects_what_does_not_fit_and_allocates_nothing():
     rc = ext.lib.sd_gemm_dsd_noalloc(A.data_ptr(), big, 1, B.data_ptr(), big, 1, out.data_ptr(), N, 1,
                                      mask.data_ptr(), big // 64, 1, big, N, big, 64, ctypes.c_float(2.0), 0, None)
     assert rc == 1 and b"scratch" in ext.lib.sd_last_error()
+
+
+def test_noalloc_under_graph_capture_after_a_first_call():
+    """What the entry point is for: captured in a HIP graph (after one eager call on the device, which does the
+    one-time symbol lookup and kernel set-up) and replayed on changing inputs, with eager work and synchronisations
+    between the replays; every replay against sd_gemm_dsd on the same inputs."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(23)
+    M, N, K, bs, p = 1024, 384, 768, 64, 0.5
+    A = make_operand(M, K, torch.float16, "cuda", gen=gen)
+    B = make_operand(N, K, torch.float16, "cuda", scale=K ** -0.5, gen=gen)
+    mask = cpu_mask((M // bs, K // bs), p, gen).cuda()
+    out = torch.empty(M, N, dtype=torch.float16, device="cuda")
+    ext.gemm_dsd_noalloc(A, B, mask, bs, 2.0, out)  # first use on this device, outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ext.gemm_dsd_noalloc(A, B, mask, bs, 2.0, out)
+    for rep in range(3):
+        A.copy_(make_operand(M, K, torch.float16, "cuda", gen=gen))          # eager work between the replays
+        mask.copy_(cpu_mask((M // bs, K // bs), p, gen).cuda())
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, ext.gemm_dsd(A, B, mask, bs, 2.0)), rep
