@@ -30,10 +30,11 @@
  *   - Return value: SD_OK, or an error code with the reason in sd_last_error() (thread-local).
  *     Shapes and strides are always validated on the host (the reference only has assert()s,
  *     matmul_dsd.cuh:79-95).  The library allocates no device memory; workspaces are the caller's.
- *   - Supported block sizes: multiples of 64, and 32.  M, N, K are arbitrary (edge tiles are predicated);
- *     the mask has ceil(M/block_size) x ceil(K/block_size) entries.  The kernels work on 64 x 64 tiles: a larger
- *     block size is listed with every mask entry repeated, and 32 with four mask entries merged into one list
- *     entry that remembers which of its 32 x 32 quadrants are kept (the report's block splitting, report.pdf
+ *   - Supported block sizes: multiples of 32.  M, N, K are arbitrary (edge tiles are predicated);
+ *     the mask has ceil(M/block_size) x ceil(K/block_size) entries.  The kernels work on 64 x 64 tiles: a multiple
+ *     of 64 is listed with every mask entry repeated, and an odd multiple of 32 (32, 96, 160, ...) on the grid of its
+ *     32-blocks merged two by two, a list entry remembering which of its 32 x 32 quadrants are kept (the report's
+ *     block splitting, report.pdf
  *     section 3.3, in both directions; the reference's Triton path takes any block size divisible by its tile,
  *     flash_dropout/triton/utils.py:6-19, its CUDA path only 128, matmul_dsd.cuh:92-93).
  */
@@ -123,6 +124,11 @@ int sd_build_lists(const uint8_t* mask, int64_t mb, int64_t kb, int64_t mask_str
  * the entry say which: bit 2a + b = mask entry (2i + a, 2j + b) kept (row_idx, the list by columns, stores them as the
  * list of the transposed mask needs them: halves swapped).  The *_lists entry points take such lists when called with
  * block_size 32: the 64 x 64 tile of a kept entry is computed and its dropped quadrants contribute / come out as zeros.
+ * split == -k (k = 3, 5, ...; -1 is the same as 0): the mask is at block size 32 * k; its entries are repeated k x k
+ * times onto the grid of 32-blocks and that grid is merged two by two as above.  out_mb x out_kb is the grid of
+ * 64-blocks of the masked matrix, ceil(M / 64) x ceil(K / 64): it must end inside the mask's last row and column of
+ * entries, (mb - 1) * k < 2 * out_mb and out_mb <= ceil(mb * k / 2).  A 32-block past the end of the matrix but inside
+ * the mask's last entry counts as kept when that entry is (nothing of it is ever loaded or stored).
  * split >= 1: the same lists for the mask with every entry repeated split x split times, cropped
  * to out_mb x out_kb ((mb-1)*split < out_mb <= mb*split, likewise out_kb); capacities out_mb*out_kb.
  * A mask drawn at block size 64*split over an [M,K] operand is listed with out_mb = ceil(M/64),

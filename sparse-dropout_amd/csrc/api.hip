@@ -62,8 +62,8 @@ int check_common(const void* A, int64_t asr, int64_t asc, const void* B, int64_t
 
 int check_sparse(int64_t bs, float scale) {
   SD_REQUIRE(bs > 0, "block_size must be positive");
-  if (bs % 64 != 0 && bs != 32)
-    return fail(SD_ERR_UNSUPPORTED, "block_size %lld: only 32 and multiples of 64 are supported", (long long)bs);
+  if (bs % 32 != 0)
+    return fail(SD_ERR_UNSUPPORTED, "block_size %lld: only multiples of 32 are supported", (long long)bs);
   SD_REQUIRE(scale == scale, "scale is NaN");
   return SD_OK;
 }
@@ -113,9 +113,10 @@ GemmArgs make_args(const void* A, int64_t asr, int64_t asc, const void* B, int64
   g.M = M;
   g.N = N;
   g.K = K;
-  // block size 32: the lists are on the 64 grid and carry the keep bits of each entry's four 32-blocks
-  g.bs = bs == 32 ? 64 : bs;
-  g.quads = bs == 32;
+  // an odd multiple of 32 (the *_lists calls pass 32 for all of them): the lists are on the 64 grid and carry the
+  // keep bits of each entry's four 32-blocks
+  g.quads = bs % 64 == 32;
+  g.bs = g.quads ? 64 : bs;
   g.scale = scale;
   g.row_ptr = row_ptr;
   g.col_idx = col_idx;
@@ -219,12 +220,15 @@ static int check_list_grid(int64_t mb, int64_t kb, int64_t split, int64_t out_mb
                            const int32_t* row_ptr, const int32_t* col_idx, const int32_t* col_ptr,
                            const int32_t* row_idx) {
   SD_REQUIRE(mb > 0 && kb > 0, "build_lists: mask must be non-empty (got %lld x %lld)", (long long)mb, (long long)kb);
-  SD_REQUIRE(split >= 0 && split < (1 << 16), "build_lists: split must be >= 0 (got %lld)", (long long)split);
-  if (split == 0) {
-    // a mask at half the listed granularity, merged two by two
-    SD_REQUIRE(out_mb == (mb + 1) / 2 && out_kb == (kb + 1) / 2,
-               "build_lists: a %lld x %lld grid does not match a %lld x %lld mask merged two by two", (long long)out_mb,
-               (long long)out_kb, (long long)mb, (long long)kb);
+  SD_REQUIRE(split > -(1 << 16) && split < (1 << 16), "build_lists: split out of range (got %lld)", (long long)split);
+  if (split <= 0) {
+    // a mask at block size 32 * sub listed on the 64 grid: its 32-blocks merged two by two.  The grid must end inside
+    // the mask's last row / column of entries (for sub == 1 that fixes it)
+    const int64_t sub = split ? -split : 1;
+    SD_REQUIRE(2 * out_mb > (mb - 1) * sub && out_mb <= (mb * sub + 1) / 2 && 2 * out_kb > (kb - 1) * sub &&
+                   out_kb <= (kb * sub + 1) / 2,
+               "build_lists: a %lld x %lld grid of 64-blocks does not match a %lld x %lld mask at block size %lld",
+               (long long)out_mb, (long long)out_kb, (long long)mb, (long long)kb, (long long)(32 * sub));
     SD_REQUIRE(out_kb < (1 << 28), "build_lists: merged lists keep four bits of every entry for the quadrants");
   } else {
     // the listed grid is the mask repeated split x split, cropped inside its last row / column of entries
@@ -425,10 +429,11 @@ static int lists_in_workspace(const uint8_t* mask, int64_t msr, int64_t msc, int
   const int64_t mb = ceil_div(rows, *bs), kb = ceil_div(cols, *bs);
   SD_REQUIRE(mb > 0 && kb > 0, "empty mask");
   int64_t split = 1, out_mb = mb, out_kb = kb;
-  if (*bs == 32) {  // listed on the 64 grid with quadrant bits; the *_lists calls are told so by block size 32
-    split = 0;
+  if (*bs % 64 == 32) {  // listed on the 64 grid with quadrant bits; the *_lists calls are told so by block size 32
+    split = -(*bs / 32);
     out_mb = ceil_div(rows, 64);
     out_kb = ceil_div(cols, 64);
+    *bs = 32;
   } else if (*bs > 64 && *bs % 64 == 0 && ceil_div(rows, 64) * ceil_div(cols, 64) < kMaxDim &&
              workspace_bytes >= sd_workspace_bytes(ceil_div(rows, 64), ceil_div(cols, 64))) {
     split = *bs / 64;
@@ -483,7 +488,11 @@ int sd_gemm_sdd(const void* A, int64_t asr, int64_t asc, const void* B, int64_t 
 }
 
 // granularity of the lists the fused calls build and take: 64 for block sizes that are multiples of 64
-static int64_t list_granule(int64_t bs) { return (bs % 64 == 0 || bs == 32) ? 64 : bs; }
+static int64_t list_granule(int64_t bs) { return bs % 32 == 0 ? 64 : bs; }
+// what tells the *_lists calls that the lists carry quadrant bits: block size 32, whatever odd multiple of 32 the mask has
+static int64_t lists_block_size(int64_t bs) { return bs % 64 == 32 ? 32 : list_granule(bs); }
+// the `split` argument of the list builders for a mask at this block size
+static int64_t list_split(int64_t bs) { return bs % 64 == 32 ? -(bs / 32) : bs / list_granule(bs); }
 
 int sd_dropout_matmul_forward(const void* X, int64_t xsr, int64_t xsc, const void* W, int64_t wsr, int64_t wsc,
                               void* Y, int64_t ysr, int64_t ysc, const uint8_t* mask, int64_t msr, int64_t msc,
@@ -518,7 +527,7 @@ int sd_dropout_matmul_forward_act(const void* X, int64_t xsr, int64_t xsc, const
   SD_REQUIRE(M > 0 && K > 0, "dropout_matmul_forward: empty operand");
   SD_REQUIRE(row_ptr && col_idx, "dropout_matmul_forward: the CSR list arrays are required");
   if (int rc = check_act(act, pre_out, pre_stride_r, pre_stride_c, M, N, false)) return rc;
-  const int64_t g = list_granule(bs), split = bs / g;  // 0 for block size 32: merged two by two
+  const int64_t g = list_granule(bs), split = list_split(bs);  // negative for odd multiples of 32: merged two by two
   const int64_t mb = ceil_div(M, bs), kb = ceil_div(K, bs), out_mb = ceil_div(M, g), out_kb = ceil_div(K, g);
   const float scale = (float)(1.0 / (1.0 - p));  // in double, as the reference's Python evaluates it
   // what the list calls below would check, up front: the single launch takes the same arguments
@@ -539,7 +548,7 @@ int sd_dropout_matmul_forward_act(const void* X, int64_t xsr, int64_t xsc, const
   };
   if (N > 0 && !generic_forced() && !separate_forward_forced()) {
     // lists and product in one launch where the pair qualifies (small products, where a launch is a large part)
-    const GemmArgs a = with_act(make_args(X, xsr, xsc, W, wsr, wsc, Y, ysr, ysc, M, N, K, bs == 32 ? 32 : g, scale,
+    const GemmArgs a = with_act(make_args(X, xsr, xsc, W, wsr, wsc, Y, ysr, ysc, M, N, K, lists_block_size(bs), scale,
                                           row_ptr, col_idx, workspace, workspace_bytes));
     const int rc = forward_with_lists(a, mask, msr, msc, seed, offset, rng_state, (float)p, mb, kb, mask_out, split, out_mb,
                                       out_kb, row_ptr, col_idx, col_ptr, row_idx, dtype, (hipStream_t)stream);
@@ -562,7 +571,7 @@ int sd_dropout_matmul_forward_act(const void* X, int64_t xsr, int64_t xsc, const
       return rc;
   }
   if (N == 0) return SD_OK;
-  return sd_gemm_dsd_lists_act(X, xsr, xsc, W, wsr, wsc, Y, ysr, ysc, row_ptr, col_idx, M, N, K, bs == 32 ? 32 : g,
+  return sd_gemm_dsd_lists_act(X, xsr, xsc, W, wsr, wsc, Y, ysr, ysc, row_ptr, col_idx, M, N, K, lists_block_size(bs),
                                scale, dtype, act, pre_out, pre_stride_r, pre_stride_c, workspace, workspace_bytes,
                                stream);
 }
@@ -590,7 +599,7 @@ int sd_dropout_matmul_backward_act(const void* dY, int64_t gsr, int64_t gsc, con
   }
   if (int rc = check_sparse(bs, 1.f)) return rc;
   SD_REQUIRE(dX || dW, "dropout_matmul_backward: nothing to compute");
-  const int64_t g = bs == 32 ? 32 : list_granule(bs);  // 32: lists on the 64 grid with quadrant bits
+  const int64_t g = lists_block_size(bs);  // 32: lists on the 64 grid with quadrant bits
   const float scale = (float)(1.0 / (1.0 - p));  // in double, as the reference's Python evaluates it
   if (dX && dW && row_ptr && col_idx && col_ptr && row_idx && !generic_forced() && !separate_backward_forced()) {
     // both gradients in one launch where the pair qualifies (same operands and checks as the two calls below)

@@ -159,12 +159,13 @@ static int launch_lists(const MaskSrc& src, int64_t mb, int64_t kb, int32_t* row
   return check_launch("build_lists");
 }
 
-// Lists over an mb x kb grid in which every stored mask entry covers split x split grid entries; split == 0: the
-// stored mask is at half the granularity (stored_mb x stored_kb entries) and is merged two by two.
+// Lists over an mb x kb grid in which every stored mask entry covers split x split grid entries; split <= 0: the
+// grid is of 64-blocks and the stored mask (stored_mb x stored_kb entries) is at block size 32 * |split| (0 counts as
+// -1): its 32-blocks are merged two by two, the four keep bits of an entry kept beside it.
 int build_lists(const uint8_t* mask, int64_t msr, int64_t msc, int64_t stored_mb, int64_t stored_kb, int64_t split,
                 int64_t mb, int64_t kb, int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr,
                 int32_t* row_idx, hipStream_t stream) {
-  MaskSrc src{mask, msr, msc, (int32_t)(split ? split : 1), split ? 1 : 2, (int32_t)stored_mb, (int32_t)stored_kb,
+  MaskSrc src{mask, msr, msc, (int32_t)(split > 0 ? split : (split < 0 ? -split : 1)), split > 0 ? 1 : 2, (int32_t)stored_mb, (int32_t)stored_kb,
               0, 0, 0, 0, 0.f, nullptr};
   return launch_lists(src, mb, kb, row_ptr, col_idx, col_ptr, row_idx, nullptr, 0, stream);
 }
@@ -173,7 +174,7 @@ int build_lists(const uint8_t* mask, int64_t msr, int64_t msc, int64_t stored_mb
 int random_lists(uint64_t seed, uint64_t offset, uint64_t* state, float p, int64_t stored_mb, int64_t stored_kb,
                  uint8_t* mask_out, int64_t split, int64_t mb, int64_t kb, int32_t* row_ptr,
                  int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx, hipStream_t stream) {
-  MaskSrc src{nullptr, 0, 0, (int32_t)(split ? split : 1), split ? 1 : 2, (int32_t)stored_mb, (int32_t)stored_kb,
+  MaskSrc src{nullptr, 0, 0, (int32_t)(split > 0 ? split : (split < 0 ? -split : 1)), split > 0 ? 1 : 2, (int32_t)stored_mb, (int32_t)stored_kb,
               (uint32_t)seed, (uint32_t)(seed >> 32), (uint32_t)offset, (uint32_t)(offset >> 32), p, state};
   bool advanced = false;
   if (int rc = launch_lists(src, mb, kb, row_ptr, col_idx, col_ptr, row_idx, mask_out, stored_mb, stream, &advanced))
@@ -189,10 +190,10 @@ int forward_with_lists(const GemmArgs& g, const uint8_t* mask, int64_t msr, int6
                        uint64_t* state, float p, int64_t stored_mb, int64_t stored_kb, uint8_t* mask_out, int64_t split,
                        int64_t mb, int64_t kb, int32_t* row_ptr, int32_t* col_idx, int32_t* col_ptr, int32_t* row_idx,
                        int dtype, hipStream_t stream) {
-  MaskSrc src{mask, msr, msc, (int32_t)(split ? split : 1), split ? 1 : 2, (int32_t)stored_mb, (int32_t)stored_kb,
+  MaskSrc src{mask, msr, msc, (int32_t)(split > 0 ? split : (split < 0 ? -split : 1)), split > 0 ? 1 : 2, (int32_t)stored_mb, (int32_t)stored_kb,
               0, 0, 0, 0, 0.f, nullptr};
   if (mask == nullptr) {
-    src = MaskSrc{nullptr, 0, 0, (int32_t)(split ? split : 1), split ? 1 : 2, (int32_t)stored_mb, (int32_t)stored_kb,
+    src = MaskSrc{nullptr, 0, 0, (int32_t)(split > 0 ? split : (split < 0 ? -split : 1)), split > 0 ? 1 : 2, (int32_t)stored_mb, (int32_t)stored_kb,
                   (uint32_t)seed, (uint32_t)(seed >> 32), (uint32_t)offset, (uint32_t)(offset >> 32), p, state};
   }
   return launch_forward_with_lists(g, src, mb, kb, row_ptr, col_idx, col_ptr, row_idx, mask ? nullptr : mask_out,

@@ -36,9 +36,10 @@ struct Philox {
 // Where "is block (i, j) dropped" comes from: a stored bool mask, or a Bernoulli(p) draw that is a pure
 // function of (seed, offset, entry index), so every reader recomputes the same value and no pass over
 // a stored mask is needed.  Each stored / drawn entry covers split x split entries of the listed grid
-// (a logical block size that is a multiple of the 64 the kernels work in), or, with merge == 2, a quarter of
-// one: a mask at block size 32 is listed on the 64 grid, an entry being kept when any of its four 32-blocks
-// is, with those four keep bits stored in the top bits of its list entry (quad_bits).
+// (a logical block size that is a multiple of the 64 the kernels work in), or, with merge == 2, the listed grid is
+// twice as coarse as a grid of 32-blocks of which every stored entry covers split x split: a mask at block size
+// 32 * split (32, 96, 160, ...) is listed on the 64 grid, an entry being kept when any of its four 32-blocks is, with
+// those four keep bits stored in the top bits of its list entry (quad_bits).
 struct MaskSrc {
   const uint8_t* mask;  // null: drawn
   int64_t st_row, st_col;
@@ -84,7 +85,8 @@ struct MaskSrc {
     for (int a = 0; a < 2; ++a)
 #pragma unroll
       for (int b = 0; b < 2; ++b) {
-        const int32_t si = 2 * i + a, sj = 2 * j + b;
+        // 32-blocks (2i + a, 2j + b); a stored entry covers split x split of them (block size 32 * split)
+        const int32_t si = (2 * i + a) / split, sj = (2 * j + b) / split;
         if (si < mb && sj < kb && !dropped_entry(si, sj)) q |= 1u << (2 * a + b);
       }
     return q;

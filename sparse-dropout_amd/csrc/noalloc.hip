@@ -46,7 +46,7 @@ int sd_gemm_dsd_noalloc(const void* A, int64_t asr, int64_t asc, const void* B, 
                         int64_t N, int64_t K, int64_t bs, float scale, int dtype, void* stream) {
   SD_REQUIRE(M >= 0 && N >= 0 && K >= 0 && bs > 0, "gemm_dsd_noalloc: negative dimension or block size");
   // the list the mask form would build: at 64 granularity when the block size is a larger multiple of 64, or 32
-  const int64_t g = ((bs > 64 && bs % 64 == 0) || bs == 32) ? 64 : bs;
+  const int64_t g = bs % 32 == 0 ? 64 : bs;
   const int64_t mb = sd::ceil_div(M, g), kb = sd::ceil_div(K, g);
   SD_REQUIRE(mb < (1 << 24) && kb < (1 << 24), "gemm_dsd_noalloc: block grid %lld x %lld too large", (long long)mb,
              (long long)kb);

@@ -93,9 +93,9 @@ def _block_size(block_size) -> int:
 
 
 def _list_grid_size(bs: int) -> int:
-    """Edge of the blocks the kept-block lists are over: 64 for a block size of 32 (the lists then carry, in the
+    """Edge of the blocks the kept-block lists are over: 64 for an odd multiple of 32 (the lists then carry, in the
     top four bits of every entry, which of the entry's four 32-blocks are kept), else the block size."""
-    return 64 if bs == 32 else bs
+    return 64 if bs % 64 == 32 else bs
 
 
 def _check_operand(name: str, x: torch.Tensor) -> None:
@@ -252,7 +252,7 @@ class GEMM:
         C = self._out(A, B, out, transposed_out)
         if M == 0 or N == 0:
             return C
-        if (bs > 64 and bs % 64 == 0) or bs == 32:  # the 64-granular list: the library splits / merges the mask
+        if bs > 64 and bs % 32 == 0 or bs == 32:  # the 64-granular list: the library splits / merges the mask
             ws_bytes = self.lib.sd_workspace_bytes(ceil(M / 64), ceil((K if mask_cols == "K" else N) / 64))
         else:
             ws_bytes = self.lib.sd_workspace_bytes(mb, cb)
@@ -294,12 +294,12 @@ class GEMM:
     @staticmethod
     def _list_grid(mb, kb, split, grid):
         split = int(split)
-        if split < 0:
-            raise ValueError(f"split must be >= 0, got {split}")
-        if split == 0:  # a mask of block size 32 merged two by two onto the 64 grid
-            out_mb, out_kb = ((mb + 1) // 2, (kb + 1) // 2) if grid is None else (int(grid[0]), int(grid[1]))
-            if (out_mb, out_kb) != ((mb + 1) // 2, (kb + 1) // 2):
-                raise ValueError(f"grid {(out_mb, out_kb)} does not match a {(mb, kb)} mask merged two by two")
+        if split <= 0:  # a mask of block size 32 * sub: its 32-blocks merged two by two onto the 64 grid
+            sub = -split if split else 1
+            full = ((mb * sub + 1) // 2, (kb * sub + 1) // 2)
+            out_mb, out_kb = full if grid is None else (int(grid[0]), int(grid[1]))
+            if not ((mb - 1) * sub < 2 * out_mb and out_mb <= full[0] and (kb - 1) * sub < 2 * out_kb and out_kb <= full[1]):
+                raise ValueError(f"grid {(out_mb, out_kb)} of 64-blocks does not match a {(mb, kb)} mask at block size {32 * sub}")
             return split, out_mb, out_kb
         out_mb, out_kb = (mb * split, kb * split) if grid is None else (int(grid[0]), int(grid[1]))
         if not ((mb - 1) * split < out_mb <= mb * split and (kb - 1) * split < out_kb <= kb * split):
@@ -409,8 +409,9 @@ class GEMM:
         split, grid, kernel_bs = 1, None, bs
         if bs > 64 and bs % 64 == 0:
             split, grid, kernel_bs = bs // 64, (ceil(rows / 64), ceil(cols / 64)), 64
-        elif bs == 32:  # merged two by two onto the 64 grid; the *_lists calls are told so by block size 32
-            split, grid = 0, (ceil(rows / 64), ceil(cols / 64))
+        elif bs % 64 == 32:  # 32, 96, 160, ...: the 32-blocks merged two by two onto the 64 grid; the *_lists calls
+            # are told so by block size 32
+            split, grid, kernel_bs = -(bs // 32), (ceil(rows / 64), ceil(cols / 64)), 32
         if mask is None:
             mask, lists = self.random_lists(shape, p, seed, 0, device, split, grid)
         else:
@@ -570,7 +571,7 @@ class GEMM:
         if not 0.0 <= p < 1.0:
             raise ValueError(f"p must be in [0, 1), got {p}")
         M, K, N = x.shape[0], x.shape[1], w.shape[0]
-        g = 64 if (bs % 64 == 0 or bs == 32) else bs
+        g = 64 if bs % 32 == 0 else bs
         mb, kb, out_mb, out_kb = ceil(M / bs), ceil(K / bs), ceil(M / g), ceil(K / g)
         if mb == 0 or kb == 0:
             raise ValueError("mask must be non-empty")
@@ -595,7 +596,7 @@ class GEMM:
                        row_idx.data_ptr(), M, N, K, bs, _DTYPES[x.dtype], code,
                        *(_mat(pre) if pre is not None else (None, 0, 0)), ws_ptr, ws_bytes, self._stream(x))
         # block size 32 stays 32 for the backward call: it says that the lists carry quadrant bits
-        return (y, mask, KeptLists(row_ptr, col_idx, col_ptr, row_idx, (out_mb, out_kb)), (32 if bs == 32 else g),
+        return (y, mask, KeptLists(row_ptr, col_idx, col_ptr, row_idx, (out_mb, out_kb)), (32 if bs % 64 == 32 else g),
                 pre if code else (y if want_pre else None))
 
     def dropout_matmul_backward(self, dy: torch.Tensor, w: torch.Tensor, x: torch.Tensor, lists: KeptLists,
@@ -611,7 +612,7 @@ class GEMM:
         M, K, N = x.shape[0], x.shape[1], w.shape[0]
         if tuple(dy.shape) != (M, N) or dy.dtype != x.dtype or dy.device != x.device:
             raise ValueError(f"dy must be a [{M}, {N}] {x.dtype} tensor on {x.device}")
-        g = 64 if (bs % 64 == 0 or bs == 32) else bs
+        g = 64 if bs % 32 == 0 else bs
         if tuple(lists.shape) != (ceil(M / g), ceil(K / g)):
             raise ValueError(f"lists are for a {lists.shape} mask, operands need {(ceil(M / g), ceil(K / g))}")
         if N % 8 and N > 0 and M > 0 and K > 0 and (need_dx or need_dw):

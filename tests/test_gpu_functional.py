@@ -598,9 +598,10 @@ def test_model_harness_runs_every_variant(name):
     assert rel_fro(fused0(x), plain(x).float()) <= 3e-3
 
 
-def test_block_size_32_through_autograd_and_the_fused_mlp():
-    """block_size = 32 end to end: the single layer's autograd function (one library call per direction) and the
-    fused MLP, against the oracle under the masks the library drew."""
+@pytest.mark.parametrize("bs", [32, 96, 160])
+def test_odd_multiples_of_32_through_autograd_and_the_fused_mlp(bs):
+    """block_size = 32, 96, 160 end to end: the single layer's autograd function (one library call per direction)
+    and the fused MLP, against the oracle under the masks the library drew."""
     import flash_dropout.functional as F
     from flash_dropout.hip import GEMM
 
@@ -610,27 +611,27 @@ def test_block_size_32_through_autograd_and_the_fused_mlp():
     w = (torch.randn(N, K, generator=gen) * K ** -0.5).half()
     dy = torch.randn(M, N, generator=gen).half()
     xg, wg = x.cuda().requires_grad_(), w.cuda().requires_grad_()
-    y = F.hip_blockwise_dropout_matmul(xg, wg, 32, p, seed=123)
+    y = F.hip_blockwise_dropout_matmul(xg, wg, bs, p, seed=123)
     y.backward(dy.cuda())
-    mask = O.random_mask(O.mask_shape(M, K, 32), p, 123)
-    assert max_tile_rel_fro(y, O.dsd_forward(to_np(x), to_np(w), mask, 32, p, np.float32), tile=32) <= REL_FRO_TOL
-    assert max_tile_rel_fro(xg.grad, O.sdd_dx(to_np(dy), to_np(w), mask, 32, p, np.float32), tile=32) <= REL_FRO_TOL
-    assert max_tile_rel_fro(wg.grad, O.dsd_dw(to_np(dy), to_np(x), mask, 32, p, np.float32), tile=32) <= REL_FRO_TOL
+    mask = O.random_mask(O.mask_shape(M, K, bs), p, 123)
+    assert max_tile_rel_fro(y, O.dsd_forward(to_np(x), to_np(w), mask, bs, p, np.float32), tile=32) <= REL_FRO_TOL
+    assert max_tile_rel_fro(xg.grad, O.sdd_dx(to_np(dy), to_np(w), mask, bs, p, np.float32), tile=32) <= REL_FRO_TOL
+    assert max_tile_rel_fro(wg.grad, O.dsd_dw(to_np(dy), to_np(x), mask, bs, p, np.float32), tile=32) <= REL_FRO_TOL
     # the mask form that allocates nothing takes it too
     ext = GEMM()
     out = torch.empty(M, N, dtype=torch.float16, device="cuda")
-    ext.gemm_dsd_noalloc(x.cuda(), w.cuda(), torch.from_numpy(mask).cuda(), 32, 1 / (1 - p), out)
+    ext.gemm_dsd_noalloc(x.cuda(), w.cuda(), torch.from_numpy(mask).cuda(), bs, 1 / (1 - p), out)
     assert torch.equal(out, y.detach())
     # fused MLP, ReLU, given masks
     dims = (352, 264, 96)
     ws = [((torch.rand(dims[i + 1], dims[i], generator=gen) * 2 - 1) * dims[i] ** -0.5).half() for i in range(2)]
-    masks = [cpu_mask(O.mask_shape(M, dims[i], 32), p, gen) for i in range(2)]
+    masks = [cpu_mask(O.mask_shape(M, dims[i], bs), p, gen) for i in range(2)]
     dy2 = torch.randn(M, dims[-1], generator=gen).half()
     xg = x.cuda().requires_grad_()
     wgs = [t.cuda().requires_grad_() for t in ws]
-    out = F.hip_blockwise_dropout_mlp(xg, wgs, 32, p, "relu", masks=[m.cuda() for m in masks])
+    out = F.hip_blockwise_dropout_mlp(xg, wgs, bs, p, "relu", masks=[m.cuda() for m in masks])
     out.backward(dy2.cuda())
-    rout, rdx, rdws = O.mlp_forward_backward(to_np(x), [to_np(t) for t in ws], [m.numpy() for m in masks], 32, p,
+    rout, rdx, rdws = O.mlp_forward_backward(to_np(x), [to_np(t) for t in ws], [m.numpy() for m in masks], bs, p,
                                              "relu", to_np(dy2), np.float32, hidden_dtype=np.float16)
     assert max_tile_rel_fro(out, rout, tile=32) <= REL_FRO_TOL
     assert max_tile_rel_fro(xg.grad, rdx, tile=32) <= REL_FRO_TOL

@@ -216,7 +216,7 @@ def test_errors_through_the_shim():
         ext.gemm_dsd(A, A, torch.zeros(1, 2, dtype=torch.bool, device="cuda"), 64, 1.0)
     with pytest.raises(ValueError, match="row or column major"):
         ext.gemm(A[::2, ::2], A[:64, :64])
-    with pytest.raises(NotImplementedError, match="multiples of 64"):
+    with pytest.raises(NotImplementedError, match="multiples of 32"):
         ext.gemm_dsd(A, A, torch.zeros(3, 3, dtype=torch.bool, device="cuda"), 48, 1.0)
     with pytest.raises(ValueError, match="reduction dims"):
         ext.gemm(A, A[:, :64])
@@ -547,3 +547,56 @@ def test_block_size_32_on_ragged_and_model_shapes(M, N, K, p, dtype):
     assert torch.equal(ext.gemm_sdd_lists(dC, B.T, lists, 32, s), dA)
     dBl = ext.gemm_dsd_lists(A.T, dC.T, lists.transposed(), 32, s, transposed_out=True).T
     assert max_tile_rel_fro(dBl, rdB, tile=32) <= REL_FRO_TOL
+
+
+# ---- odd multiples of 32 (96, 160): the mask split to its 32-blocks, those merged onto the kernels' 64 grid ----------
+@pytest.mark.parametrize("mnk,p", list(product(REF_MNKS, REF_PS)))
+@pytest.mark.parametrize("bs", [96, 160])
+def test_reference_grid_at_odd_multiples_of_32(mnk, p, bs, tile_policy):
+    """The reference's shape and drop-rate grid at block sizes 96 and 160, which its Triton path takes (any block size
+    its 32-wide tiles divide, flash_dropout/triton/utils.py:6-19): Y, dX and dW against the oracle at that block size
+    (the shapes are not multiples of it: the mask's last row and column of blocks are cropped), dropped blocks of dX
+    exactly zero."""
+    if tile_policy == "big":
+        pytest.skip("two shape policies are enough here")
+    M, N, K = mnk
+    gen = torch.Generator().manual_seed(24)
+    A = make_operand(M, K, torch.float16, "cuda", gen=gen)
+    B = make_operand(N, K, torch.float16, "cuda", scale=K ** -0.5, gen=gen)
+    dC = make_operand(M, N, torch.float16, "cuda", gen=gen)
+    mask = cpu_mask(O.mask_shape(M, K, bs), p, gen).cuda()
+    C, dA, dB = _three_products(A, B, dC, mask, bs, p)
+    rC, rdA, rdB = _oracle_products(A, B, dC, mask, bs, p)
+    atol = 0.2 * max(1.0, (1 / (1 - p)) / 10)
+    _check(C, rC, "C", atol)
+    _check(dB, rdB, "dB", atol)
+    _check(dA, rdA, "dA", atol)
+    keep = O.expand_keep(mask.cpu().numpy(), bs, M, K)
+    assert (dA.cpu().numpy()[~keep] == 0).all(), "dropped dX blocks must be exactly zero"
+
+
+@pytest.mark.parametrize("M,N,K,bs", [(1000, 136, 200, 96), (100, 70, 50, 96), (4096, 1024, 784, 160), (130, 64, 290, 96),
+                                      (16384, 384, 1536, 224)])
+def test_odd_multiples_of_32_on_ragged_and_model_shapes(M, N, K, bs):
+    """Ragged shapes (against the block size, the 64 grid and the 32 grid), the generic kernel (K = 50) and a model
+    shape: mask forms and list forms of all three products at block sizes 96, 160 and 224."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    p = 0.4
+    gen = torch.Generator().manual_seed(M + K + bs)
+    A = make_operand(M, K, torch.float16, "cuda", gen=gen)
+    B = make_operand(N, K, torch.float16, "cuda", scale=K ** -0.5, gen=gen)
+    dC = make_operand(M, N, torch.float16, "cuda", gen=gen)
+    mk = cpu_mask(O.mask_shape(M, K, bs), p, gen)
+    C, dA, dB = _three_products(A, B, dC, mk.cuda(), bs, p)
+    rC, rdA, rdB = _oracle_products(A, B, dC, mk, bs, p)
+    for got, ref, what in ((C, rC, "C"), (dA, rdA, "dA"), (dB, rdB, "dB")):
+        assert max_tile_rel_fro(got, ref, tile=32) <= REL_FRO_TOL, what
+    keep = O.expand_keep(mk.numpy(), bs, M, K)
+    assert (to_np(dA)[~keep] == 0).all()
+    # the list forms on lists built once: block size 32 tells them that the lists carry quadrant bits
+    lists = ext.build_lists(mk.cuda(), split=-(bs // 32), grid=(-(-M // 64), -(-K // 64)))
+    s = 1 / (1 - p)
+    assert torch.equal(ext.gemm_dsd_lists(A, B, lists, 32, s), C)
+    assert torch.equal(ext.gemm_sdd_lists(dC, B.T, lists, 32, s), dA)

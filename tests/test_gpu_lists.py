@@ -115,3 +115,43 @@ def test_merged_lists_of_a_block_size_32_mask_bit_exact(shape, p):
     rp, ci = O.compact_csr_quads(want)
     assert np.array_equal(lists.row_ptr.cpu().numpy(), rp)
     assert np.array_equal(lists.col_idx[: lists.nnz()].cpu().numpy(), ci)
+
+
+@pytest.mark.parametrize("rows,cols,bs", [(96, 96, 96), (100, 130, 96), (1000, 784, 96), (4096, 4096, 160), (70, 700, 224),
+                                          (8192, 8192, 96)])
+@pytest.mark.parametrize("p", [0.0, 0.5, 0.9])
+def test_merged_lists_of_odd_multiples_of_32_bit_exact(rows, cols, bs, p):
+    """split = -k: a mask at block size 32 * k (96, 160, 224) over a [rows, cols] matrix, listed on the matrix's grid of
+    64-blocks with the quadrant keep bits: against the oracle's composition (every mask entry repeated k x k times onto
+    the grid of 32-blocks, that grid merged two by two), by rows and by columns, for a stored and a drawn mask."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    k = bs // 32
+    shape = O.mask_shape(rows, cols, bs)
+    grid64 = O.mask_shape(rows, cols, 64)
+    gen = torch.Generator().manual_seed(rows + cols + bs)
+    mask = torch.rand(*shape, generator=gen) < p
+
+    def want(m):
+        # the mask's 32-blocks, as far as the 64 grid reaches (a 32-block past the matrix but inside the mask's last
+        # entry keeps that entry's value)
+        m32 = O.split_mask(m, k, (min(shape[0] * k, 2 * grid64[0]), min(shape[1] * k, 2 * grid64[1])))
+        return O.compact_csr_quads(m32), O.compact_csr_quads(m32.T)
+
+    def check(lists, m):
+        (rp, ci), (cp, ri) = want(m)
+        assert lists.shape == grid64
+        assert np.array_equal(lists.row_ptr.cpu().numpy(), rp)
+        assert np.array_equal(lists.col_idx[: lists.nnz()].cpu().numpy(), ci)
+        assert np.array_equal(lists.col_ptr.cpu().numpy(), cp)
+        assert np.array_equal(lists.row_idx[: lists.nnz()].cpu().numpy(), ri)
+
+    check(ext.build_lists(mask.cuda(), split=-k, grid=grid64), mask.numpy())
+    check(ext.build_lists(mask.t().contiguous().cuda().t(), split=-k, grid=grid64), mask.numpy())  # column-major mask
+    drawn, lists = ext.random_lists(shape, p, seed=11, split=-k, grid=grid64)
+    assert np.array_equal(drawn.cpu().numpy(), O.random_mask(shape, p, 11))
+    check(lists, O.random_mask(shape, p, 11))
+    # the element mask is the one of the block size: what makes the composition the right oracle
+    m32 = O.split_mask(mask.numpy(), k, O.mask_shape(rows, cols, 32))
+    assert np.array_equal(O.expand_keep(m32, 32, rows, cols), O.expand_keep(mask.numpy(), bs, rows, cols))

@@ -58,7 +58,7 @@ def test_host_validation_rejects_bad_arguments_without_touching_the_gpu():
     assert rc == 1 and b"row stride" in lib.sd_last_error()
     # unsupported block size
     rc = lib.sd_gemm_dsd_lists(fake, 96, 1, fake, 96, 1, fake, 96, 1, fake, fake, 96, 96, 96, 48, 1.0, 0, None, 0, None)
-    assert rc == 2 and b"multiples of 64" in lib.sd_last_error()
+    assert rc == 2 and b"multiples of 32" in lib.sd_last_error()
     # workspace too small
     rc = lib.sd_gemm_dsd(fake, 128, 1, fake, 128, 1, fake, 128, 1, fake, 2, 1, 128, 128, 128, 64, 2.0, 0, fake, 8, None)
     assert rc == 1 and b"workspace too small" in lib.sd_last_error()
