@@ -773,7 +773,9 @@ __device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int til
         const uint32_t e3 = step_e[step + 3];  // a VGPR until the end of the step
         // which of the wave's two row blocks keep this K block: wave-uniform, in a scalar register (2-3 % against
         // per-lane conditions)
-        const uint32_t m = (row_quads(step_flags(e0), 2 * rh_u) ? 1u : 0u) | (row_quads(step_flags(e0), 2 * rh_u + 1) ? 2u : 0u);
+        // (a mask of block size 32 keeps or drops each 32 x 32 quadrant of a tile: four bits per row block)
+        const uint32_t q_rows[2] = {row_quads(step_flags(e0), 2 * rh_u), row_quads(step_flags(e0), 2 * rh_u + 1)};
+        const uint32_t m = (q_rows[0] ? 1u : 0u) | (q_rows[1] ? 2u : 0u);
         // ---- memory phase.  The loads go first (they then have the rest of this phase and the whole compute phase to
         // land: 3 % faster than behind the reads), in one branch per group; the reads stay in code common to both
         // groups (under a branch per group the compiler keeps two sets of fragment registers and spills).
@@ -800,15 +802,23 @@ __device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int til
         // ---- compute phase
         __builtin_amdgcn_s_setprio(1);
 #pragma unroll
-        for (int rr = 0; rr < 2; ++rr)
-          if (m & (1u << rr)) {
+        for (int rr = 0; rr < 2; ++rr) {
+          const uint32_t q = q_rows[rr];
+          {
+            // some quadrants of the X tile are dropped: quadrant (row half h, reduction half kk) feeds the MFMAs of the
+            // 16-row tiles 2h, 2h + 1 at depth kk and nothing else, so dropping it is leaving those eight out
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-              for (int mt = 0; mt < 4; ++mt)
+              for (int h = 0; h < 2; ++h)
+                if ((q >> (2 * h + kk)) & 1u) {
 #pragma unroll
-                for (int nt = 0; nt < NT16; ++nt) acc[rr][mt][nt] = T::mfma16(af[rr][kk][mt], bf[nt][kk], acc[rr][mt][nt]);
+                  for (int mt = 2 * h; mt < 2 * h + 2; ++mt)
+#pragma unroll
+                    for (int nt = 0; nt < NT16; ++nt) acc[rr][mt][nt] = T::mfma16(af[rr][kk][mt], bf[nt][kk], acc[rr][mt][nt]);
+                }
           }
+        }
         __builtin_amdgcn_s_setprio(0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's loads have landed
         if (!(grp1 && step + 1 == nsteps)) __syncthreads();  // (group 1's last compute phase is nobody's memory phase)
@@ -1432,7 +1442,9 @@ __device__ __forceinline__ void sdd_pp_body(const GemmArgs& g, int tiles_m, int 
   constexpr int R = G::R, GW = G::GW, G_BOFF = G::BOFF, G_STAGE = G::STAGE;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const uint32_t smem_a = lds_address(smem);
-  uint32_t* flags = reinterpret_cast<uint32_t*>(smem);                   // bit r: tile (row block rb0 + r, column block c) kept
+  // bit r: tile (row block rb0 + r, column block c) kept; bits 8 + 4r .. 11 + 4r: which of its four 32 x 32 quadrants
+  // (all of them unless the mask has block size 32)
+  uint32_t* flags = reinterpret_cast<uint32_t*>(smem);
   int* rec = reinterpret_cast<int*>(smem + 4 * ((Cb + 3) & ~3));        // c_lo, c_hi, ncols, group-1 slots, cols[6], waves[8]
 
   int tm, gi;
@@ -1445,7 +1457,7 @@ __device__ __forceinline__ void sdd_pp_body(const GemmArgs& g, int tiles_m, int 
   // ---- per-column keep flags of this row quad -------------------------------------------------------
   {
     const int rows = (rb0 + R <= Mb) ? R : Mb - rb0;
-    const uint32_t init = g.row_ptr ? 0u : ((1u << rows) - 1u);
+    const uint32_t init = g.row_ptr ? 0u : (((1u << rows) - 1u) | (((1u << (4 * rows)) - 1u) << 8));
     for (int i = tid; i < Cb; i += THREADS) flags[i] = init;
     if (tid < 32) rec[tid] = 0;
   }
@@ -1454,7 +1466,10 @@ __device__ __forceinline__ void sdd_pp_body(const GemmArgs& g, int tiles_m, int 
     for (int r = 0; r < R; ++r) {
       if (rb0 + r >= Mb) break;
       const int beg = g.row_ptr[rb0 + r], end = g.row_ptr[rb0 + r + 1];
-      for (int i = beg + tid; i < end; i += THREADS) atomicOr(&flags[entry_block(g.col_idx[i])], 1u << r);
+      for (int i = beg + tid; i < end; i += THREADS) {
+        const int32_t e = g.col_idx[i];
+        atomicOr(&flags[entry_block(e)], (1u << r) | (entry_quads(e) << (8 + 4 * r)));
+      }
     }
     __syncthreads();
   }
@@ -1497,9 +1512,10 @@ __device__ __forceinline__ void sdd_pp_body(const GemmArgs& g, int tiles_m, int 
     int n = 0, used0 = 0, used1 = 0;
     uint32_t g1_slots = 0, rowmask = 0;
     for (int c = lo; c < hi; ++c) {
-      const uint32_t f = (uint32_t)__builtin_amdgcn_readfirstlane((int)flags[c]) & 0xfu;
+      const uint32_t fq = (uint32_t)__builtin_amdgcn_readfirstlane((int)flags[c]), f = fq & 0xfu;
       if (!f) continue;
       const int cnt = __builtin_popcount(f), w = (cnt + 1) / 2;
+      auto quads_of = [&](int r) { return (fq >> (8 + 4 * r)) & 0xfu; };
       int gsel = used0 <= used1 ? 0 : 1;
       if (4 - (gsel ? used1 : used0) < w) gsel ^= 1;
       const int wv = 4 * gsel + (gsel ? used1 : used0);
@@ -1510,8 +1526,8 @@ __device__ __forceinline__ void sdd_pp_body(const GemmArgs& g, int tiles_m, int 
       const int r_d = m ? __builtin_ctz(m) : 0;
       if (lane == 0) {
         rec[4 + n] = c;
-        rec[10 + wv] = n | (r_a << 4) | (r_b << 8) | ((cnt >= 2 ? 2 : 1) << 12);
-        if (w == 2) rec[10 + wv + 1] = n | (r_c << 4) | (r_d << 8) | ((cnt - 2) << 12);
+        rec[10 + wv] = n | (r_a << 4) | (r_b << 8) | ((cnt >= 2 ? 2 : 1) << 12) | (int)(quads_of(r_a) << 16) | (int)(quads_of(r_b) << 20);
+        if (w == 2) rec[10 + wv + 1] = n | (r_c << 4) | (r_d << 8) | ((cnt - 2) << 12) | (int)(quads_of(r_c) << 16) | (int)(quads_of(r_d) << 20);
       }
       if (gsel) { used1 += w; g1_slots |= 1u << n; } else used0 += w;
       rowmask |= f;
@@ -1537,6 +1553,7 @@ __device__ __forceinline__ void sdd_pp_body(const GemmArgs& g, int tiles_m, int 
   const uint32_t mine = (uint32_t)__builtin_amdgcn_readfirstlane(rec[10 + wave]);
   const int my_j = (int)(mine & 0xfu), n_mine = (int)((mine >> 12) & 3u);
   const int my_r[2] = {(int)((mine >> 4) & 0xfu), (int)((mine >> 8) & 0xfu)};
+  const uint32_t my_q[2] = {(mine >> 16) & 0xfu, (mine >> 20) & 0xfu};  // kept quadrants of the wave's tiles
   const int my_c = __builtin_amdgcn_readfirstlane(rec[4 + my_j]);
 
   // ---- zeros for the dropped tiles of the group's column range ----------------------------------------
@@ -1685,12 +1702,22 @@ __device__ __forceinline__ void sdd_pp_body(const GemmArgs& g, int tiles_m, int 
 #pragma unroll
     for (int k = 0; k < 2; ++k)
       if (k < n_mine) {
+        {
+          // a mask of block size 32 drops quadrants of a kept tile: their MFMAs are left out and their accumulators stay
+          // zero, which is what the epilogue then stores
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk)
+          for (int mh = 0; mh < 2; ++mh)
 #pragma unroll
-          for (int mt = 0; mt < 4; ++mt)
+            for (int nh = 0; nh < 2; ++nh)
+              if ((my_q[k] >> (2 * mh + nh)) & 1u) {
 #pragma unroll
-            for (int nt = 0; nt < 4; ++nt) acc[k][mt][nt] = T::mfma16(af[k][kk][mt], bf[kk][nt], acc[k][mt][nt]);
+                for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+                  for (int mt = 2 * mh; mt < 2 * mh + 2; ++mt)
+#pragma unroll
+                    for (int nt = 2 * nh; nt < 2 * nh + 2; ++nt) acc[k][mt][nt] = T::mfma16(af[k][kk][mt], bf[kk][nt], acc[k][mt][nt]);
+              }
+        }
       }
     __builtin_amdgcn_s_setprio(0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's loads have landed
@@ -1788,8 +1815,9 @@ int launch_dsd_s(const GemmArgs& g, int splits, hipStream_t stream) {
 
 template <typename T, bool TRANS, bool CM>
 int launch_dsd(const GemmArgs& g, bool mid, int splits, hipStream_t stream) {
-  // masks of block size 32 (quadrant keep bits in the lists) run on the ragged-edge instance, which masks fragments
-  const bool ragged = g.M % BS != 0 || g.N % BS != 0 || g.K % BS != 0 || g.quads;
+  // masks of block size 32 (quadrant keep bits in the lists): the 256 x 256 shape leaves out the MFMAs of dropped
+  // quadrants on aligned operands; elsewhere they run on the ragged-edge instance, which zeroes fragments
+  const bool ragged = g.M % BS != 0 || g.N % BS != 0 || g.K % BS != 0 || (g.quads && mid);
   if (mid)
     return ragged ? launch_dsd_s<T, TRANS, CM, true, DsdMid>(g, splits, stream)
                   : launch_dsd_s<T, TRANS, CM, false, DsdMid>(g, splits, stream);
@@ -1845,8 +1873,8 @@ int launch_sdd_shape(const GemmArgs& g, hipStream_t stream) {
 
 // the big shape when its grid (a workgroup per 4 x 4 tiles, per 4 x 6 at high drop rates) gives more than half of
 // the CUs a workgroup
-template <typename T, bool EDGE>
-int launch_sdd_group(const GemmArgs& g, hipStream_t stream) {
+template <typename T>
+int launch_sdd_group(const GemmArgs& g, bool ragged, hipStream_t stream) {
   const int64_t Mb = (g.M + BS - 1) / BS, Cb = (g.N + BS - 1) / BS;
   // workgroups the big shape would have: a group spans 4 column blocks with everything kept, 6 once few enough tiles
   // are kept for the width and not the tile count to end a group (measured: worth counting that way from p = 0.7).
@@ -1856,7 +1884,10 @@ int launch_sdd_group(const GemmArgs& g, hipStream_t stream) {
   const int64_t big = ((Mb + 3) / 4) * ((Cb + cols - 1) / cols);
   const int policy = tile_policy.load(std::memory_order_relaxed);
   const bool mid = policy == kTileMid || (policy == kTileAuto && big <= 128);
-  return mid ? launch_sdd_shape<T, EDGE, SddMid>(g, stream) : launch_sdd_shape<T, EDGE, SddBig>(g, stream);
+  // masks of block size 32 (quadrant keep bits in the lists): the big shape leaves out the MFMAs of dropped quadrants
+  // on aligned operands; the other instances zero them in the epilogue, which lives in the ragged-edge code
+  if (!mid) return (ragged ? launch_sdd_shape<T, true, SddBig> : launch_sdd_shape<T, false, SddBig>)(g, stream);
+  return (ragged || g.quads ? launch_sdd_shape<T, true, SddMid> : launch_sdd_shape<T, false, SddMid>)(g, stream);
 }
 
 int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
@@ -1870,9 +1901,8 @@ int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
   const int64_t tiles = (((g.M + BS - 1) / BS + 1) / 2) * ((Cb + 3) / 4);  // the larger of the two shapes' grids
   if (!layout_ok || !shape_ok || !align_ok || tiles > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
   if (Cb > G_MAX_CB) return SD_ERR_UNSUPPORTED;
-  const bool edge = g.N % BS != 0 || g.K % BS != 0 || g.quads;  // quadrant zeroing lives in the edge instance
-  if (dtype == SD_BF16) return edge ? launch_sdd_group<BF16, true>(g, stream) : launch_sdd_group<BF16, false>(g, stream);
-  return edge ? launch_sdd_group<F16, true>(g, stream) : launch_sdd_group<F16, false>(g, stream);
+  const bool ragged = g.N % BS != 0 || g.K % BS != 0;
+  return dtype == SD_BF16 ? launch_sdd_group<BF16>(g, ragged, stream) : launch_sdd_group<F16>(g, ragged, stream);
 }
 
 template <typename T, bool RAGGED, int FORM>
@@ -2101,7 +2131,7 @@ int launch_forward_with_lists(const GemmArgs& g, const MaskSrc& src, int64_t mb,
   const int64_t tiles = plan.mid ? dsd_tiles<DsdMid>(g.M, g.N) : dsd_tiles<DsdBig>(g.M, g.N);
   const int splits = usable_splits(g, plan, kDsd);
   if (splits < 1 || tiles * splits > forward_lists_limit()) return SD_ERR_UNSUPPORTED;
-  const bool ragged = g.M % BS != 0 || g.N % BS != 0 || g.K % BS != 0 || g.quads;
+  const bool ragged = g.M % BS != 0 || g.N % BS != 0 || g.K % BS != 0 || (g.quads && plan.mid);
   const FlatJobs f = flat_jobs(src, mb, kb, row_ptr, col_idx, col_ptr, row_idx, mask_out, mask_rows,
                                plan.mid ? DsdMid::THREADS : DsdBig::THREADS);
   if (dtype == SD_BF16) {
@@ -2173,9 +2203,9 @@ int launch_backward_pair(const GemmArgs& gx, const GemmArgs& gw, int dtype, hipS
   const int64_t w_wgs = (plan.mid ? dsd_tiles<DsdMid>(gw.M, gw.N) : dsd_tiles<DsdBig>(gw.M, gw.N)) * splits;
   if (x_wgs > pair_limit() || w_wgs > pair_limit()) return SD_ERR_UNSUPPORTED;
   if ((x_Mb + 1) / 2 * ((x_Cb + 3) / 4) + dsd_tiles<DsdMid>(gw.M, gw.N) > 0x7fffffffLL) return SD_ERR_UNSUPPORTED;
-  // either product ragged (or on a block-size-32 mask): the instances that handle edges, for both
-  const bool edge = gx.N % BS != 0 || gx.K % BS != 0 || gx.quads || gw.M % BS != 0 || gw.N % BS != 0 ||
-                    gw.K % BS != 0 || gw.quads;
+  // either product ragged (or, on the smaller shapes, on a block-size-32 mask): the instances that handle edges, for both
+  const bool edge = gx.N % BS != 0 || gx.K % BS != 0 || gw.M % BS != 0 || gw.N % BS != 0 || gw.K % BS != 0 ||
+                    ((gx.quads || gw.quads) && x_mid);
   if (dtype == SD_BF16) {
     if (x_mid) return edge ? launch_pair_t<BF16, true, SddMid, DsdMid>(gx, gw, splits, stream)
                            : launch_pair_t<BF16, false, SddMid, DsdMid>(gx, gw, splits, stream);

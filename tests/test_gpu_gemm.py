@@ -327,6 +327,60 @@ def test_4096_bf16_and_block_size_32_against_the_full_oracle(dtype, bs, tile_pol
     assert (dA.float().cpu().numpy()[~keep] == 0).all(), "dropped dX blocks must be exactly zero"
 
 
+def test_quadrant_masks_on_the_256_tile_kernels_leave_out_the_dropped_quadrants(tile_policy):
+    """Masks of block size 32 on aligned operands under the 256 x 256 workgroup shape: the kernels that alternate
+    memory and compute phases take them (not the ragged-edge instances) and leave out the MFMAs of dropped 32 x 32
+    quadrants.  Structured masks - one quadrant per 64-tile kept, a checkerboard of quadrants, whole 32-rows and
+    32-columns dropped, nearly everything dropped - against the oracle per 32 x 32 block; dropped blocks of dX
+    exactly zero."""
+    from flash_dropout.hip import GEMM
+
+    if tile_policy != "big":
+        pytest.skip("the 256 x 256 shape is what this test is about")
+    ext = GEMM()
+    M, N, K = 768, 512, 640
+    gen = torch.Generator().manual_seed(21)
+    A = make_operand(M, K, torch.float16, "cuda", gen=gen)
+    B = make_operand(N, K, torch.float16, "cuda", scale=K ** -0.5, gen=gen)
+    dC = make_operand(M, N, torch.float16, "cuda", gen=gen)
+    mb, kb = M // 32, K // 32
+    masks = {f"bernoulli_{p}": cpu_mask((mb, kb), p, gen) for p in (0.3, 0.7, 0.95)}
+    for qi in range(4):  # one quadrant of every 64-tile kept
+        m = torch.ones(mb, kb, dtype=torch.bool)
+        m[qi // 2::2, qi % 2::2] = False
+        masks[f"only_quadrant_{qi}"] = m
+    m = torch.zeros(mb, kb, dtype=torch.bool)
+    m[::2, ::2] = True
+    m[1::2, 1::2] = True
+    masks["checkerboard"] = m
+    m = torch.zeros(mb, kb, dtype=torch.bool)
+    m[1::2, :] = True
+    masks["odd_32_rows_dropped"] = m
+    m = torch.zeros(mb, kb, dtype=torch.bool)
+    m[:, ::2] = True
+    masks["even_32_columns_dropped"] = m
+    m = torch.ones(mb, kb, dtype=torch.bool)
+    m[mb - 1, kb - 1] = False
+    masks["single_last_quadrant"] = m
+    masks["none_dropped"] = torch.zeros(mb, kb, dtype=torch.bool)
+    a, b, dc = to_np(A), to_np(B), to_np(dC)
+    for name, mk in masks.items():
+        _, lists, kbs = ext.kept_lists(M, K, 32, mask=mk.cuda())
+        C = ext.gemm_dsd_lists(A, B, lists, kbs, 2.0)
+        assert ext.last_kernel_detail().startswith("dsd:big splits"), (name, ext.last_kernel_detail())
+        dA = ext.gemm_sdd_lists(dC, B.T, lists, kbs, 2.0)
+        assert ext.last_kernel_detail() == "sdd:big", (name, ext.last_kernel_detail())
+        dB = ext.gemm_dsd_lists(A.T, dC.T, lists.transposed(), kbs, 2.0).T
+        assert ext.last_kernel_detail().startswith("dsd:big:strided splits"), (name, ext.last_kernel_detail())
+        mkn = mk.numpy()
+        for got, ref, what in ((C, O.gemm_dsd(a, b, mkn, 32, 2.0, np.float32), "C"),
+                               (dA, O.gemm_sdd(dc, b.T, mkn, 32, 2.0, np.float32), "dA"),
+                               (dB, O.gemm_dsd(a.T, dc.T, mkn.T, 32, 2.0, np.float32).T, "dB")):
+            assert max_tile_rel_fro(got, ref, tile=32) <= REL_FRO_TOL, (name, what)
+        keep = O.expand_keep(mkn, 32, M, K)
+        assert (dA.cpu().numpy()[~keep] == 0).all(), name
+
+
 def _structured_masks(mb, cb, gen):
     """Masks that steer the grouped SDD kernel through its branches: groups cut by the 6-active-column
     limit, by the 16-kept-tile limit, long runs of all-dropped columns, single tiles, ragged row quads."""
