@@ -76,9 +76,10 @@ constexpr int STEP_PAD = 4;
 //           products whose 256 x 256 tiles would leave most of the 256 CUs without one; two workgroups fit
 //           a CU (72 KB of LDS, under 128 VGPRs).  More LDS fragment traffic per MFMA (1.5 KB against
 //           0.75 KB), which is why the big shape wins as soon as it can fill the chip
-template <int RH_, int NS_, int NT_, int RW_ = 2>
+template <int RH_, int NS_, int NT_, int RW_ = 2, int NST_ = 2>
 struct DsdShape {
   static constexpr int RH = RH_, NS = NS_, NT = NT_, RW = RW_;  // RW: row blocks a wave owns (2 or 1)
+  static constexpr int NST = NST_;           // stages of LDS (steps whose tiles are resident or on their way)
   static constexpr int R = RW * RH;          // row blocks per workgroup
   static constexpr int NW = RH * NS;         // waves
   static constexpr int THREADS = 64 * NW;
@@ -88,13 +89,16 @@ struct DsdShape {
   static constexpr int STAGE = B_TILE + R * TILE;
   static constexpr int BL = B_TILE / 1024 / NW;  // wave-wide 1 KB loads per wave for the W tile
   static constexpr int AL = TILE / 1024 / NW;    // ... for one X tile
-  static constexpr int SMEM_STEPS = 2 * STAGE;
+  static constexpr int SMEM_STEPS = NST * STAGE;
   static constexpr int SMEM_SCRATCH = SMEM_STEPS + 4 * (MAX_STEPS + STEP_PAD);  // uint32 per K block while merging
   static constexpr int SMEM_BYTES = SMEM_SCRATCH + 4 * MAX_STEPS + 16;
   static_assert(BL >= 1 && AL >= 1 && BL * NW * 1024 == B_TILE && AL * NW * 1024 == TILE, "loads must divide evenly");
 };
 using DsdBig = DsdShape<2, 4, 2>;  // (8 waves of 1 row block x 128 columns, DsdShape<4, 2, 4, 1>, measured 2-4 % slower)
 using DsdMid = DsdShape<2, 4, 1, 1>;
+// The same on aligned operands with four stages: a step of this shape is 16 MFMAs per wave, far shorter than a load's
+// way through L2 and memory, so three steps are kept in flight instead of one (one workgroup per CU: 136 KB of LDS)
+using DsdMidDeep = DsdShape<2, 4, 1, 1, 4>;
 // 256 rows x 128 columns, 8 waves: the shape of the implicit-GEMM convolution, whose input patch has to
 // fit in LDS next to the stages
 using DsdConv = DsdShape<2, 4, 1>;
@@ -131,6 +135,24 @@ __device__ inline void load16_to_lds(const char* base, uint32_t lane_off, uint32
   const uint32_t a = uniform(lds_dst);
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(sb), "s"(a)
                : "memory");
+}
+
+// Waits until at most n of the wave's loads are outstanding (they return in order: everything issued before the last
+// n has landed).  n is wave-uniform and only known at run time, the instruction takes an immediate.
+__device__ inline void wait_loads_all_but(int n) {
+  if (n >= 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+  else if (n == 11) asm volatile("s_waitcnt vmcnt(11)" ::: "memory");
+  else if (n == 10) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+  else if (n == 9) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+  else if (n == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  else if (n == 7) asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
+  else if (n == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+  else if (n == 5) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+  else if (n == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  else if (n == 3) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+  else if (n == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+  else if (n == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -827,6 +849,101 @@ __device__ __forceinline__ void dsd_body(const GemmArgs& g, int tiles_m, int til
         e2 = uniform(e3);
       }
     }
+  } else if constexpr (IMPLICIT == 0 && !RAGGED && S::NST > 2) {
+    // ---- the step loop of the 128 x 128 shape on aligned operands: three steps in flight ---------------------------
+    // A step here is 12 fragment reads and 16 MFMAs per wave; with one step in flight every step waits out a whole
+    // load latency (measured: 2200 clocks a step, whatever the drop rate).  So the tiles of steps s + 1 .. s + 3 are on
+    // their way while step s computes: four stages, one barrier per step (it publishes step s and frees the stage of
+    // step s - 1, into which the loads of step s + 3 go right behind it).  A wave waits for its own loads of step s
+    // only: loads return in order, so it allows as many outstanding as it issued for the two steps after - a number
+    // that depends on which X tiles those steps keep, hence the choice among waits below.
+    static_assert(RW == 1 && S::NST == 4, "one row block per wave, four stages");
+    constexpr int NST = S::NST;
+    const int rh_u = (int)uniform((uint32_t)rh);
+    const bool w_any = TRANS || wave_u * BL * 8 < nvalid;  // this wave's rows of the W tile are columns inside C
+    // (reduction-strided W tile: lanes whose columns lie past N fetch column 0 of their row instead - readable, and
+    // those columns are never stored)
+    uint32_t b_ld[BL];
+#pragma unroll
+    for (int jj = 0; jj < BL; ++jj) {
+      b_ld[jj] = b_lane[jj];
+      if constexpr (TRANS) {
+        constexpr int CPR = BN / 8;
+        const int row = (wave * BL + jj) * (64 / CPR) + lane / CPR;
+        if (!b_valid[jj]) b_ld[jj] = (uint32_t)(row * g.b.sc) * 2u;
+      }
+    }
+    auto loads_of = [&](uint32_t e) {  // load instructions this wave issues for a step
+      const uint32_t fl = step_flags(e);
+      int n = w_any ? BL : 0;
+#pragma unroll
+      for (int r = 0; r < R; ++r) n += row_quads(fl, r) ? AL : 0;
+      return n;
+    };
+    auto issue = [&](uint32_t e, int stage) {
+      const int kb = step_block(e);
+      const uint32_t fl = step_flags(e);
+      const uint32_t st_a = smem_a + (uint32_t)(stage * STAGE);
+      const char* bp = b_tile0 + kb * b_red_stride;
+      const char* ap = a_tile0 + kb * red_stride;
+      if (w_any) {
+#pragma unroll
+        for (int jj = 0; jj < BL; ++jj) load16_to_lds(bp, b_ld[jj], st_a + (uint32_t)((wave_u * BL + jj) * 1024));
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if (row_quads(fl, r)) {
+#pragma unroll
+          for (int i = 0; i < AL; ++i)
+            load16_to_lds(ap + r * a_rstride, a_lane[i], st_a + (uint32_t)(A_OFF + r * TILE + (wave_u * AL + i) * 1024));
+        }
+    };
+    if (nsteps > 0) {
+      uint32_t e0 = uniform(step_e[0]), e1 = uniform(step_e[1]), e2 = uniform(step_e[2]), e3 = uniform(step_e[3]);
+      issue(e0, 0);
+      int c1 = 0, c2 = 0;
+      if (nsteps > 1) {
+        issue(e1, 1);
+        c1 = (int)uniform((uint32_t)loads_of(e1));
+      }
+      if (nsteps > 2) {
+        issue(e2, 2);
+        c2 = (int)uniform((uint32_t)loads_of(e2));
+      }
+      u32x4 bf[NT16][2];
+      u32x4 af[2][4];
+      for (int step = 0; step < nsteps; ++step) {
+        const uint32_t e4 = step_e[step + 4];  // a VGPR until the end of the step
+        wait_loads_all_but(c1 + c2);
+        __syncthreads();
+        int c3 = 0;
+        if (step + 3 < nsteps) {
+          issue(e3, (step + 3) % NST);
+          c3 = (int)uniform((uint32_t)loads_of(e3));
+        }
+        if (row_quads(step_flags(e0), rh_u)) {
+          const char* st = smem + (step % NST) * STAGE;
+          const char* at = st + A_OFF + rh * TILE;
+          read_b(st, 0, bf);
+          read_a(at, 0, af[0]);
+          read_b(st, 1, bf);
+          read_a(at, 1, af[1]);
+#pragma unroll
+          for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+              for (int nt = 0; nt < NT16; ++nt) acc[0][mt][nt] = T::mfma16(af[kk][mt], bf[nt][kk], acc[0][mt][nt]);
+        }
+        e0 = e1;
+        e1 = e2;
+        e2 = e3;
+        e3 = uniform(e4);
+        c1 = c2;
+        c2 = c3;
+      }
+      __syncthreads();  // the epilogue reuses the stages
+    }
   } else if constexpr (IMPLICIT == 0) {
     // The products that read their operands from memory run the units of all steps as one chain: the barrier
     // that publishes the next stage stands in front of the MFMAs of a step's LAST unit, not behind them.  By
@@ -1056,8 +1173,9 @@ __global__ __launch_bounds__(S::THREADS) void forward_lists_kernel(GemmArgs g, i
 //           two 80 KB stages, all of the LDS
 // SddMid   2 row blocks x at most 4 active column blocks and 8 kept tiles, one slot per wave: twice as many
 //           workgroups with half the loads per step each, for outputs that give the big shape too few
-template <int R_, int GW_, int SLOTS_>
+template <int R_, int GW_, int SLOTS_, int NST_ = 2>
 struct SddShape {
+  static constexpr int NST = NST_;       // stages of LDS (steps whose tiles are resident or on their way)
   static constexpr int R = R_;           // row blocks per workgroup
   static constexpr int GW = GW_;         // column blocks with kept tiles per group
   static constexpr int SLOTS = SLOTS_;   // whole tiles a wave can own
@@ -1065,7 +1183,7 @@ struct SddShape {
   static constexpr int BOFF = R * TILE;  // dY tiles first, then W tiles
   static constexpr int STAGE = (R + GW) * TILE;
   // two stages; at least the eight 64 x 68 fp32 staging tiles of the epilogue
-  static constexpr int SMEM = 2 * STAGE > 8 * BS * (BS + 4) * 4 ? 2 * STAGE : 8 * BS * (BS + 4) * 4;
+  static constexpr int SMEM = NST * STAGE > 8 * BS * (BS + 4) * 4 ? NST * STAGE : 8 * BS * (BS + 4) * 4;
   static constexpr int MINCOLS = GW < MAXT / R ? GW : MAXT / R;  // column blocks a group is sure to cover
   // Groups never straddle a multiple of WINDOW column blocks, and a workgroup is launched for (window, group in
   // the window): whatever the masks of two row quads, their workgroups of one window need the same W tiles
@@ -1075,6 +1193,11 @@ struct SddShape {
 };
 using SddBig = SddShape<4, 6, 2>;
 using SddMid = SddShape<2, 4, 1>;
+// On aligned operands, outputs too small for the big shape run with more steps in flight (a step of these shapes is
+// far shorter than a load's way through L2 and memory): the shape above with three stages, and for outputs that give
+// even that one too few workgroups, 2 row blocks x 2 column blocks (4 tiles, on waves 0-3; all 8 waves load) with four
+using SddMidDeep = SddShape<2, 4, 1, 3>;
+using SddSmall = SddShape<2, 2, 1, 4>;
 constexpr int G_MAX_CB = 8192;             // per-column flags share the first stage (of either shape) before the loads start
 
 // EDGE = the output width or the reduction length is not a multiple of 64 (both multiples of 8): the
@@ -1357,6 +1480,30 @@ __device__ __forceinline__ void sdd_body(const GemmArgs& g, int tiles_m, int gma
       for (int nt = 0; nt < 4; ++nt) acc[k][mt][nt] = T::mfma16(af[u & 1][mt], bf[u & 1][nt], acc[k][mt][nt]);
   };
 
+  if constexpr (!EDGE && G::NST > 2) {
+    // ---- more than one step in flight: the tiles of steps s + 1 .. s + NST - 2 are on their way while step s
+    // computes; one barrier per step publishes step s and frees the stage of step s - 1, which the loads of step
+    // s + NST - 1 go into right behind it.  Every step costs this wave the same number of loads, so "my loads of
+    // step s have landed" is "at most (steps still in flight) x (loads per step) outstanding".
+    static_assert(SLOTS == 1, "one tile per wave");
+    constexpr int NST = G::NST;
+    const int n_ld = __builtin_popcount(rowmask) + ncols;
+    for (int s0 = 0; s0 < NST - 1 && s0 < nsteps; ++s0) issue_loads(s0, s0);
+    for (int step = 0; step < nsteps; ++step) {
+      const int left = nsteps - 1 - step;
+      wait_loads_all_but((left < NST - 2 ? left : NST - 2) * n_ld);
+      __syncthreads();
+      if (step + NST - 1 < nsteps) issue_loads(step + NST - 1, (step + NST - 1) % NST);
+      if (act[0]) {
+        const int stage = step % NST;
+        read_unit(stage, 0);
+        read_unit(stage, 1);
+        mfma_unit(std::integral_constant<int, 0>{}, 0, false);
+        mfma_unit(std::integral_constant<int, 0>{}, 1, false);
+      }
+    }
+    __syncthreads();  // the epilogue reuses the stages
+  } else {
   issue_loads(0, 0);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
@@ -1394,6 +1541,7 @@ __device__ __forceinline__ void sdd_body(const GemmArgs& g, int tiles_m, int gma
     } else {
       boundary(step, stage, false);
     }
+  }
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------------
@@ -1813,14 +1961,26 @@ int launch_dsd_s(const GemmArgs& g, int splits, hipStream_t stream) {
   return SD_OK;
 }
 
+template <typename S>
+int64_t dsd_tiles(int64_t M, int64_t N) {
+  return ((M + BS * S::R - 1) / (BS * S::R)) * ((N + S::BN - 1) / S::BN);
+}
+bool mid_tiles_fit_one_round(const GemmArgs& g, int splits) { return dsd_tiles<DsdMid>(g.M, g.N) * splits <= 256; }
+
 template <typename T, bool TRANS, bool CM>
 int launch_dsd(const GemmArgs& g, bool mid, int splits, hipStream_t stream) {
   // masks of block size 32 (quadrant keep bits in the lists): the 256 x 256 shape leaves out the MFMAs of dropped
   // quadrants on aligned operands; elsewhere they run on the ragged-edge instance, which zeroes fragments
   const bool ragged = g.M % BS != 0 || g.N % BS != 0 || g.K % BS != 0 || (g.quads && mid);
-  if (mid)
-    return ragged ? launch_dsd_s<T, TRANS, CM, true, DsdMid>(g, splits, stream)
-                  : launch_dsd_s<T, TRANS, CM, false, DsdMid>(g, splits, stream);
+  if (mid) {
+    if (ragged) return launch_dsd_s<T, TRANS, CM, true, DsdMid>(g, splits, stream);
+    // one round of workgroups or less: a CU has one workgroup whatever its LDS, and the four-stage loop is the faster
+    // one (4096 x 1024 x 4096: 67 -> 52 us; 2048^3: 39 -> 30 us).  With more, two workgroups of the two-stage shape
+    // share a CU and keep its LDS busier than one of the four-stage shape can (8192^3 on this shape: 1.09 against
+    // 1.34 ms).
+    return mid_tiles_fit_one_round(g, splits) ? launch_dsd_s<T, TRANS, CM, false, DsdMidDeep>(g, splits, stream)
+                                              : launch_dsd_s<T, TRANS, CM, false, DsdMid>(g, splits, stream);
+  }
   return ragged ? launch_dsd_s<T, TRANS, CM, true, DsdBig>(g, splits, stream)
                 : launch_dsd_s<T, TRANS, CM, false, DsdBig>(g, splits, stream);
 }
@@ -1831,10 +1991,6 @@ struct DsdPlan {
   bool mid;
   int splits;
 };
-template <typename S>
-int64_t dsd_tiles(int64_t M, int64_t N) {
-  return ((M + BS * S::R - 1) / (BS * S::R)) * ((N + S::BN - 1) / S::BN);
-}
 // One round of workgroups (one per CU) when the output alone gives fewer than half of that and the
 // reduction is long enough to pay for the extra pass: at least 8 reduction blocks per split.
 int splits_for(int64_t tiles, int64_t M, int64_t N, int64_t K) {
@@ -1867,7 +2023,7 @@ int launch_sdd_shape(const GemmArgs& g, hipStream_t stream) {
   const int tiles_m = (Mb + G::R - 1) / G::R, gmax = (Cb + G::MINCOLS - 1) / G::MINCOLS;
   hipLaunchKernelGGL((sdd_group_kernel<T, EDGE, G>), dim3((unsigned)(tiles_m * gmax)), dim3(THREADS), G::SMEM, stream,
                      g, tiles_m, gmax, Mb, Cb);
-  note_kernel("sdd:%s%s", G::R == 4 ? "big" : "mid", EDGE ? ":ragged" : "");
+  note_kernel("sdd:%s%s", G::R == 4 ? "big" : (G::GW == 2 ? "small" : "mid"), EDGE ? ":ragged" : "");
   return check_launch("sdd_group_kernel");
 }
 
@@ -1887,7 +2043,13 @@ int launch_sdd_group(const GemmArgs& g, bool ragged, hipStream_t stream) {
   // masks of block size 32 (quadrant keep bits in the lists): the big shape leaves out the MFMAs of dropped quadrants
   // on aligned operands; the other instances zero them in the epilogue, which lives in the ragged-edge code
   if (!mid) return (ragged ? launch_sdd_shape<T, true, SddBig> : launch_sdd_shape<T, false, SddBig>)(g, stream);
-  return (ragged || g.quads ? launch_sdd_shape<T, true, SddMid> : launch_sdd_shape<T, false, SddMid>)(g, stream);
+  if (ragged || g.quads) return launch_sdd_shape<T, true, SddMid>(g, stream);
+  // aligned: the loops with several steps in flight (the two-stage shape holds a CU alone as well: its epilogue's
+  // staging tiles take 136 KB).  Half a round of workgroups or less on the 2 x 4 shape: the 2 x 2 shape, twice as many
+  // (4096 x 4096 -> 1024 columns: 93 us on 128 workgroups of the two-stage shape).
+  const int64_t mid_wgs = ((Mb + 1) / 2) * ((Cb + 3) / 4);
+  if (policy == kTileAuto && mid_wgs <= 128) return launch_sdd_shape<T, false, SddSmall>(g, stream);
+  return launch_sdd_shape<T, false, SddMidDeep>(g, stream);
 }
 
 int try_sdd(const GemmArgs& g, int dtype, hipStream_t stream) {
@@ -2135,11 +2297,13 @@ int launch_forward_with_lists(const GemmArgs& g, const MaskSrc& src, int64_t mb,
   const FlatJobs f = flat_jobs(src, mb, kb, row_ptr, col_idx, col_ptr, row_idx, mask_out, mask_rows,
                                plan.mid ? DsdMid::THREADS : DsdBig::THREADS);
   if (dtype == SD_BF16) {
+    if (plan.mid && !ragged && mid_tiles_fit_one_round(g, splits)) return launch_forward_lists_t<BF16, false, DsdMidDeep>(g, splits, f, stream);
     if (plan.mid) return ragged ? launch_forward_lists_t<BF16, true, DsdMid>(g, splits, f, stream)
                                 : launch_forward_lists_t<BF16, false, DsdMid>(g, splits, f, stream);
     return ragged ? launch_forward_lists_t<BF16, true, DsdBig>(g, splits, f, stream)
                   : launch_forward_lists_t<BF16, false, DsdBig>(g, splits, f, stream);
   }
+  if (plan.mid && !ragged && mid_tiles_fit_one_round(g, splits)) return launch_forward_lists_t<F16, false, DsdMidDeep>(g, splits, f, stream);
   if (plan.mid) return ragged ? launch_forward_lists_t<F16, true, DsdMid>(g, splits, f, stream)
                               : launch_forward_lists_t<F16, false, DsdMid>(g, splits, f, stream);
   return ragged ? launch_forward_lists_t<F16, true, DsdBig>(g, splits, f, stream)
@@ -2207,13 +2371,14 @@ int launch_backward_pair(const GemmArgs& gx, const GemmArgs& gw, int dtype, hipS
   const bool edge = gx.N % BS != 0 || gx.K % BS != 0 || gw.M % BS != 0 || gw.N % BS != 0 || gw.K % BS != 0 ||
                     ((gx.quads || gw.quads) && x_mid);
   if (dtype == SD_BF16) {
+    // (the smaller SDD shape holds a CU alone anyway: the loops with more stages cost nothing)
     if (x_mid) return edge ? launch_pair_t<BF16, true, SddMid, DsdMid>(gx, gw, splits, stream)
-                           : launch_pair_t<BF16, false, SddMid, DsdMid>(gx, gw, splits, stream);
+                           : launch_pair_t<BF16, false, SddMidDeep, DsdMidDeep>(gx, gw, splits, stream);
     return edge ? launch_pair_t<BF16, true, SddBig, DsdBig>(gx, gw, splits, stream)
                 : launch_pair_t<BF16, false, SddBig, DsdBig>(gx, gw, splits, stream);
   }
   if (x_mid) return edge ? launch_pair_t<F16, true, SddMid, DsdMid>(gx, gw, splits, stream)
-                         : launch_pair_t<F16, false, SddMid, DsdMid>(gx, gw, splits, stream);
+                         : launch_pair_t<F16, false, SddMidDeep, DsdMidDeep>(gx, gw, splits, stream);
   return edge ? launch_pair_t<F16, true, SddBig, DsdBig>(gx, gw, splits, stream)
               : launch_pair_t<F16, false, SddBig, DsdBig>(gx, gw, splits, stream);
 }

@@ -381,6 +381,40 @@ def test_quadrant_masks_on_the_256_tile_kernels_leave_out_the_dropped_quadrants(
         assert (dA.cpu().numpy()[~keep] == 0).all(), name
 
 
+@pytest.mark.parametrize("M,N,K", [(128, 64, 64), (256, 192, 128), (384, 320, 192), (1024, 448, 1024),
+                                   (2048, 2048, 2048), (4096, 1024, 1024)])
+@pytest.mark.parametrize("p", [0.0, 0.5, 0.9])
+def test_loops_with_several_steps_in_flight(M, N, K, p, tile_policy):
+    """Aligned products too small for the 256 x 256 shapes run loops that keep two or three steps in flight: fewer
+    steps than stages (K = 64, 128, 192), column tiles that overhang N (N = 64 mod 128), steps in which a wave keeps
+    nothing (p = 0.9), and the routes themselves."""
+    from flash_dropout.hip import GEMM
+
+    ext = GEMM()
+    gen = torch.Generator().manual_seed(M + N + K)
+    A = make_operand(M, K, torch.float16, "cuda", gen=gen)
+    B = make_operand(N, K, torch.float16, "cuda", scale=K ** -0.5, gen=gen)
+    dC = make_operand(M, N, torch.float16, "cuda", gen=gen)
+    mk = cpu_mask((M // 64, K // 64), p, gen)
+    lists = ext.build_lists(mk.cuda())
+    s = 1 / (1 - p)
+    C = ext.gemm_dsd_lists(A, B, lists, 64, s)
+    routes = [ext.last_kernel_detail()]
+    dA = ext.gemm_sdd_lists(dC, B.T, lists, 64, s, keep_hint=1 - p)
+    routes.append(ext.last_kernel_detail())
+    dB = ext.gemm_dsd_lists(A.T, dC.T, lists.transposed(), 64, s).T
+    routes.append(ext.last_kernel_detail())
+    if tile_policy == "auto" and (M, N, K) == (2048, 2048, 2048):
+        assert routes == ["dsd:mid splits=1", "sdd:small", "dsd:mid:strided splits=1"], routes
+    if tile_policy == "mid":
+        assert routes[1] == "sdd:mid", routes
+    rC, rdA, rdB = _oracle_products(A, B, dC, mk, 64, p)
+    for got, ref, what in ((C, rC, "C"), (dA, rdA, "dA"), (dB, rdB, "dB")):
+        assert max_tile_rel_fro(got, ref) <= REL_FRO_TOL, (what, routes)
+    keep = O.expand_keep(mk.numpy(), 64, M, K)
+    assert (dA.cpu().numpy()[~keep] == 0).all()
+
+
 def _structured_masks(mb, cb, gen):
     """Masks that steer the grouped SDD kernel through its branches: groups cut by the 6-active-column
     limit, by the 16-kept-tile limit, long runs of all-dropped columns, single tiles, ragged row quads."""
