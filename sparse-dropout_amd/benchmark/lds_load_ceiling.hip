@@ -14,6 +14,11 @@
 //   staged    the shared pattern with the tiles going through registers instead: global_load_dwordx4 for the next
 //             step at the top of a step, ds_write_b128 into the other stage behind the step's fragment reads
 // It prints bytes into LDS per second over the chip; the GEMM kernels' own rate is to be read against these.
+// A second kernel leaves out the barrier: every wave streams on its own with 8 to 16 loads in flight ("free"), which is
+// what the path delivers when nothing synchronises - from L1 (a wave re-reads its own 8 KB), from L2 with the tile rows
+// of the shared pattern (8 rows x 128 B per load, 16 KB apart), with the same panels packed tile by tile (each load
+// 1 KB contiguous, a 32 KB tile one run: what a pre-packed operand layout would give), with rows of 256 B (4 per
+// load), and into registers instead of LDS.
 //
 //   hipcc --offload-arch=gfx950 -O3 -w -Xclang -target-feature -Xclang -packed-fp32-ops \
 //         -o /tmp/lds_load_ceiling sparse-dropout_amd/benchmark/lds_load_ceiling.hip && /tmp/lds_load_ceiling
@@ -121,6 +126,49 @@ __global__ __launch_bounds__(THREADS) void stream(const char* src, size_t region
   if (threadIdx.x == 0) sink[wg] = *reinterpret_cast<int*>(smem + (steps & 1) * 4);
 }
 
+// pattern 0: the wave's own 8 KB again and again (L1); 1: tile rows of the shared panels; 2: the panels packed tile by
+// tile; 3: rows of 256 B.  Eight loads per iteration, then a wait that leaves the last eight in flight.
+template <bool TO_LDS>
+__global__ __launch_bounds__(THREADS) void free_run(const char* src, int iters, int pattern, int positions, int* sink) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const uint32_t smem_a = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)(lds_void*)smem);
+  const int lane = threadIdx.x % 64, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+  const int wg = blockIdx.x;
+  const size_t ROW = 16384;
+  uint32_t lane_off = lane * 16;
+  if (pattern == 1) lane_off = (uint32_t)((lane / 8) * ROW + (lane % 8) * 16);
+  if (pattern == 3) lane_off = (uint32_t)((lane / 16) * ROW + (lane % 16) * 16);
+  const int xcd = wg % 8, slot = wg / 8;
+  const int pr = slot % 8, pc = slot / 8 % 4;
+  u32x4 x = {0, 0, 0, 0};
+  u32x4 regs[8];
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int l = wave * 8 + i;  // the 64 loads of a 64 KB step
+      const int panel = l < 32 ? pr : 8 + pc;
+      const size_t pbase = ((size_t)xcd * 12 + panel) * 256 * ROW;
+      const char* p;
+      if (pattern == 0) p = src + ((size_t)wg * 8 + wave) * 8192 + i * 1024;
+      else if (pattern == 1) p = src + pbase + (size_t)(l % 32) * 8 * ROW + (size_t)(it % positions) * 128;
+      else if (pattern == 2) p = src + (((size_t)xcd * 12 + panel) * positions + (it % positions)) * 32768 + (size_t)(l % 32) * 1024;
+      else p = src + pbase + (size_t)(l % 32) * 8 * ROW + (size_t)((it % positions) / 2) * 256 + (size_t)(it & 1) * 4 * ROW;
+      if (TO_LDS) {
+        load16_to_lds(p, lane_off, smem_a + (it & 1) * STAGE + l * 1024);
+      } else {
+        if (it > 0) x ^= regs[i];
+        regs[i] = *reinterpret_cast<const u32x4*>(p + lane_off);
+      }
+    }
+    if (TO_LDS) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (!TO_LDS)
+    for (int i = 0; i < 8; ++i) x ^= regs[i];
+  if ((x.x ^ x.y ^ x.z ^ x.w) == 0x12345678u) sink[wg] = 1;
+  if (threadIdx.x == 0) sink[wg] = *reinterpret_cast<int*>(smem + 4);
+}
+
 int main() {
   const int wgs = 256, steps = 2048;
   const size_t bytes = (size_t)8 << 30;
@@ -143,6 +191,9 @@ int main() {
       {"staged, 384 MB of panels", 3, 0, 0, 128},
       {"staged, 384 MB + 24 KB LDS reads / wave", 3, 0, 24, 128},
       {"staged, p=.5 step: 48 KB + 14 KB reads / wave", 3, 0, 14, 128, 6},
+      // the fragment volume of four waves of 128 x 128 (32 KB each) spread over this kernel's eight
+      {"shared, 384 MB + 16 KB LDS reads / wave", 2, 0, 16, 128},
+      {"p=.5 step: 48 KB loads + 10 KB reads / wave", 2, 0, 10, 128, 6},
   };
   for (auto& c : cases) {
     for (int rep = 0; rep < 2; ++rep) {
@@ -160,6 +211,34 @@ int main() {
       if (hipGetLastError() != hipSuccess) { printf("launch failed\n"); return 1; }
       const double tb = (double)wgs * steps * (c.nl * THREADS / 64 * 1024) / (ms * 1e-3) / 1e12;
       printf("%-40s %8.3f ms  %6.2f TB/s into LDS  (%.1f B/clk/CU at 2.4 GHz)\n", c.name, ms, tb, tb * 1e12 / 256 / 2.4e9);
+    }
+  }
+  hipFuncSetAttribute((const void*)free_run<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * STAGE);
+  hipFuncSetAttribute((const void*)free_run<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * STAGE);
+  struct { const char* name; int pattern; bool to_lds; } free_cases[] = {
+      {"free: own 8 KB per wave (L1)", 0, true},
+      {"free: own 8 KB per wave (L1) -> registers", 0, false},
+      {"free: shared panels, 8 rows x 128 B per load", 1, true},
+      {"free: shared panels, 8 x 128 B -> registers", 1, false},
+      {"free: shared panels packed, 1 KB per load", 2, true},
+      {"free: shared panels, 4 rows x 256 B per load", 3, true},
+  };
+  for (auto& c : free_cases) {
+    for (int rep = 0; rep < 2; ++rep) {
+      hipEvent_t e0, e1; hipEventCreate(&e0); hipEventCreate(&e1);
+      auto launch = [&](int n) {
+        if (c.to_lds) free_run<true><<<wgs, THREADS, 2 * STAGE>>>(d, n, c.pattern, 64, sink);
+        else free_run<false><<<wgs, THREADS, 2 * STAGE>>>(d, n, c.pattern, 64, sink);
+      };
+      launch(64);
+      hipDeviceSynchronize();
+      hipEventRecord(e0);
+      launch(steps);
+      hipEventRecord(e1); hipEventSynchronize(e1);
+      float ms; hipEventElapsedTime(&ms, e0, e1);
+      if (hipGetLastError() != hipSuccess) { printf("launch failed\n"); return 1; }
+      const double tb = (double)wgs * steps * STAGE / (ms * 1e-3) / 1e12;
+      printf("%-48s %8.3f ms  %6.2f TB/s          (%.1f B/clk/CU at 2.4 GHz)\n", c.name, ms, tb, tb * 1e12 / 256 / 2.4e9);
     }
   }
   return 0;
