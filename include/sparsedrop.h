@@ -74,7 +74,8 @@ const char* sd_last_error(void);
 const char* sd_last_kernel(void);
 
 /* What that call ran on, in more detail: kernel family, workgroup shape and reduction splits, e.g. "dsd:big splits=1",
- * "dsd:mid:strided:ragged splits=4", "sdd:mid", "generic", "conv_fwd:implicit:rows-per-step", "conv_dw:implicit
+ * "dsd:mid:strided:ragged splits=4", "sdd:mid", "sdd:small" (shapes: 256 x 256 / 128 x 128 output tiles for DSD, 4 / 2 / 2
+ * row blocks by column groups of up to 6 / 4 / 2 blocks for SDD), "generic", "conv_fwd:implicit:rows-per-step", "conv_dw:implicit
  * splits=85", "conv_dx:fused".  The conv entry points that return SD_ERR_UNSUPPORTED leave it unchanged (the caller's
  * explicit route then shows its own GEMM here).  Diagnostic text, not a stable format. */
 const char* sd_last_kernel_detail(void);

@@ -46,8 +46,11 @@ def main() -> None:
     ap.add_argument("--shape", type=int, nargs=3, metavar=("M", "N", "K"), help="one shape instead of the built-in list")
     ap.add_argument("--p", type=float, nargs="+", default=[0.0, 0.5])
     ap.add_argument("--dtype", choices=["float16", "bfloat16"], default="float16")
+    ap.add_argument("--tile-policy", choices=sorted(GEMM.TILE_POLICIES), default="auto",
+                    help="force a workgroup shape (to check what the library picks by itself)")
     args = ap.parse_args()
     ext = GEMM()
+    ext.set_tile_policy(args.tile_policy)
     dtype = getattr(torch, args.dtype)
     flush = torch.empty(FLUSH_BYTES, dtype=torch.int8, device="cuda")
     gen = torch.Generator(device="cuda").manual_seed(0)
