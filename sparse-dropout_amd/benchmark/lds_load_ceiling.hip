@@ -19,6 +19,8 @@
 // of the shared pattern (8 rows x 128 B per load, 16 KB apart), with the same panels packed tile by tile (each load
 // 1 KB contiguous, a 32 KB tile one run: what a pre-packed operand layout would give), with rows of 256 B (4 per
 // load), and into registers instead of LDS.
+// A third kernel ("deep") is the first with smaller steps and more stages: NL x 8 KB per step, NST - 1 steps in flight,
+// with and without fragment reads - whether keeping more steps in flight lifts the rate of a step that also reads.
 //
 //   hipcc --offload-arch=gfx950 -O3 -w -Xclang -target-feature -Xclang -packed-fp32-ops \
 //         -o /tmp/lds_load_ceiling sparse-dropout_amd/benchmark/lds_load_ceiling.hip && /tmp/lds_load_ceiling
@@ -169,6 +171,69 @@ __global__ __launch_bounds__(THREADS) void free_run(const char* src, int iters, 
   if (threadIdx.x == 0) sink[wg] = *reinterpret_cast<int*>(smem + 4);
 }
 
+// NL loads of 1 KB per wave and step (shared-panel pattern), NST stages: the loads of step s + NST - 1 go out right behind
+// the barrier that publishes step s; `reads` as in the first kernel
+template <int NL, int NST>
+__global__ __launch_bounds__(THREADS) void deep(const char* src, int steps, int reads, int positions, int* sink) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int DSTAGE = NL * 8 * 1024;
+  const uint32_t smem_a = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)(lds_void*)smem);
+  const int lane = threadIdx.x % 64, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+  const int wg = blockIdx.x;
+  const size_t ROW = 16384;
+  const uint32_t lane_off = (uint32_t)((lane / 8) * ROW + (lane % 8) * 16);
+  const int xcd = wg % 8, slot = wg / 8;
+  const int pr = slot % 8, pc = slot / 8 % 4;
+  auto issue = [&](int step, int stage) {
+    const uint32_t st = smem_a + stage * DSTAGE + wave * (NL * 1024);
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const int l = wave * 8 + i;
+      const int panel = l < 32 ? pr : 8 + pc;
+      const char* p = src + ((size_t)xcd * 12 + panel) * 256 * ROW + (size_t)(l % 32) * 8 * ROW + (size_t)(step % positions) * 128;
+      load16_to_lds(p, lane_off, st + i * 1024);
+    }
+  };
+  u32x4 x = {0, 0, 0, 0};
+  for (int s = 0; s < NST - 1 && s < steps; ++s) issue(s, s);
+  for (int step = 0; step < steps; ++step) {
+    const int left = steps - 1 - step;
+    const int ahead = left < NST - 2 ? left : NST - 2;  // younger steps that may still be in flight
+    static_assert(NL == 4 || NL == 6, "the waits below");
+    if (ahead == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else if (ahead == 1) { if (NL == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); else asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); }
+    else if (ahead == 2) { if (NL == 6) asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); else asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); }
+    else asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    __syncthreads();
+    if (step + NST - 1 < steps) issue(step + NST - 1, (step + NST - 1) % NST);
+    const char* st = smem + (step % NST) * DSTAGE + lane * 16;
+    for (int i = 0; i < reads; ++i) x ^= *reinterpret_cast<const u32x4*>(st + ((wave * 5 + i) % (NL * 8)) * 1024);
+  }
+  if ((x.x ^ x.y ^ x.z ^ x.w) == 0x12345678u) sink[wg] = 1;
+  if (threadIdx.x == 0) sink[wg] = *reinterpret_cast<int*>(smem + 4);
+}
+template <int NL, int NST>
+int run_deep(const char* d, int reads, int* sink) {
+  constexpr int SMEM = NL * 8 * 1024 * NST;
+  static_assert(SMEM <= 160 * 1024, "LDS of a CU");
+  hipFuncSetAttribute((const void*)deep<NL, NST>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+  const int wgs = 256, steps = 2048;
+  for (int rep = 0; rep < 2; ++rep) {
+    hipEvent_t e0, e1; hipEventCreate(&e0); hipEventCreate(&e1);
+    deep<NL, NST><<<wgs, THREADS, SMEM>>>(d, 64, reads, 128, sink);
+    hipDeviceSynchronize();
+    hipEventRecord(e0);
+    deep<NL, NST><<<wgs, THREADS, SMEM>>>(d, steps, reads, 128, sink);
+    hipEventRecord(e1); hipEventSynchronize(e1);
+    float ms; hipEventElapsedTime(&ms, e0, e1);
+    if (hipGetLastError() != hipSuccess) { printf("launch failed\n"); return 1; }
+    const double tb = (double)wgs * steps * (NL * 8 * 1024) / (ms * 1e-3) / 1e12;
+    printf("deep: %d KB step, %d in flight, %2d KB reads / wave  %8.3f ms  %6.2f TB/s into LDS  (%.0f clocks per step at 2.4 GHz)\n",
+           NL * 8, NST - 1, reads, ms, tb, ms * 1e-3 / steps * 2.4e9);
+  }
+  return 0;
+}
+
 int main() {
   const int wgs = 256, steps = 2048;
   const size_t bytes = (size_t)8 << 30;
@@ -213,6 +278,10 @@ int main() {
       printf("%-40s %8.3f ms  %6.2f TB/s into LDS  (%.1f B/clk/CU at 2.4 GHz)\n", c.name, ms, tb, tb * 1e12 / 256 / 2.4e9);
     }
   }
+  if (run_deep<6, 2>(d, 0, sink) || run_deep<6, 2>(d, 14, sink) || run_deep<6, 3>(d, 0, sink) || run_deep<6, 3>(d, 14, sink) ||
+      run_deep<4, 2>(d, 0, sink) || run_deep<4, 2>(d, 12, sink) || run_deep<4, 3>(d, 0, sink) || run_deep<4, 3>(d, 12, sink) ||
+      run_deep<4, 5>(d, 0, sink) || run_deep<4, 5>(d, 12, sink))
+    return 1;
   hipFuncSetAttribute((const void*)free_run<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * STAGE);
   hipFuncSetAttribute((const void*)free_run<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * STAGE);
   struct { const char* name; int pattern; bool to_lds; } free_cases[] = {

@@ -2296,14 +2296,18 @@ int launch_forward_with_lists(const GemmArgs& g, const MaskSrc& src, int64_t mb,
   const bool ragged = g.M % BS != 0 || g.N % BS != 0 || g.K % BS != 0 || (g.quads && plan.mid);
   const FlatJobs f = flat_jobs(src, mb, kb, row_ptr, col_idx, col_ptr, row_idx, mask_out, mask_rows,
                                plan.mid ? DsdMid::THREADS : DsdBig::THREADS);
+  // the four-stage shape holds a CU alone, the list builder's blocks included: only when they all find a CU of their own
+  // in one round (else the blocks that build the lists wait for a product workgroup to finish, and the two-stage shape,
+  // which shares a CU with them, is as fast)
+  const bool deep = plan.mid && !ragged && tiles * splits + f.blocks() <= 256;
   if (dtype == SD_BF16) {
-    if (plan.mid && !ragged && mid_tiles_fit_one_round(g, splits)) return launch_forward_lists_t<BF16, false, DsdMidDeep>(g, splits, f, stream);
+    if (deep) return launch_forward_lists_t<BF16, false, DsdMidDeep>(g, splits, f, stream);
     if (plan.mid) return ragged ? launch_forward_lists_t<BF16, true, DsdMid>(g, splits, f, stream)
                                 : launch_forward_lists_t<BF16, false, DsdMid>(g, splits, f, stream);
     return ragged ? launch_forward_lists_t<BF16, true, DsdBig>(g, splits, f, stream)
                   : launch_forward_lists_t<BF16, false, DsdBig>(g, splits, f, stream);
   }
-  if (plan.mid && !ragged && mid_tiles_fit_one_round(g, splits)) return launch_forward_lists_t<F16, false, DsdMidDeep>(g, splits, f, stream);
+  if (deep) return launch_forward_lists_t<F16, false, DsdMidDeep>(g, splits, f, stream);
   if (plan.mid) return ragged ? launch_forward_lists_t<F16, true, DsdMid>(g, splits, f, stream)
                               : launch_forward_lists_t<F16, false, DsdMid>(g, splits, f, stream);
   return ragged ? launch_forward_lists_t<F16, true, DsdBig>(g, splits, f, stream)
