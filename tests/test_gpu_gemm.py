@@ -327,7 +327,8 @@ def test_4096_bf16_and_block_size_32_against_the_full_oracle(dtype, bs, tile_pol
     assert (dA.float().cpu().numpy()[~keep] == 0).all(), "dropped dX blocks must be exactly zero"
 
 
-def test_quadrant_masks_on_the_256_tile_kernels_leave_out_the_dropped_quadrants(tile_policy):
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_quadrant_masks_on_the_256_tile_kernels_leave_out_the_dropped_quadrants(dtype, tile_policy):
     """Masks of block size 32 on aligned operands under the 256 x 256 workgroup shape: the kernels that alternate
     memory and compute phases take them (not the ragged-edge instances) and leave out the MFMAs of dropped 32 x 32
     quadrants.  Structured masks - one quadrant per 64-tile kept, a checkerboard of quadrants, whole 32-rows and
@@ -340,9 +341,9 @@ def test_quadrant_masks_on_the_256_tile_kernels_leave_out_the_dropped_quadrants(
     ext = GEMM()
     M, N, K = 768, 512, 640
     gen = torch.Generator().manual_seed(21)
-    A = make_operand(M, K, torch.float16, "cuda", gen=gen)
-    B = make_operand(N, K, torch.float16, "cuda", scale=K ** -0.5, gen=gen)
-    dC = make_operand(M, N, torch.float16, "cuda", gen=gen)
+    A = make_operand(M, K, dtype, "cuda", gen=gen)
+    B = make_operand(N, K, dtype, "cuda", scale=K ** -0.5, gen=gen)
+    dC = make_operand(M, N, dtype, "cuda", gen=gen)
     mb, kb = M // 32, K // 32
     masks = {f"bernoulli_{p}": cpu_mask((mb, kb), p, gen) for p in (0.3, 0.7, 0.95)}
     for qi in range(4):  # one quadrant of every 64-tile kept
@@ -378,13 +379,14 @@ def test_quadrant_masks_on_the_256_tile_kernels_leave_out_the_dropped_quadrants(
                                (dB, O.gemm_dsd(a.T, dc.T, mkn.T, 32, 2.0, np.float32).T, "dB")):
             assert max_tile_rel_fro(got, ref, tile=32) <= REL_FRO_TOL, (name, what)
         keep = O.expand_keep(mkn, 32, M, K)
-        assert (dA.cpu().numpy()[~keep] == 0).all(), name
+        assert (dA.float().cpu().numpy()[~keep] == 0).all(), name
 
 
 @pytest.mark.parametrize("M,N,K", [(128, 64, 64), (256, 192, 128), (384, 320, 192), (1024, 448, 1024),
                                    (2048, 2048, 2048), (4096, 1024, 1024)])
 @pytest.mark.parametrize("p", [0.0, 0.5, 0.9])
-def test_loops_with_several_steps_in_flight(M, N, K, p, tile_policy):
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_loops_with_several_steps_in_flight(M, N, K, p, dtype, tile_policy):
     """Aligned products too small for the 256 x 256 shapes run loops that keep two or three steps in flight: fewer
     steps than stages (K = 64, 128, 192), column tiles that overhang N (N = 64 mod 128), steps in which a wave keeps
     nothing (p = 0.9), and the routes themselves."""
@@ -392,9 +394,9 @@ def test_loops_with_several_steps_in_flight(M, N, K, p, tile_policy):
 
     ext = GEMM()
     gen = torch.Generator().manual_seed(M + N + K)
-    A = make_operand(M, K, torch.float16, "cuda", gen=gen)
-    B = make_operand(N, K, torch.float16, "cuda", scale=K ** -0.5, gen=gen)
-    dC = make_operand(M, N, torch.float16, "cuda", gen=gen)
+    A = make_operand(M, K, dtype, "cuda", gen=gen)
+    B = make_operand(N, K, dtype, "cuda", scale=K ** -0.5, gen=gen)
+    dC = make_operand(M, N, dtype, "cuda", gen=gen)
     mk = cpu_mask((M // 64, K // 64), p, gen)
     lists = ext.build_lists(mk.cuda())
     s = 1 / (1 - p)
@@ -412,7 +414,7 @@ def test_loops_with_several_steps_in_flight(M, N, K, p, tile_policy):
     for got, ref, what in ((C, rC, "C"), (dA, rdA, "dA"), (dB, rdB, "dB")):
         assert max_tile_rel_fro(got, ref) <= REL_FRO_TOL, (what, routes)
     keep = O.expand_keep(mk.numpy(), 64, M, K)
-    assert (dA.cpu().numpy()[~keep] == 0).all()
+    assert (dA.float().cpu().numpy()[~keep] == 0).all()
 
 
 def _structured_masks(mb, cb, gen):
