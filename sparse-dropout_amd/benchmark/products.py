@@ -64,7 +64,7 @@ def main() -> None:
         print(f"{name:13s} M={M} N={N} K={K}   torch.matmul: forward {t[0]:.0f}  dX {t[1]:.0f}  dW {t[2]:.0f}  sum {sum(t):.0f} us",
               flush=True)
         for p in args.p:
-            mask = torch.rand(M // 64, K // 64, device="cuda", generator=gen) < p
+            mask = torch.rand(-(-M // 64), -(-K // 64), device="cuda", generator=gen) < p
             lists = ext.build_lists(mask)
             lt = lists.transposed()
             s = 1 / (1 - p)
